@@ -1,0 +1,27 @@
+from .llama import ConfigError, LlamaConfig, RopeScaling, llama_model_spec
+from .registry import (
+    ARCHITECTURES,
+    ArchSpec,
+    architecture_name,
+    get_architecture,
+    load_config,
+    register_architecture,
+)
+from .spec import LayerRun, LayerSpec, ModelSpec, PartSpec
+
+__all__ = [
+    "ARCHITECTURES",
+    "ArchSpec",
+    "ConfigError",
+    "LayerRun",
+    "LayerSpec",
+    "LlamaConfig",
+    "ModelSpec",
+    "PartSpec",
+    "RopeScaling",
+    "architecture_name",
+    "get_architecture",
+    "llama_model_spec",
+    "load_config",
+    "register_architecture",
+]

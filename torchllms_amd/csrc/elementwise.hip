@@ -1,0 +1,291 @@
+// Row-wise kernels: embedding gather, RMS norm fused with the residual sum, rotary position
+// encoding fused with the write of keys and values into cache pages, SwiGLU gate, bias.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+
+// ----------------------------------------------------------------------------- errors
+static thread_local char g_last_error[512] = "";
+
+int tl_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int tl_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return TL_OK;
+}
+
+TL_EXPORT const char* tl_last_error() { return g_last_error; }
+TL_EXPORT int tl_abi_version() { return 1; }
+
+// ----------------------------------------------------------------------------- embedding
+// out[t, :] = table[tokens[t], :].  One block per token; 16-byte copies when the row allows.
+template <typename T>
+__global__ void embed_kernel(const int32_t* __restrict__ tokens, const T* __restrict__ table,
+                             T* __restrict__ out, int hidden) {
+  const int t = blockIdx.x;
+  const T* src = table + (size_t)tokens[t] * hidden;
+  T* dst = out + (size_t)t * hidden;
+  constexpr int VEC = 16 / sizeof(T);
+  if (hidden % VEC == 0) {
+    const uint4* s4 = reinterpret_cast<const uint4*>(src);
+    uint4* d4 = reinterpret_cast<uint4*>(dst);
+    for (int i = threadIdx.x; i < hidden / VEC; i += blockDim.x) d4[i] = s4[i];
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+  }
+}
+
+TL_EXPORT int tl_embed(const int32_t* tokens, const void* table, void* out, int n_tokens, int hidden,
+                       int dtype, hipStream_t stream) {
+  TL_REQUIRE(n_tokens >= 0 && hidden > 0, "embed: bad sizes n_tokens=%d hidden=%d", n_tokens, hidden);
+  if (n_tokens == 0) return TL_OK;
+  if (dtype == TL_F32)
+    embed_kernel<float><<<n_tokens, 256, 0, stream>>>(tokens, (const float*)table, (float*)out, hidden);
+  else if (dtype == TL_BF16)
+    embed_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(tokens, (const bf16_t*)table, (bf16_t*)out, hidden);
+  else
+    return tl_fail(TL_ERR_ARG, "embed: unknown dtype %d", dtype);
+  return tl_check_launch("embed");
+}
+
+// ----------------------------------------------------------------------------- RMS norm
+// For output row r (source row s = rows ? rows[r] : r):
+//   h   = T(float(x[s]) + float(delta[s]))            (delta optional; sum in 32-bit, one rounding)
+//   n   = T(float(h) * 1/sqrt(mean(float(h)^2) + eps))
+//   y   = T(float(n) * float(weight))
+// h is written to h_out when given.  Statistics are 32-bit with a fixed reduction order.
+constexpr int kNormThreads = 256;
+
+template <typename T, typename WT>
+__global__ void __launch_bounds__(kNormThreads)
+rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ delta, const int32_t* __restrict__ rows,
+               const WT* __restrict__ weight, T* __restrict__ h_out, T* __restrict__ y, int hidden,
+               float eps) {
+  __shared__ float scratch[kNormThreads / kWave];
+  extern __shared__ float row_cache[];  // hidden floats: the summed row, kept between the passes
+  const int r = blockIdx.x;
+  const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+  const T* xr = x + s * hidden;
+  const T* dr = delta ? delta + s * hidden : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += kNormThreads) {
+    float v = to_f32(xr[i]);
+    if (dr) v = to_f32(from_f32<T>(v + to_f32(dr[i])));
+    row_cache[i] = v;
+    ss += v * v;
+  }
+  ss = block_sum<kNormThreads / kWave>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+  T* yr = y + (size_t)r * hidden;
+  T* hr = h_out ? h_out + (size_t)r * hidden : nullptr;
+  for (int i = threadIdx.x; i < hidden; i += kNormThreads) {
+    const float v = row_cache[i];
+    if (hr) hr[i] = from_f32<T>(v);
+    const float n = to_f32(from_f32<T>(v * inv));
+    yr[i] = from_f32<T>(n * to_f32(weight[i]));
+  }
+}
+
+TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, const void* weight,
+                         int weight_dtype, void* h_out, void* y, int n_rows, int hidden, float eps,
+                         int dtype, hipStream_t stream) {
+  TL_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm: bad sizes n_rows=%d hidden=%d", n_rows, hidden);
+  TL_REQUIRE(!(rows && h_out), "rmsnorm: h_out cannot be combined with a row gather");
+  TL_REQUIRE((size_t)hidden * sizeof(float) <= 160 * 1024 - 1024, "rmsnorm: hidden=%d does not fit LDS", hidden);
+  if (n_rows == 0) return TL_OK;
+  const size_t lds = (size_t)hidden * sizeof(float);
+#define TL_NORM_LAUNCH(T, WT)                                                                       \
+  do {                                                                                              \
+    if (lds > 48 * 1024) {                                                                          \
+      hipError_t e = hipFuncSetAttribute((const void*)rmsnorm_kernel<T, WT>,                        \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);     \
+      if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "rmsnorm: %s", hipGetErrorString(e));         \
+    }                                                                                               \
+    rmsnorm_kernel<T, WT><<<n_rows, kNormThreads, lds, stream>>>(                                   \
+        (const T*)x, (const T*)delta, rows, (const WT*)weight, (T*)h_out, (T*)y, hidden, eps);      \
+  } while (0)
+  if (dtype == TL_F32 && weight_dtype == TL_F32)
+    TL_NORM_LAUNCH(float, float);
+  else if (dtype == TL_BF16 && weight_dtype == TL_BF16)
+    TL_NORM_LAUNCH(bf16_t, bf16_t);
+  else if (dtype == TL_BF16 && weight_dtype == TL_F32)
+    TL_NORM_LAUNCH(bf16_t, float);
+  else
+    return tl_fail(TL_ERR_ARG, "rmsnorm: unsupported dtypes x=%d weight=%d", dtype, weight_dtype);
+#undef TL_NORM_LAUNCH
+  return tl_check_launch("rmsnorm");
+}
+
+// ----------------------------------------------------------------------------- rotary + KV write
+// qkv: [n_tokens, (Hq + 2 Hkv) * dh], each row = q heads | k heads | v heads.
+// For token t at position p: angle_i = float(p) * inv_freq[i], i < rotary_dim/2 (32-bit), and
+//   pairing 0 (interleaved): (x[2i], x[2i+1])     pairing 1 (half split): (x[i], x[i + rotary_dim/2])
+//   x0' = x0 cos - x1 sin ;  x1' = x1 cos + x0 sin        (32-bit, then one rounding)
+// q is rotated in place.  k is rotated and, with v, stored at slot_mapping[t] = page * P + offset
+// of pages laid out [page][Hkv][P][dh]; slot < 0 skips the store.  Without pages k is rotated in place.
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_kv_heads, int head_dim,
+                                     const int32_t* __restrict__ positions,
+                                     const float* __restrict__ inv_freq, int rotary_dim, int pairing,
+                                     T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                     const int32_t* __restrict__ slot_mapping, int page_size) {
+  const int t = blockIdx.x;
+  const int half = head_dim / 2;
+  const int rot_half = rotary_dim / 2;
+  const float pos = (float)positions[t];
+  const int row = (n_q_heads + 2 * n_kv_heads) * head_dim;
+  T* base = qkv + (size_t)t * row;
+  const int slot = slot_mapping ? slot_mapping[t] : -1;
+  const int page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+  const bool store = k_pages != nullptr && slot >= 0;
+
+  // queries and keys: one thread per (head, pair)
+  const int n_rot_heads = n_q_heads + n_kv_heads;
+  for (int w = threadIdx.x; w < n_rot_heads * half; w += blockDim.x) {
+    const int h = w / half;
+    const int i = w % half;
+    T* head = base + (size_t)h * head_dim;
+    int i0, i1;
+    float x0, x1;
+    if (i < rot_half) {
+      if (pairing == 0) {
+        i0 = 2 * i;
+        i1 = 2 * i + 1;
+      } else {
+        i0 = i;
+        i1 = i + rot_half;
+      }
+      const float a0 = to_f32(head[i0]);
+      const float a1 = to_f32(head[i1]);
+      const float ang = pos * inv_freq[i];
+      const float c = cosf(ang);
+      const float s = sinf(ang);
+      x0 = a0 * c - a1 * s;
+      x1 = a1 * c + a0 * s;
+    } else {
+      // channels beyond rotary_dim pass unchanged
+      i0 = rotary_dim + 2 * (i - rot_half);
+      i1 = i0 + 1;
+      x0 = to_f32(head[i0]);
+      x1 = to_f32(head[i1]);
+    }
+    const T r0 = from_f32<T>(x0);
+    const T r1 = from_f32<T>(x1);
+    if (h < n_q_heads || k_pages == nullptr) {
+      head[i0] = r0;
+      head[i1] = r1;
+    }
+    if (h >= n_q_heads && store) {
+      const int kh = h - n_q_heads;
+      T* dst = k_pages + (((size_t)page * n_kv_heads + kh) * page_size + off) * head_dim;
+      dst[i0] = r0;
+      dst[i1] = r1;
+    }
+  }
+  // values
+  if (store && v_pages != nullptr) {
+    const T* vsrc = base + (size_t)(n_q_heads + n_kv_heads) * head_dim;
+    for (int w = threadIdx.x; w < n_kv_heads * head_dim; w += blockDim.x) {
+      const int kh = w / head_dim;
+      const int d = w % head_dim;
+      v_pages[(((size_t)page * n_kv_heads + kh) * page_size + off) * head_dim + d] = vsrc[w];
+    }
+  }
+}
+
+TL_EXPORT int tl_rope_kv_write(void* qkv, int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
+                               const int32_t* positions, const float* inv_freq, int rotary_dim,
+                               int pairing, void* k_pages, void* v_pages, const int32_t* slot_mapping,
+                               int page_size, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n_tokens >= 0 && n_q_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "rope: bad sizes");
+  TL_REQUIRE(head_dim % 2 == 0, "rope: head_dim=%d must be even", head_dim);
+  TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
+             "rope: rotary_dim=%d must be even and at most head_dim=%d", rotary_dim, head_dim);
+  TL_REQUIRE(pairing == 0 || pairing == 1, "rope: pairing must be 0 (interleaved) or 1 (half split)");
+  TL_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope: inv_freq missing");
+  TL_REQUIRE(k_pages == nullptr || (slot_mapping != nullptr && page_size > 0),
+             "rope: pages given without slot_mapping/page_size");
+  if (n_tokens == 0) return TL_OK;
+  const int threads = 256;
+  if (dtype == TL_F32)
+    rope_kv_write_kernel<float><<<n_tokens, threads, 0, stream>>>(
+        (float*)qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, rotary_dim, pairing,
+        (float*)k_pages, (float*)v_pages, slot_mapping, page_size);
+  else if (dtype == TL_BF16)
+    rope_kv_write_kernel<bf16_t><<<n_tokens, threads, 0, stream>>>(
+        (bf16_t*)qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, rotary_dim, pairing,
+        (bf16_t*)k_pages, (bf16_t*)v_pages, slot_mapping, page_size);
+  else
+    return tl_fail(TL_ERR_ARG, "rope: unknown dtype %d", dtype);
+  return tl_check_launch("rope_kv_write");
+}
+
+// ----------------------------------------------------------------------------- SwiGLU gate
+// gate_up: [n, 2F] = gate | up.  out[n, F] = T(float(T(silu(gate))) * float(up)), silu(z) = z / (1 + e^-z).
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int n, int inter) {
+  const size_t total = (size_t)n * inter;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = idx / inter;
+    const int c = (int)(idx % inter);
+    const float g = to_f32(gate_up[r * 2 * inter + c]);
+    const float u = to_f32(gate_up[r * 2 * inter + inter + c]);
+    const float act = to_f32(from_f32<T>(g / (1.0f + expf(-g))));
+    out[idx] = from_f32<T>(act * u);
+  }
+}
+
+TL_EXPORT int tl_silu_mul(const void* gate_up, void* out, int n, int inter, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && inter > 0, "silu_mul: bad sizes n=%d inter=%d", n, inter);
+  if (n == 0) return TL_OK;
+  const size_t total = (size_t)n * inter;
+  const int threads = 256;
+  const int blocks = (int)((total + threads - 1) / threads < 65536 ? (total + threads - 1) / threads : 65536);
+  if (dtype == TL_F32)
+    silu_mul_kernel<float><<<blocks, threads, 0, stream>>>((const float*)gate_up, (float*)out, n, inter);
+  else if (dtype == TL_BF16)
+    silu_mul_kernel<bf16_t><<<blocks, threads, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, n, inter);
+  else
+    return tl_fail(TL_ERR_ARG, "silu_mul: unknown dtype %d", dtype);
+  return tl_check_launch("silu_mul");
+}
+
+// ----------------------------------------------------------------------------- bias
+// x[n, width] += bias[width]  (sum in 32-bit, one rounding)
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const T* __restrict__ bias, int n, int width, int row_stride) {
+  const size_t total = (size_t)n * width;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = idx / width;
+    const int c = (int)(idx % width);
+    T* p = x + r * row_stride + c;
+    *p = from_f32<T>(to_f32(*p) + to_f32(bias[c]));
+  }
+}
+
+TL_EXPORT int tl_add_bias(void* x, const void* bias, int n, int width, int row_stride, int dtype,
+                          hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && width > 0 && row_stride >= width, "add_bias: bad sizes");
+  if (n == 0) return TL_OK;
+  const size_t total = (size_t)n * width;
+  const int threads = 256;
+  const int blocks = (int)((total + threads - 1) / threads < 65536 ? (total + threads - 1) / threads : 65536);
+  if (dtype == TL_F32)
+    add_bias_kernel<float><<<blocks, threads, 0, stream>>>((float*)x, (const float*)bias, n, width, row_stride);
+  else if (dtype == TL_BF16)
+    add_bias_kernel<bf16_t><<<blocks, threads, 0, stream>>>((bf16_t*)x, (const bf16_t*)bias, n, width, row_stride);
+  else
+    return tl_fail(TL_ERR_ARG, "add_bias: unknown dtype %d", dtype);
+  return tl_check_launch("add_bias");
+}

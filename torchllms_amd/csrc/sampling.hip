@@ -1,0 +1,189 @@
+// Next-token choice from 32-bit logits, one block per row.
+//   temperature == 0 : argmax(logits), the lowest index among equal maxima.
+//   temperature  > 0 : x = logits / max(temperature, 1e-5); optionally everything below the k-th
+//                      largest x is dropped (ties kept); the token is argmax_i exp(x_i - max x) / q_i
+//                      with q_i ~ Exponential(1): an exponential race, which draws from softmax(x).
+// q_i comes from a counter-based generator (Philox 4x32-10) keyed by the row's seed; the counter is
+// (i / 4, step), so a row's draw depends on its own seed and step only, never on the batch.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 1024;
+constexpr int kWaves = kThreads / kWave;
+
+__device__ __forceinline__ void philox_round(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
+  const uint64_t p0 = (uint64_t)0xD2511F53u * c[0];
+  const uint64_t p1 = (uint64_t)0xCD9E8D57u * c[2];
+  const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0;
+  const uint32_t n1 = (uint32_t)p1;
+  const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+  const uint32_t n3 = (uint32_t)p0;
+  c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+}
+
+// Four 32-bit words for (block index `blk`, step) under `seed`.
+__device__ __forceinline__ void philox4(uint64_t seed, uint32_t blk, uint64_t step, uint32_t (&out)[4]) {
+  uint32_t k0 = (uint32_t)seed, k1 = (uint32_t)(seed >> 32);
+  uint32_t c[4] = {blk, (uint32_t)step, (uint32_t)(step >> 32), 0u};
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    philox_round(c, k0, k1);
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c[0]; out[1] = c[1]; out[2] = c[2]; out[3] = c[3];
+}
+
+// Uniform in (0, 1): 24 random bits, centred in their cell, so neither 0 nor 1 can occur.
+__device__ __forceinline__ float uniform_open(uint32_t bits) {
+  return ((float)(bits >> 8) + 0.5f) * (1.0f / 16777216.0f);
+}
+
+__device__ __forceinline__ float uniform_at(uint64_t seed, uint64_t step, int i) {
+  uint32_t r[4];
+  philox4(seed, (uint32_t)i >> 2, step, r);
+  return uniform_open(r[i & 3]);
+}
+
+// Order-preserving map float -> uint32 (larger float, larger key).
+__device__ __forceinline__ uint32_t float_key(float v) {
+  const uint32_t u = __float_as_uint(v);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+struct Best {
+  float val;
+  int idx;
+};
+__device__ __forceinline__ Best better(Best a, Best b) {
+  if (b.val > a.val || (b.val == a.val && b.idx < a.idx)) return b;
+  return a;
+}
+__device__ __forceinline__ Best block_best(Best v, Best* scratch) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    Best o;
+    o.val = __shfl_xor(v.val, off, kWave);
+    o.idx = __shfl_xor(v.idx, off, kWave);
+    v = better(v, o);
+  }
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  Best total = scratch[0];
+  for (int w = 1; w < kWaves; ++w) total = better(total, scratch[w]);
+  return total;
+}
+
+__global__ void __launch_bounds__(kThreads)
+sample_kernel(const float* __restrict__ logits, int row_stride, int vocab,
+              const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
+              const uint64_t* __restrict__ seeds, const uint64_t* __restrict__ steps,
+              int32_t* __restrict__ out) {
+  __shared__ Best best_scratch[kWaves];
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t sel_prefix, sel_remaining;
+  const int row = blockIdx.x;
+  const float* x = logits + (size_t)row * row_stride;
+  const float temp = temperature[row];
+  const int tid = threadIdx.x;
+  constexpr int kNone = 0x7fffffff;
+
+  if (temp == 0.f) {
+    Best b = {-INFINITY, kNone};
+    for (int i = tid; i < vocab; i += kThreads) b = better(b, Best{x[i], i});
+    b = block_best(b, best_scratch);
+    if (tid == 0) out[row] = b.idx;
+    return;
+  }
+  const float tdiv = fmaxf(temp, 1e-5f);
+
+  // k-th largest scaled logit by radix selection over the order-preserving keys, 8 bits a pass
+  float pivot = -INFINITY;
+  int k = top_k ? top_k[row] : 0;
+  if (k > 0 && k < vocab) {
+    if (tid == 0) {
+      sel_prefix = 0;
+      sel_remaining = (uint32_t)k;
+    }
+    for (int shift = 24; shift >= 0; shift -= 8) {
+      for (int i = tid; i < 256; i += kThreads) hist[i] = 0;
+      __syncthreads();
+      const uint32_t prefix = sel_prefix;
+      const uint32_t mask = shift == 24 ? 0u : (0xFFFFFFFFu << (shift + 8));
+      for (int i = tid; i < vocab; i += kThreads) {
+        const uint32_t key = float_key(x[i] / tdiv);
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        uint32_t remaining = sel_remaining;
+        int bin = 255;
+        for (; bin > 0; --bin) {
+          if (hist[bin] >= remaining) break;
+          remaining -= hist[bin];
+        }
+        sel_prefix = prefix | ((uint32_t)bin << shift);
+        sel_remaining = remaining;
+      }
+      __syncthreads();
+    }
+    const uint32_t key = sel_prefix;
+    const uint32_t u = (key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key;
+    pivot = __uint_as_float(u);
+  }
+
+  Best mx = {-INFINITY, kNone};
+  for (int i = tid; i < vocab; i += kThreads) mx = better(mx, Best{x[i] / tdiv, i});
+  mx = block_best(mx, best_scratch);
+  const float m = mx.val;
+
+  const uint64_t seed = seeds[row];
+  const uint64_t step = steps[row];
+  Best b = {-INFINITY, kNone};
+  // each thread handles whole groups of four indices, so one generator call serves four draws
+  for (int i4 = tid * 4; i4 < vocab; i4 += kThreads * 4) {
+    uint32_t r[4];
+    philox4(seed, (uint32_t)i4 >> 2, step, r);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i4 + u;
+      if (i >= vocab) break;
+      const float xi = x[i] / tdiv;
+      if (xi < pivot) continue;
+      const float q = -logf(uniform_open(r[u]));
+      b = better(b, Best{expf(xi - m) / q, i});
+    }
+  }
+  b = block_best(b, best_scratch);
+  if (tid == 0) out[row] = b.idx;
+}
+
+__global__ void philox_uniform_kernel(uint64_t seed, uint64_t step, float* out, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = uniform_at(seed, step, i);
+}
+
+}  // namespace
+
+// logits: [n_rows, vocab] 32-bit with row stride `row_stride`.  temperature[n_rows]; top_k[n_rows] or
+// null (entries <= 0: no cut); seeds[n_rows], steps[n_rows]: generator key and counter of each row.
+TL_EXPORT int tl_sample(const float* logits, int row_stride, int n_rows, int vocab, const float* temperature,
+                        const int32_t* top_k, const uint64_t* seeds, const uint64_t* steps, int32_t* out,
+                        hipStream_t stream) {
+  TL_REQUIRE(n_rows >= 0 && vocab > 0 && row_stride >= vocab, "sample: bad sizes");
+  TL_REQUIRE(temperature && seeds && steps && out, "sample: null argument");
+  if (n_rows == 0) return TL_OK;
+  sample_kernel<<<n_rows, kThreads, 0, stream>>>(logits, row_stride, vocab, temperature, top_k, seeds, steps, out);
+  return tl_check_launch("sample");
+}
+
+// The uniforms the sampler uses for (seed, step), indices 0..n-1; for tests of the sampler.
+TL_EXPORT int tl_philox_uniform(uint64_t seed, uint64_t step, float* out, int n, hipStream_t stream) {
+  TL_REQUIRE(n >= 0, "philox_uniform: bad size");
+  if (n == 0) return TL_OK;
+  philox_uniform_kernel<<<(n + 255) / 256, 256, 0, stream>>>(seed, step, out, n);
+  return tl_check_launch("philox_uniform");
+}

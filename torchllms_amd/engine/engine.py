@@ -1,0 +1,174 @@
+"""The engine: a model, its cache and the one step function that everything else drives.
+
+``Engine.step`` takes a batch of (request, its next tokens) — portions of prompts beside single
+decoded tokens, cut anywhere —, runs exactly those tokens as one batch against the cache, and
+returns the logits at the wanted places.  Generation, the scheduler and trace replay all go
+through it.  The reference's counterpart is ``Transformer.forward`` with a ``PagedKVPool``
+(reference: torchllms/models/networks.py:909-1049), which must be given *all* live rollouts in
+claim order (networks.py:985-990); here any subset of the live requests may run, in any order.
+"""
+
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheManager, OutOfPages, group_layers
+from ..config.registry import ArchSpec, get_architecture, load_config
+from ..parts.model import Model
+from ..weights.loader import load_weights
+from ..weights.random_init import random_tensors
+from .context import StepContext, upload
+from .layout import StepEntry, StepLayout, build_step_layout
+
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "fp32": torch.float32, "bf16": torch.bfloat16}
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"dtype must be float32 or bfloat16, got {dtype}")
+        return dtype
+    try:
+        return DTYPES[str(dtype)]
+    except KeyError:
+        raise ValueError(f"dtype must be one of {sorted(DTYPES)}, got {dtype!r}") from None
+
+
+def require_gpu(device) -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError(
+            "this engine runs on an AMD GPU only (there is no CPU path); "
+            f"asked for device {device}, torch.cuda.is_available()={torch.cuda.is_available()}"
+        )
+    return device
+
+
+class Engine:
+    def __init__(
+        self,
+        arch: ArchSpec,
+        config,
+        tensors: Dict[str, torch.Tensor],
+        dtype: torch.dtype,
+        page_size: int = 16,
+        num_pages: Optional[int] = None,
+        kv_memory_gb: Optional[float] = None,
+        max_seqs: int = 8,
+        max_model_len: Optional[int] = None,
+        device="cuda:0",
+    ):
+        """``tensors``: the model's tensors under the parts' own names, on ``device``.
+        Pool size: ``num_pages`` pages per group, else what ``kv_memory_gb`` holds, else room for
+        ``max_seqs`` requests of ``max_model_len`` tokens (reference: networks.py:872-884)."""
+        self.device = require_gpu(device)
+        self.arch = arch
+        self.config = config
+        self.dtype = dtype
+        self.spec = arch.model_spec(config)
+        self.model = Model(self.spec)
+        self.model.bind(tensors)
+        self.vocab_size = self.spec.vocab_size
+        self.max_model_len = int(max_model_len or self.spec.max_positions)
+        self.page_size = page_size
+        groups, states = group_layers(self.model.cache_needs())
+        if num_pages is None:
+            per_page = CacheManager.bytes_per_page(groups, page_size, dtype)
+            if kv_memory_gb is not None and per_page > 0:
+                num_pages = max(int(kv_memory_gb * (1 << 30)) // per_page, 1)
+            else:
+                num_pages = max_seqs * (-(-self.max_model_len // page_size))
+        self.cache = CacheManager(groups, states, page_size, num_pages, max_seqs, dtype=dtype, device=self.device)
+        self.steps_run = 0
+        self.tokens_run = 0
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_folder(cls, folder, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+        """A model folder holds ``config.json`` and safetensors; the architecture named in
+        config.json picks the model."""
+        device = require_gpu(device)
+        dtype = parse_dtype(dtype)
+        arch, config = load_config(folder)
+        spec = arch.model_spec(config)
+        expected = Model(spec).param_specs()
+        ignore = ["head.weight"] if "head.weight" not in expected else []
+        tensors = load_weights(folder, arch.weight_rules(config), expected, dtype, device=device, ignore_when_present=ignore)
+        return cls(arch, config, tensors, dtype, device=device, **kw)
+
+    @classmethod
+    def from_random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", norm_jitter: float = 0.0,
+                    draw_on_device: bool = False, **kw) -> "Engine":
+        """Random weights without a folder: same values as ``write_model_folder`` with this seed
+        when drawn on the CPU; ``draw_on_device`` draws on the GPU instead (large models)."""
+        device = require_gpu(device)
+        dtype = parse_dtype(dtype)
+        arch = get_architecture(config.architectures[0])
+        expected = Model(arch.model_spec(config)).param_specs()
+        if draw_on_device:
+            tensors = random_tensors(expected, seed, dtype, norm_jitter, device=device)
+        else:
+            tensors = {}
+            for name, t in random_tensors(expected, seed, torch.float32, norm_jitter).items():
+                tensors[name] = t.to(dtype).to(device)
+        return cls(arch, config, tensors, dtype, device=device, **kw)
+
+    # ------------------------------------------------------------------ requests
+    def admit(self, rid: Hashable) -> int:
+        return self.cache.admit(rid)
+
+    def free(self, rid: Hashable) -> None:
+        self.cache.free(rid)
+
+    def num_tokens(self, rid: Hashable) -> int:
+        return self.cache.num_tokens(rid)
+
+    # ------------------------------------------------------------------ the step
+    def plan(self, entries: Sequence[StepEntry]) -> StepLayout:
+        """Reserve pages for the step's tokens (all or nothing) and lay the step out."""
+        seen = set()
+        for e in entries:
+            if e.rid in seen:
+                raise ValueError(f"request {e.rid!r} appears twice in one step")
+            seen.add(e.rid)
+            if not self.cache.has(e.rid):
+                raise KeyError(f"request {e.rid!r} is not live (admit it first)")
+            n = len(e.tokens)
+            if n == 0:
+                raise ValueError(f"request {e.rid!r}: an entry needs at least one token")
+            for tok in e.tokens:
+                if not 0 <= int(tok) < self.vocab_size:
+                    raise ValueError(f"request {e.rid!r}: token id {tok} outside the vocabulary of {self.vocab_size}")
+            if self.cache.num_tokens(e.rid) + n > self.max_model_len:
+                raise ValueError(
+                    f"request {e.rid!r}: {self.cache.num_tokens(e.rid)} + {n} tokens exceed max_model_len={self.max_model_len}"
+                )
+        # all-or-nothing over the whole batch: count the pages the step takes from every pool
+        for gi, pool in enumerate(self.cache.pools):
+            need = sum(self.cache.new_pages_needed(e.rid, len(e.tokens)) for e in entries)
+            if need > pool.free_count:
+                raise OutOfPages(
+                    f"step needs {need} new pages in group {self.cache.groups[gi].name}, {pool.free_count} are free"
+                )
+        starts = [self.cache.extend(e.rid, len(e.tokens)) for e in entries]
+        slots = [self.cache.slot(e.rid) for e in entries]
+        tables = [[self.cache.block_table(e.rid, g) for e in entries] for g in range(len(self.cache.groups))]
+        return build_step_layout(entries, starts, slots, tables, self.page_size)
+
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run one batch; returns float32 logits [number of wanted places, vocab], in the order
+        of the entries and of their ``want`` lists."""
+        if not entries:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        layout = self.plan(entries)
+        ctx = upload(layout, self.device)
+        logits = self.model.forward(ctx, self.cache)
+        for e in entries:
+            self.cache.advance(e.rid, len(e.tokens))
+        self.steps_run += 1
+        self.tokens_run += layout.n_tokens
+        return logits

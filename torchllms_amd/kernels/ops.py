@@ -1,0 +1,258 @@
+"""The kernels as functions of ``torch`` tensors.
+
+Every function checks on the host that shapes, dtypes and devices are what the kernel and its grid
+assume, launches on torch's current HIP stream and raises ``KernelError`` when a launcher refuses.
+Tensors must live on the GPU: there is no CPU path.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .lib import KernelError, check, core
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {dtype}; kernels take float32 and bfloat16") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _gpu(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel arguments must be GPU tensors (there is no CPU path)")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _i32(t: Optional[torch.Tensor], what: str) -> None:
+    if t is not None and (t.dtype != torch.int32 or not t.is_contiguous()):
+        raise KernelError(f"{what} must be a contiguous int32 tensor")
+
+
+def embed(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """``table[tokens]``; tokens int32 [n], table [vocab, hidden].  The caller has checked ids < vocab."""
+    _gpu(tokens, table)
+    _i32(tokens, "tokens")
+    if table.dim() != 2 or not table.is_contiguous():
+        raise KernelError("embedding table must be a contiguous matrix")
+    n, hidden = tokens.numel(), table.shape[1]
+    out = torch.empty((n, hidden), dtype=table.dtype, device=table.device)
+    check(core().tl_embed(tokens.data_ptr(), table.data_ptr(), out.data_ptr(), n, hidden, dtype_code(table.dtype), _stream()))
+    return out
+
+
+def rmsnorm(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    eps: float,
+    delta: Optional[torch.Tensor] = None,
+    rows: Optional[torch.Tensor] = None,
+    return_sum: bool = False,
+):
+    """RMS norm of ``x (+ delta)`` row by row, optionally of the rows ``rows`` only.
+
+    Returns ``y`` or, with ``return_sum``, ``(x + delta, y)``.
+    """
+    _gpu(x, weight, delta, rows)
+    _i32(rows, "rows")
+    if x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("rmsnorm input must be a contiguous [rows, hidden] tensor")
+    hidden = x.shape[1]
+    if weight.shape != (hidden,) or not weight.is_contiguous():
+        raise KernelError(f"rmsnorm weight must have shape ({hidden},), got {tuple(weight.shape)}")
+    if delta is not None and (delta.shape != x.shape or delta.dtype != x.dtype or not delta.is_contiguous()):
+        raise KernelError("rmsnorm delta must match the input")
+    if rows is not None and return_sum:
+        raise KernelError("rmsnorm cannot return the sum together with a row gather")
+    n = x.shape[0] if rows is None else rows.numel()
+    y = torch.empty((n, hidden), dtype=x.dtype, device=x.device)
+    h_out = torch.empty_like(x) if return_sum else None
+    check(
+        core().tl_rmsnorm(
+            x.data_ptr(), _ptr(delta), _ptr(rows), weight.data_ptr(), dtype_code(weight.dtype),
+            _ptr(h_out), y.data_ptr(), n, hidden, float(eps), dtype_code(x.dtype), _stream(),
+        )
+    )
+    return (h_out, y) if return_sum else y
+
+
+def rope_kv_write(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    positions: torch.Tensor,
+    inv_freq: Optional[torch.Tensor],
+    rotary_dim: int,
+    pairing: int,
+    k_pages: Optional[torch.Tensor] = None,
+    v_pages: Optional[torch.Tensor] = None,
+    slot_mapping: Optional[torch.Tensor] = None,
+    page_size: int = 0,
+) -> None:
+    """Rotate the query and key heads of ``qkv`` [n, (Hq + 2 Hkv) * dh] by position and store keys
+    and values into pages [pages, Hkv, page_size, dh] at ``slot_mapping`` (page * page_size + offset)."""
+    _gpu(qkv, positions, inv_freq, k_pages, v_pages, slot_mapping)
+    _i32(positions, "positions")
+    _i32(slot_mapping, "slot_mapping")
+    n = qkv.shape[0]
+    width = (n_q_heads + 2 * n_kv_heads) * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] != width or not qkv.is_contiguous():
+        raise KernelError(f"qkv must be contiguous [n, {width}], got {tuple(qkv.shape)}")
+    if positions.numel() != n:
+        raise KernelError("positions must have one entry per token")
+    if rotary_dim > 0:
+        if inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2 or not inv_freq.is_contiguous():
+            raise KernelError(f"inv_freq must be float32 with {rotary_dim // 2} entries")
+    if k_pages is not None:
+        if v_pages is None or slot_mapping is None or slot_mapping.numel() != n:
+            raise KernelError("pages need v_pages and one slot per token")
+        for pg in (k_pages, v_pages):
+            if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+                raise KernelError(
+                    f"pages must be contiguous [pages, {n_kv_heads}, {page_size}, {head_dim}] of {qkv.dtype}, got {tuple(pg.shape)} {pg.dtype}"
+                )
+    check(
+        core().tl_rope_kv_write(
+            qkv.data_ptr(), n, n_q_heads, n_kv_heads, head_dim, positions.data_ptr(), _ptr(inv_freq),
+            rotary_dim, pairing, _ptr(k_pages), _ptr(v_pages), _ptr(slot_mapping), page_size,
+            dtype_code(qkv.dtype), _stream(),
+        )
+    )
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` for ``gate_up`` [n, 2F] = gate | up."""
+    _gpu(gate_up)
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2 or not gate_up.is_contiguous():
+        raise KernelError("silu_mul input must be contiguous [n, 2F]")
+    n, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((n, inter), dtype=gate_up.dtype, device=gate_up.device)
+    check(core().tl_silu_mul(gate_up.data_ptr(), out.data_ptr(), n, inter, dtype_code(gate_up.dtype), _stream()))
+    return out
+
+
+def add_bias_(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """In place ``x[:, :len(bias)] += bias`` for a row-major matrix ``x``."""
+    _gpu(x, bias)
+    if x.dim() != 2 or x.stride(1) != 1 or bias.dim() != 1 or bias.numel() > x.shape[1] or bias.dtype != x.dtype:
+        raise KernelError("add_bias: x must be a row-major matrix and bias a vector of its dtype")
+    check(core().tl_add_bias(x.data_ptr(), bias.data_ptr(), x.shape[0], bias.numel(), x.stride(0), dtype_code(x.dtype), _stream()))
+    return x
+
+
+def attention_generic(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    token_seq: torch.Tensor,
+    positions: torch.Tensor,
+    block_table: torch.Tensor,
+    window: int,
+    scale: float,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Attention of each token's query heads (the first Hq * dh columns of ``qkv``) over the paged
+    keys and values of its request; returns [n, Hq * dh]."""
+    _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
+    _i32(token_seq, "token_seq")
+    _i32(positions, "positions")
+    n = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention: qkv must be row-major with at least Hq * dh columns")
+    if token_seq.numel() != n or positions.numel() != n:
+        raise KernelError("attention: token_seq and positions need one entry per token")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("attention: block_table must be an int32 matrix")
+    page_size = k_pages.shape[2]
+    for pg in (k_pages, v_pages):
+        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+            raise KernelError("attention: pages must be contiguous [pages, Hkv, page_size, dh] of the query's dtype")
+    if out is None:
+        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    check(
+        core().tl_attention_generic(
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
+            n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), dtype_code(qkv.dtype), _stream(),
+        )
+    )
+    return out
+
+
+def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x @ w.T`` in true 32-bit arithmetic; x [m, k], w [n, k], both float32."""
+    _gpu(x, w)
+    if x.dtype != torch.float32 or w.dtype != torch.float32:
+        raise KernelError("gemm_f32 takes float32 tensors")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelError(f"gemm_f32: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
+    m, k = x.shape
+    n = w.shape[0]
+    out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    check(core().tl_gemm_f32(x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k, _stream()))
+    return out
+
+
+def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x @ w.T``.  float32: the 32-bit kernel above.  bfloat16: the BLAS library's matrix product
+    (the reference uses its library's here as well: torchllms/models/networks.py:474-493)."""
+    if x.dtype == torch.float32:
+        return gemm_f32(x, w)
+    _gpu(x, w)
+    return torch.nn.functional.linear(x, w)
+
+
+def sample(
+    logits: torch.Tensor,
+    temperature: torch.Tensor,
+    seeds: torch.Tensor,
+    steps: torch.Tensor,
+    top_k: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """One token per row of float32 ``logits`` [n, vocab]; see csrc/sampling.hip for the rule.
+    ``temperature`` float32 [n]; ``seeds``/``steps`` int64 [n] (read as unsigned); ``top_k`` int32 [n]."""
+    _gpu(logits, temperature, seeds, steps, top_k)
+    _i32(top_k, "top_k")
+    if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("sample: logits must be a row-major float32 matrix")
+    n, vocab = logits.shape
+    if temperature.dtype != torch.float32 or temperature.numel() != n:
+        raise KernelError("sample: temperature must be float32 [n]")
+    for t, what in ((seeds, "seeds"), (steps, "steps")):
+        if t.dtype != torch.int64 or t.numel() != n or not t.is_contiguous():
+            raise KernelError(f"sample: {what} must be int64 [n]")
+    if top_k is not None and top_k.numel() != n:
+        raise KernelError("sample: top_k must be int32 [n]")
+    out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    check(
+        core().tl_sample(
+            logits.data_ptr(), logits.stride(0), n, vocab, temperature.data_ptr(), _ptr(top_k),
+            seeds.data_ptr(), steps.data_ptr(), out.data_ptr(), _stream(),
+        )
+    )
+    return out
+
+
+def philox_uniform(seed: int, step: int, n: int, device) -> torch.Tensor:
+    """The uniforms the sampler draws for (seed, step) at indices 0..n-1."""
+    out = torch.empty((n,), dtype=torch.float32, device=device)
+    check(core().tl_philox_uniform(seed & (2**64 - 1), step & (2**64 - 1), out.data_ptr(), n, _stream()))
+    return out

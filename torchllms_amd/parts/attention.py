@@ -1,0 +1,107 @@
+"""Grouped-query attention over paged keys and values."""
+
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..config.spec import PartSpec
+from ..kernels import ops
+from ..kernels.attention import paged_attention
+from .base import MIXERS, POSITIONS, KVNeed, Mixer, ParamSpec
+
+
+@MIXERS.register("attention")
+class Attention(Mixer):
+    """q/k/v projections, position encoding on q and k, keys and values appended to the cache,
+    causal attention of the new queries over everything cached for their request, output
+    projection (reference: torchllms/models/networks.py:460-558; plain formula 355-397).
+
+    Query head h reads key/value head ``h // (num_heads / num_kv_heads)``.  ``window`` w > 0
+    limits a query at position p to keys p-w+1..p.  ``shares_kv``: this layer has no k/v
+    projections and reads the cache of the run named by the execution order.
+    """
+
+    def __init__(
+        self,
+        hidden_size: int,
+        num_heads: int,
+        num_kv_heads: int,
+        head_dim: int,
+        qkv_bias: bool,
+        softmax_scale: float,
+        window: int,
+        position: PartSpec,
+        shares_kv: bool = False,
+    ):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.qkv_bias = qkv_bias
+        self.softmax_scale = float(softmax_scale)
+        self.window = int(window)
+        self.shares_kv = shares_kv
+        self.position = POSITIONS.build(position)
+        self.wqkv: Optional[torch.Tensor] = None
+        self.bqkv: Optional[torch.Tensor] = None
+        self.wo: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        q = self.num_heads * self.head_dim
+        kv = self.num_kv_heads * self.head_dim
+        specs = {"wq.weight": ParamSpec((q, self.hidden_size)), "wo.weight": ParamSpec((self.hidden_size, q))}
+        if not self.shares_kv:
+            specs["wk.weight"] = ParamSpec((kv, self.hidden_size))
+            specs["wv.weight"] = ParamSpec((kv, self.hidden_size))
+        if self.qkv_bias:
+            specs["wq.bias"] = ParamSpec((q,), init="zeros")
+            if not self.shares_kv:
+                specs["wk.bias"] = ParamSpec((kv,), init="zeros")
+                specs["wv.bias"] = ParamSpec((kv,), init="zeros")
+        return specs
+
+    def cache_need(self):
+        if self.shares_kv:
+            return None
+        return KVNeed(num_kv_heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window)
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        names = ["wq"] if self.shares_kv else ["wq", "wk", "wv"]
+        # one fused projection [q rows | k rows | v rows]: a single matrix product per token batch
+        self.wqkv = torch.cat([tensors[f"{n}.weight"] for n in names], dim=0).contiguous()
+        if self.qkv_bias:
+            self.bqkv = torch.cat([tensors[f"{n}.bias"] for n in names], dim=0).contiguous()
+        self.wo = tensors["wo.weight"].contiguous()
+        self.position.to(self.wo.device)
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        n_kv_in_row = 0 if self.shares_kv else self.num_kv_heads
+        qkv = ops.linear(x, self.wqkv)
+        if self.bqkv is not None:
+            ops.add_bias_(qkv, self.bqkv)
+        rot = self.position.rotary_args()
+        g = cache.group
+        store = cache.writes and not self.shares_kv
+        ops.rope_kv_write(
+            qkv,
+            self.num_heads,
+            n_kv_in_row,
+            self.head_dim,
+            ctx.positions,
+            rot.inv_freq if rot else None,
+            rot.rotary_dim if rot else 0,
+            rot.pairing if rot else 0,
+            cache.k_pages if store else None,
+            cache.v_pages if store else None,
+            ctx.slot_mappings[g] if store else None,
+            cache.page_size if store else 0,
+        )
+        attn = paged_attention(
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
+            ctx, g, self.window, self.softmax_scale,
+        )
+        return ops.linear(attn, self.wo)

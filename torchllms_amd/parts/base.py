@@ -1,0 +1,200 @@
+"""Interfaces and registries of the parts a model is put together from.
+
+A part is built from its ``PartSpec.params`` alone: it is told its sizes and constants and
+never learns which model it sits in.  These registries hold them:
+
+======================  ==========================================================
+``MIXERS``              token mixers (attention, anything with state of its own)
+``FEED_FORWARDS``       per-token feed-forward networks (dense or routed)
+``NORMS``               normalisations
+``POSITIONS``           position encodings used inside a mixer
+``BLOCKS``              arrangements of mixer / feed-forward / norms in one layer
+``EMBEDDINGS``          token id -> vector
+``HEADS``               vector -> logits
+======================  ==========================================================
+
+A part declares its tensors with ``param_specs()`` (names local to the part) and receives
+them, already on the device and in their final dtype, through ``bind()``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, Optional, Tuple
+
+import torch
+
+from ..config.spec import PartSpec
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One tensor a part expects.
+
+    ``kind``: "matrix" (kept in the model's compute dtype), "vector" (compute dtype, but a
+    tensor stored in 32-bit stays in 32-bit), "int" (an integer table, kept as int32).
+    ``init``: how the random-weights mode fills it: "normal" N(0, 0.02), "ones", "zeros".
+    """
+
+    shape: Tuple[int, ...]
+    kind: str = "matrix"
+    init: str = "normal"
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """A mixer that keeps keys and values of past tokens in pages.
+
+    ``window`` = 0: every past token stays visible.  ``window`` = w > 0: a token at position p
+    sees positions p-w+1 .. p only, so pages that lie wholly before that may be given back.
+    """
+
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A mixer that keeps state of fixed size per request (one row per request slot)."""
+
+    shape: Tuple[int, ...]
+    dtype: str = "float32"
+
+
+class Part:
+    """Base of all parts."""
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Take ownership of this part's tensors (keys as in ``param_specs``)."""
+        if tensors:
+            raise ValueError(f"{type(self).__name__} takes no tensors, got {sorted(tensors)}")
+
+
+class Norm(Part):
+    """y = norm(x).  ``forward_add`` fuses the residual sum that precedes the norm."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def forward_add(self, h: torch.Tensor, delta: Optional[torch.Tensor]):
+        """Return ``(h + delta, norm(h + delta))``; ``delta`` may be None."""
+        if delta is not None:
+            h = h + delta
+        return h, self.forward(h)
+
+    def forward_rows(self, h: torch.Tensor, delta: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
+        """``norm((h + delta)[rows])`` for an int32 index vector ``rows``."""
+        idx = rows.long()
+        x = h.index_select(0, idx)
+        if delta is not None:
+            x = x + delta.index_select(0, idx)
+        return self.forward(x)
+
+
+class PositionEncoding(Part):
+    """Position information applied to queries and keys inside a mixer."""
+
+    def rotary_args(self):
+        """``None`` (queries and keys pass unchanged) or a ``RotaryArgs`` that the fused
+        rotate-and-store kernel understands."""
+        return None
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self):
+        """``KVNeed``, ``StateNeed`` or None."""
+        return None
+
+    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+        """``x``: [tokens, hidden] of this step.  ``ctx``: the step's ``StepContext``.
+        ``cache``: what the cache manager holds for this run (a ``KVLayerView``, a
+        ``StateView`` or None), already pointing at the right layer."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of one layer.  ``forward`` takes the residual stream ``h`` and a pending
+    ``delta`` that has not been added to it yet (None for the first layer) and returns the
+    same pair, so the sum can be fused into whatever reads it next."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ffn_norm: Norm):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.ffn_norm = ffn_norm
+
+    #: names under which the four sub-parts' tensors appear inside a layer
+    SLOTS = ("mixer_norm", "mixer", "ffn_norm", "ffn")
+
+    def sub_parts(self) -> Dict[str, Part]:
+        return {
+            "mixer_norm": self.mixer_norm,
+            "mixer": self.mixer,
+            "ffn_norm": self.ffn_norm,
+            "ffn": self.feed_forward,
+        }
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        out = {}
+        for slot, part in self.sub_parts().items():
+            for name, spec in part.param_specs().items():
+                out[f"{slot}.{name}"] = spec
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for slot, part in self.sub_parts().items():
+            prefix = slot + "."
+            part.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
+
+    def forward(self, h, delta, ctx, cache):
+        raise NotImplementedError
+
+
+class Registry(dict):
+    def __init__(self, what: str):
+        super().__init__()
+        self.what = what
+
+    def register(self, name: str) -> Callable:
+        def deco(cls):
+            self[name] = cls
+            return cls
+
+        return deco
+
+    def build(self, spec: PartSpec, **extra: Any):
+        try:
+            cls = self[spec.kind]
+        except KeyError:
+            raise KeyError(f"no {self.what} named {spec.kind!r}; registered: {sorted(self)}") from None
+        return cls(**spec.params, **extra)
+
+
+class Embedding(Part):
+    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        """int32 token ids [n] -> [n, hidden]."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """[n, hidden] -> float32 logits [n, vocab]."""
+        raise NotImplementedError
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITIONS = Registry("position encoding")
+BLOCKS = Registry("block arrangement")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("output head")

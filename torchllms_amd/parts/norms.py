@@ -1,0 +1,38 @@
+"""Normalisations."""
+
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import NORMS, Norm, ParamSpec
+
+
+@NORMS.register("rmsnorm")
+class RMSNorm(Norm):
+    """``y = cast(x32 * rsqrt(mean(x32^2) + eps)) * weight``: statistics and scaling in 32-bit,
+    the weight multiply after the cast back (reference: torchllms/models/networks.py:186-200)."""
+
+    def __init__(self, size: int, eps: float):
+        self.size = size
+        self.eps = float(eps)
+        self.weight: Optional[torch.Tensor] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.size,), kind="vector", init="ones")}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.weight = tensors["weight"].contiguous()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.rmsnorm(x, self.weight, self.eps)
+
+    def forward_add(self, h: torch.Tensor, delta: Optional[torch.Tensor]):
+        if delta is None:
+            return h, ops.rmsnorm(h, self.weight, self.eps)
+        return ops.rmsnorm(h, self.weight, self.eps, delta=delta, return_sum=True)
+
+    def forward_rows(self, h: torch.Tensor, delta: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
+        return ops.rmsnorm(h, self.weight, self.eps, delta=delta, rows=rows)
