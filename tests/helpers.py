@@ -73,13 +73,28 @@ TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
 PAGE_SIZE = {"A": 8, "B": 16, "C": 4}
 
 
-def make_folder(tmp_path, cfg_dict: dict, seed: int = 0, dtype=torch.bfloat16, norm_jitter: float = 0.1) -> Path:
-    """A model folder with random weights, made by the package's random-weights mode."""
+def make_folder(tmp_path, cfg_dict: dict, seed: int = 0, dtype=torch.bfloat16, norm_jitter: float = 0.1,
+                sharpen: bool = False) -> Path:
+    """A model folder with random weights, made by the package's random-weights mode.
+
+    ``sharpen``: N(0, 0.02) weights give nearly uniform attention, in which one wrong or missing
+    key hardly shows.  Scaling the q and k projections so that scores have a spread of about 4
+    makes every query attend to a few keys, near and far, and a fault in any of them shows."""
+    from safetensors.torch import save_file
+
     from torchllms_amd.config import LlamaConfig
     from torchllms_amd.weights import write_model_folder
 
     cfg = LlamaConfig.from_dict(cfg_dict)
-    return write_model_folder(tmp_path, cfg, seed=seed, dtype=dtype, norm_jitter=norm_jitter)
+    folder = write_model_folder(tmp_path, cfg, seed=seed, dtype=dtype, norm_jitter=norm_jitter)
+    if sharpen:
+        _, tensors = read_folder(folder)
+        factor = 100.0 / cfg.hidden_size ** 0.5
+        for name in list(tensors):
+            if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
+                tensors[name] = (tensors[name].float() * factor).to(dtype)
+        save_file(tensors, str(folder / "model.safetensors"), metadata={"format": "pt"})
+    return folder
 
 
 def read_folder(folder) -> (dict, Dict[str, torch.Tensor]):

@@ -1,0 +1,203 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16: each request alone and
+whole; most of it in one step and the last 32 tokens one by one; in portions of changing size down
+to two tokens; and mixed, up to four live requests with so few pages that they are used again."""
+
+import pytest
+import torch
+
+from . import schedules
+from .helpers import PAGE_SIZE, TINY, make_folder, random_tokens, read_folder
+from .plain import llama as plain
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [70, 41, 100, 35, 50, 33], "B": [66, 40, 130, 35, 90], "C": [45, 300, 37, 64, 120]}
+FP32_ATOL = 2e-5
+
+
+def run_trace(engine, steps):
+    """Feed a trace through ``Engine.step``; returns {(request, position): logits row on the CPU}."""
+    from torchllms_amd.engine import StepEntry
+
+    out = {}
+    rows = schedules.positions_of(steps)
+    for s, where in zip(steps, rows):
+        entries = []
+        for e in s["entries"]:
+            if not engine.cache.has(e["id"]):
+                engine.admit(e["id"])
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+        logits = engine.step(entries).cpu()
+        assert logits.shape == (len(where), engine.vocab_size)
+        for key, row in zip(where, logits):
+            assert key not in out
+            out[key] = row
+        for rid in s["end"]:
+            engine.free(rid)
+        engine.cache.check_invariants()
+    assert engine.cache.live == []
+    assert all(p.free_count == p.num_pages for p in engine.cache.pools)
+    return out
+
+
+class Case:
+    """One tiny configuration: its folder, requests, plain logits, and engines per dtype."""
+
+    def __init__(self, name, tmp):
+        from torchllms_amd.engine import Engine
+
+        self.name = name
+        cfg = TINY[name]
+        self.folder = make_folder(tmp / name, cfg, seed=11, dtype=torch.bfloat16, norm_jitter=0.1, sharpen=True)
+        self.cfg, self.weights = read_folder(self.folder)
+        self.requests = {f"r{i}": random_tokens(n, cfg["vocab_size"], 100 + i) for i, n in enumerate(LENGTHS[name])}
+        self.plain32 = {rid: plain.forward(self.weights, self.cfg, t, torch.float32) for rid, t in self.requests.items()}
+        self.plain16 = {rid: plain.forward(self.weights, self.cfg, t, torch.bfloat16).float() for rid, t in self.requests.items()}
+        self.traces = {
+            "whole": schedules.whole(self.requests),
+            "tail": schedules.tail(self.requests),
+            "portions": schedules.portions(self.requests),
+            "mixed": schedules.mixed(self.requests),
+        }
+        page = PAGE_SIZE[name]
+        pool_tokens = max(schedules.max_live_tokens(t) for t in self.traces.values())
+        self.engines = {
+            dt: Engine.from_folder(self.folder, dtype=dt, page_size=page, num_pages=-(-pool_tokens // page), max_seqs=4)
+            for dt in ("float32", "bfloat16")
+        }
+        self._results = {}
+
+    def result(self, dtype, schedule):
+        key = (dtype, schedule)
+        if key not in self._results:
+            self._results[key] = run_trace(self.engines[dtype], self.traces[schedule])
+        return self._results[key]
+
+
+@pytest.fixture(scope="module")
+def cases(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("models")
+    return {name: Case(name, tmp) for name in TINY}
+
+
+def _max_err(result, truth):
+    worst, where = 0.0, None
+    for (rid, pos), row in result.items():
+        e = (row - truth[rid][pos]).abs().max().item()
+        if e > worst:
+            worst, where = e, (rid, pos)
+    return worst, where
+
+
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_float32_matches_the_plain_model(cases, name, schedule):
+    case = cases[name]
+    got = case.result("float32", schedule)
+    assert len(got) == sum(len(t) for t in case.requests.values())
+    err, where = _max_err(got, case.plain32)
+    assert err < FP32_ATOL, f"{name}/{schedule}: first look at {where}, max abs error {err}"
+
+
+@pytest.mark.parametrize("schedule", ["tail", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_float32_does_not_depend_on_the_schedule(cases, name, schedule):
+    """In 32-bit every kernel accumulates in an order fixed per output element, so logits are the
+    same bits however the tokens were cut into steps, batched, or placed in pages."""
+    case = cases[name]
+    ref = case.result("float32", "whole")
+    got = case.result("float32", schedule)
+    diff = [k for k in ref if not torch.equal(ref[k], got[k])]
+    assert not diff, f"{name}/{schedule}: {len(diff)} positions differ, first {sorted(diff)[0]}"
+
+
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_bfloat16_is_as_close_as_plain_bfloat16(cases, name, schedule):
+    """The yardstick for bfloat16 is the plain model run in bfloat16: the engine's distance from
+    the 32-bit truth may not exceed twice the plain bfloat16 model's own, in the maximum and in
+    the mean."""
+    case = cases[name]
+    got = case.result("bfloat16", schedule)
+    ref_max = max((case.plain16[r] - case.plain32[r]).abs().max().item() for r in case.requests)
+    ref_mean = torch.cat([(case.plain16[r] - case.plain32[r]).abs().flatten() for r in case.requests]).mean().item()
+    err, where = _max_err(got, case.plain32)
+    mean = torch.stack([(row - case.plain32[rid][pos]).abs().mean() for (rid, pos), row in got.items()]).mean().item()
+    assert err <= 2 * ref_max, f"{name}/{schedule}: {where} max abs error {err} vs plain bfloat16 {ref_max}"
+    assert mean <= 2 * ref_mean, f"{name}/{schedule}: mean abs error {mean} vs plain bfloat16 {ref_mean}"
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_bfloat16_schedules_agree(cases, name):
+    case = cases[name]
+    ref = case.result("bfloat16", "whole")
+    ref_max = max((case.plain16[r] - case.plain32[r]).abs().max().item() for r in case.requests)
+    for schedule in ("tail", "portions", "mixed"):
+        got = case.result("bfloat16", schedule)
+        err = max((ref[k] - got[k]).abs().max().item() for k in ref)
+        assert err <= 2 * ref_max, f"{name}/{schedule} differs from whole by {err}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens_of_a_sequence(cases, dtype):
+    """Positions 0, 1, 2: a one-token step at position 0, then another, then a two-token portion."""
+    from torchllms_amd.engine import StepEntry
+
+    case = cases["B"]
+    eng = case.engines[dtype]
+    toks = case.requests["r0"]
+    eng.admit("first")
+    rows = [eng.step([StepEntry("first", toks[0:1], [0])]), eng.step([StepEntry("first", toks[1:2], [0])]),
+            eng.step([StepEntry("first", toks[2:4], [0, 1])])]
+    eng.free("first")
+    got = torch.cat(rows).cpu()
+    want = case.plain32["r0"][:4]
+    tol = FP32_ATOL if dtype == "float32" else 2 * (case.plain16["r0"][:4] - want).abs().max().item()
+    assert (got - want).abs().max().item() <= tol
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(cases, dtype):
+    """A short prompt, then 280 tokens one by one: many pages, many steps."""
+    from torchllms_amd.engine import StepEntry
+
+    case = cases["C"]
+    eng = case.engines[dtype]
+    toks = case.requests["r1"]
+    eng.admit("long")
+    rows = [eng.step([StepEntry("long", toks[:20], [19])])]
+    for i in range(20, len(toks)):
+        rows.append(eng.step([StepEntry("long", toks[i : i + 1], [0])]))
+    eng.free("long")
+    got = torch.cat(rows).cpu()
+    want = case.plain32["r1"][19:]
+    tol = FP32_ATOL if dtype == "float32" else 2 * (case.plain16["r1"][19:] - want).abs().max().item()
+    err = (got - want).abs().amax(dim=1)
+    assert err.max().item() <= tol, f"first position over tolerance: {19 + int((err > tol).nonzero()[0])}"
+
+
+def test_step_refuses_what_it_cannot_run(cases):
+    from torchllms_amd.cache import OutOfPages
+    from torchllms_amd.engine import StepEntry
+
+    eng = cases["A"].engines["float32"]
+    with pytest.raises(KeyError, match="not live"):
+        eng.step([StepEntry("nobody", [1])])
+    eng.admit("x")
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        eng.step([StepEntry("x", [256])])
+    with pytest.raises(ValueError, match="twice"):
+        eng.step([StepEntry("x", [1]), StepEntry("x", [2])])
+    with pytest.raises(ValueError, match="max_model_len"):
+        eng.step([StepEntry("x", [1] * 129)])
+    eng.admit("y")
+    eng.cache.admit("hog")
+    eng.cache.extend("hog", (eng.cache.free_pages() - 1) * eng.page_size)  # one page is left
+    with pytest.raises(OutOfPages):
+        eng.step([StepEntry("x", [1, 2, 3]), StepEntry("y", [1] * (eng.page_size + 1))])
+    assert eng.cache.free_pages() == 1 and eng.num_tokens("x") == 0 and eng.cache.block_table("x") == []
+    eng.cache.free("hog")
+    assert eng.step([StepEntry("x", [1, 2, 3])]).shape == (0, 256)  # nothing wanted
+    eng.free("x")
+    eng.free("y")
+    eng.cache.check_invariants()

@@ -1,0 +1,430 @@
+"""Each kernel alone against its plain reference, at other sizes than the engine tests use."""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from .plain import llama as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _ops():
+    from torchllms_amd.kernels import ops
+
+    return ops
+
+
+def _i32(x):
+    return torch.tensor(x, dtype=torch.int32, device=DEV)
+
+
+def _close_bf16(got, want, frac=0.002):
+    """bfloat16 results may differ from the plain ones by one rounding in a few places."""
+    got, want = got.float(), want.float()
+    bad = (got - want).abs() > (want.abs() * 2 ** -7 + 1e-6)
+    assert bad.float().mean().item() <= frac, f"{int(bad.sum())} of {bad.numel()} entries are off by more than one rounding"
+    assert torch.allclose(got, want, rtol=2 ** -6, atol=1e-5)
+
+
+# ----------------------------------------------------------------------------- embedding
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [72, 128, 1001])
+def test_embed(dtype, hidden):
+    torch.manual_seed(0)
+    table = torch.randn(1000, hidden).to(dtype).to(DEV)
+    toks = torch.randint(0, 1000, (37,), dtype=torch.int32, device=DEV)
+    assert torch.equal(_ops().embed(toks, table), table[toks.long()])
+
+
+# ----------------------------------------------------------------------------- RMS norm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden, eps", [(100, 1e-5), (4096, 1e-6), (5000, 3e-4)])
+def test_rmsnorm(dtype, hidden, eps):
+    torch.manual_seed(0)
+    x = (torch.randn(9, hidden) * 3).to(dtype)
+    w = (1 + 0.2 * torch.randn(hidden)).to(dtype)
+    got = _ops().rmsnorm(x.to(DEV), w.to(DEV), eps).cpu()
+    want = plain.rms_norm(x, w, eps)
+    if dtype == torch.float32:
+        assert torch.allclose(got, want, rtol=2e-6, atol=1e-6)
+    else:
+        _close_bf16(got, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_with_residual_sum_rows_and_eps(dtype):
+    torch.manual_seed(1)
+    h = torch.randn(12, 320).to(dtype)
+    d = torch.randn(12, 320).to(dtype)
+    w = (1 + 0.2 * torch.randn(320)).to(dtype)
+    s, y = _ops().rmsnorm(h.to(DEV), w.to(DEV), 1e-5, delta=d.to(DEV), return_sum=True)
+    assert torch.equal(s.cpu(), h + d)  # the sum is rounded once, as an addition in the model's dtype
+    want = plain.rms_norm(h + d, w, 1e-5)
+    _close_bf16(y.cpu(), want) if dtype == torch.bfloat16 else torch.testing.assert_close(y.cpu(), want, rtol=2e-6, atol=1e-6)
+    rows = _i32([7, 0, 7, 11])
+    y2 = _ops().rmsnorm(h.to(DEV), w.to(DEV), 1e-5, delta=d.to(DEV), rows=rows).cpu()
+    assert torch.equal(y2, y.cpu()[[7, 0, 7, 11]])
+    # eps sits inside the root: a tiny row tells 1e-5 from 1e-6
+    tiny = torch.full((1, 64), 1e-3).to(dtype).to(DEV)
+    one = torch.ones(64, dtype=dtype, device=DEV)
+    a = _ops().rmsnorm(tiny, one, 1e-5)[0, 0].item()
+    b = _ops().rmsnorm(tiny, one, 1e-6)[0, 0].item()
+    c = float(tiny[0, 0])
+    assert a == pytest.approx(c / math.sqrt(c * c + 1e-5), rel=1e-2) and b == pytest.approx(c / math.sqrt(c * c + 1e-6), rel=1e-2)
+    assert abs(a - b) > 0.1
+
+
+def test_rmsnorm_weight_kept_in_32_bit():
+    torch.manual_seed(2)
+    x = torch.randn(4, 96).bfloat16()
+    w = 1 + 0.2 * torch.randn(96)
+    got = _ops().rmsnorm(x.to(DEV), w.to(DEV), 1e-5).cpu()
+    xf = x.float()
+    n = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).bfloat16()
+    _close_bf16(got, (n.float() * w).bfloat16())
+
+
+# ----------------------------------------------------------------------------- rotary + cache write
+def _pages(n_pages, hkv, page, dh, dtype):
+    return (torch.zeros(n_pages, hkv, page, dh, dtype=dtype, device=DEV), torch.zeros(n_pages, hkv, page, dh, dtype=dtype, device=DEV))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq, hkv, dh, page", [(6, 3, 48, 4), (5, 5, 16, 16), (8, 1, 128, 32)])
+def test_rope_and_cache_write(dtype, hq, hkv, dh, page):
+    torch.manual_seed(0)
+    n = 23
+    qkv = torch.randn(n, (hq + 2 * hkv) * dh).to(dtype)
+    pos = torch.randint(0, 500, (n,))
+    inv_freq = plain.rope_inverse_frequencies(dh, 10000.0, None)
+    n_pages = 12
+    perm = torch.randperm(n_pages * page)[:n]  # every token a slot of its own, scattered over the pages
+    k_pages, v_pages = _pages(n_pages, hkv, page, dh, dtype)
+    dev = qkv.to(DEV)
+    _ops().rope_kv_write(dev, hq, hkv, dh, _i32(pos.tolist()), inv_freq.to(DEV), dh, 0, k_pages, v_pages, _i32(perm.tolist()), page)
+    q = qkv[:, : hq * dh].view(n, hq, dh)
+    k = qkv[:, hq * dh : (hq + hkv) * dh].view(n, hkv, dh)
+    v = qkv[:, (hq + hkv) * dh :].view(n, hkv, dh)
+    want_q = plain.rope_rotate_interleaved(q, pos, inv_freq)
+    want_k = plain.rope_rotate_interleaved(k, pos, inv_freq)
+    tol = dict(rtol=1e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=1e-3)
+    torch.testing.assert_close(dev[:, : hq * dh].cpu().view(n, hq, dh), want_q, **tol)
+    got_k = torch.stack([k_pages[s // page, :, s % page].cpu() for s in perm.tolist()])
+    got_v = torch.stack([v_pages[s // page, :, s % page].cpu() for s in perm.tolist()])
+    torch.testing.assert_close(got_k, want_k, **tol)
+    assert torch.equal(got_v, v)  # values are stored as they are
+    # nothing else was touched
+    mask = torch.ones(n_pages * page, dtype=torch.bool)
+    mask[perm] = False
+    flat_k = k_pages.permute(0, 2, 1, 3).reshape(n_pages * page, hkv, dh).cpu()
+    assert flat_k[mask].abs().sum() == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_half_pairing_partial_rotary_and_no_pages(dtype):
+    torch.manual_seed(0)
+    n, hq, hkv, dh, rot = 7, 3, 1, 32, 16
+    qkv = torch.randn(n, (hq + 2 * hkv) * dh).to(dtype)
+    pos = torch.arange(3, 3 + n)
+    inv_freq = plain.rope_inverse_frequencies(rot, 100.0, None)
+    dev = qkv.to(DEV)
+    _ops().rope_kv_write(dev, hq, hkv, dh, _i32(pos.tolist()), inv_freq.to(DEV), rot, 1)
+    heads = qkv.view(n, hq + 2 * hkv, dh)
+    want = heads.clone()
+    want[:, : hq + hkv, :rot] = plain.rope_rotate_half_split(heads[:, : hq + hkv, :rot], pos, inv_freq)
+    tol = dict(rtol=1e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=1e-3)
+    torch.testing.assert_close(dev.cpu().view(n, hq + 2 * hkv, dh), want, **tol)  # k rotated in place, v and the tail untouched
+    # rotary_dim 0: nothing moves
+    dev = qkv.to(DEV)
+    _ops().rope_kv_write(dev, hq, hkv, dh, _i32(pos.tolist()), None, 0, 0)
+    assert torch.equal(dev.cpu(), qkv)
+
+
+def test_cache_write_round_trip_with_distinct_values():
+    # reference: torchllms/models/test_paged_kv.py:440-484 (append then extract, value = position)
+    hq, hkv, dh, page = 2, 2, 8, 4
+    n = 11
+    qkv = torch.zeros(n, (hq + 2 * hkv) * dh, dtype=torch.bfloat16)
+    for p in range(n):
+        qkv[p, hq * dh : (hq + hkv) * dh] = p + 1
+        qkv[p, (hq + hkv) * dh :] = -(p + 1)
+    k_pages, v_pages = _pages(5, hkv, page, dh, torch.bfloat16)
+    table = [3, 0, 4]
+    slots = [table[p // page] * page + p % page for p in range(n)]
+    _ops().rope_kv_write(qkv.to(DEV), hq, hkv, dh, _i32(list(range(n))), None, 0, 0, k_pages, v_pages, _i32(slots), page)
+    for p in range(n):
+        assert (k_pages[table[p // page], :, p % page] == p + 1).all()
+        assert (v_pages[table[p // page], :, p % page] == -(p + 1)).all()
+
+
+# ----------------------------------------------------------------------------- SwiGLU gate, bias
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    torch.manual_seed(0)
+    gu = (torch.randn(5, 2 * 203) * 3).to(dtype)
+    got = _ops().silu_mul(gu.to(DEV)).cpu()
+    want = F.silu(gu[:, :203]) * gu[:, 203:]
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, rtol=2e-6, atol=1e-6)
+    else:
+        _close_bf16(got, want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_bias(dtype):
+    torch.manual_seed(0)
+    x = torch.randn(6, 50).to(dtype)
+    b = torch.randn(30).to(dtype)
+    got = _ops().add_bias_(x.to(DEV), b.to(DEV)).cpu()
+    want = x.clone()
+    want[:, :30] = x[:, :30] + b
+    assert torch.equal(got, want)
+
+
+# ----------------------------------------------------------------------------- 32-bit matrix product
+@pytest.mark.parametrize("m, n, k", [(1, 100, 50), (7, 257, 1000), (130, 64, 64), (65, 129, 17)])
+def test_gemm_f32_is_true_32_bit(m, n, k):
+    torch.manual_seed(0)
+    x, w = torch.randn(m, k), torch.randn(n, k)
+    got = _ops().gemm_f32(x.to(DEV), w.to(DEV)).cpu()
+    want = (x.double() @ w.double().T)
+    assert (got.double() - want).abs().max().item() < 2e-6 * math.sqrt(k) * 4
+    # a row's result does not depend on the rows beside it
+    alone = _ops().gemm_f32(x[:1].to(DEV), w.to(DEV)).cpu()
+    assert torch.equal(alone[0], got[0])
+
+
+# ----------------------------------------------------------------------------- attention
+def _paged(k, v, page, n_pages, seed=0, dtype=torch.float32):
+    """Scatter dense per-request keys/values [S, Hkv, dh] into shuffled pages; returns pages and
+    the block table."""
+    S, hkv, dh = k.shape
+    g = torch.Generator().manual_seed(seed)
+    n_blocks = -(-S // page)
+    table = torch.randperm(n_pages, generator=g)[:n_blocks].tolist()
+    # unused pages hold large values: reading one shows
+    k_pages = torch.full((n_pages, hkv, page, dh), 50.0, dtype=dtype)
+    v_pages = torch.full((n_pages, hkv, page, dh), -50.0, dtype=dtype)
+    for p in range(S):
+        k_pages[table[p // page], :, p % page] = k[p]
+        v_pages[table[p // page], :, p % page] = v[p]
+    return k_pages.to(DEV), v_pages.to(DEV), table
+
+
+def _attend(fn, q, k, v, page, window=0, q_start=None, scale=None, dtype=torch.float32, n_pages=None):
+    """Run ``fn`` (a kernel wrapper) for the queries ``q`` [Sq, Hq, dh], which are the last Sq
+    positions of a request whose keys/values are ``k``, ``v`` [S, Hkv, dh]."""
+    sq, hq, dh = q.shape
+    S, hkv, _ = k.shape
+    n_pages = n_pages or (-(-S // page) + 3)
+    k_pages, v_pages, table = _paged(k.to(dtype), v.to(dtype), page, n_pages, dtype=dtype)
+    q_start = S - sq if q_start is None else q_start
+    qkv = q.reshape(sq, hq * dh).to(dtype).to(DEV).contiguous()
+    out = fn(
+        qkv, hq, hkv, dh, k_pages, v_pages, _i32([0] * sq), _i32(list(range(q_start, q_start + sq))), _i32([table]),
+        window, scale if scale is not None else dh ** -0.5,
+    )
+    return out.float().cpu()
+
+
+def _windowed_plain(q, k, v, window):
+    """The plain attention, one query at a time over the keys its window leaves."""
+    sq = q.shape[0]
+    S = k.shape[0]
+    rows = []
+    for i in range(sq):
+        p = S - sq + i
+        lo = max(p - window + 1, 0) if window > 0 else 0
+        rows.append(plain.attention(q[i : i + 1], k[lo : p + 1], v[lo : p + 1]))
+    return torch.cat(rows)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize(
+    "hq, hkv, dh, page, S, sq",
+    [(4, 2, 16, 8, 37, 37), (6, 3, 48, 4, 150, 9), (8, 1, 128, 16, 300, 1), (3, 3, 80, 32, 70, 70), (2, 1, 256, 16, 65, 2), (4, 4, 64, 1, 20, 20)],
+)
+def test_attention_generic(dtype, hq, hkv, dh, page, S, sq):
+    torch.manual_seed(0)
+    q = torch.randn(sq, hq, dh) * 2
+    k = torch.randn(S, hkv, dh)
+    v = torch.randn(S, hkv, dh)
+    if dtype == torch.bfloat16:
+        q, k, v = q.bfloat16().float(), k.bfloat16().float(), v.bfloat16().float()
+    got = _attend(_ops().attention_generic, q, k, v, page, dtype=dtype)
+    want = plain.attention(q, k, v)
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
+    else:
+        torch.testing.assert_close(got, want, rtol=2 ** -7, atol=2 ** -7)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_a_far_key_among_hundreds(dtype):
+    """One key far back matches the query; its value must come out.  A kernel that drops or
+    misplaces a block of keys, or reads the wrong page, returns something else."""
+    torch.manual_seed(0)
+    hq, hkv, dh, page, S = 4, 2, 32, 16, 700
+    k = torch.randn(S, hkv, dh) * 0.1
+    v = torch.randn(S, hkv, dh)
+    q = torch.randn(1, hq, dh) * 0.1
+    for far in (0, 1, 15, 16, 63, 64, 65, 333, 639, 640, 698, 699):
+        kk, qq = k.clone(), q.clone()
+        direction = torch.randn(dh)
+        direction /= direction.norm()
+        kk[far, :, :] = direction * 12
+        qq[0, :, :] = direction * 12 * math.sqrt(dh) / 4  # score 36 for that key, about 0 for all others
+        got = _attend(_ops().attention_generic, qq, kk, v, page, dtype=dtype).view(hq, dh)
+        want = v[far].repeat_interleave(hq // hkv, dim=0)
+        tol = 1e-4 if dtype == torch.float32 else 2e-2
+        assert (got - want).abs().max().item() < tol, f"key {far}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 64, 100])
+def test_attention_window_edge(dtype, window):
+    """The key just outside the window is made to match the query: it must not be seen.  The one
+    just inside is seen."""
+    torch.manual_seed(0)
+    hq, hkv, dh, page, S, sq = 2, 1, 16, 8, 230, 3
+    k = torch.randn(S, hkv, dh) * 0.1
+    v = torch.randn(S, hkv, dh)
+    q = torch.randn(sq, hq, dh)
+    want = _windowed_plain(q, k, v, window)
+    got = _attend(_ops().attention_generic, q, k, v, page, window=window, dtype=dtype)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+    torch.testing.assert_close(got, want, **tol)
+    p = S - 1
+    direction = torch.ones(dh) / math.sqrt(dh)
+    qq = q.clone()
+    qq[-1] = direction * 40
+    outside = p - window
+    if outside >= 0:
+        kk = k.clone()
+        kk[outside, 0] = direction * 10
+        got = _attend(_ops().attention_generic, qq, kk, v, page, window=window, dtype=dtype)
+        torch.testing.assert_close(got[-1:], _windowed_plain(qq, kk, v, window)[-1:], **tol)
+        assert (got[-1].view(hq, dh) - v[outside, 0]).abs().max() > 0.05
+    inside = p - window + 1
+    kk = k.clone()
+    kk[inside, 0] = direction * 10
+    got = _attend(_ops().attention_generic, qq, kk, v, page, window=window, dtype=dtype)
+    assert (got[-1].view(hq, dh) - v[inside, 0]).abs().max() < (1e-3 if dtype == torch.float32 else 3e-2)
+
+
+def test_attention_window_never_reads_released_pages():
+    """Blocks wholly before the window are -1 in the block table; the kernel must not touch them."""
+    torch.manual_seed(0)
+    hq, hkv, dh, page, S, window = 2, 2, 16, 4, 60, 6
+    q, k, v = torch.randn(1, hq, dh), torch.randn(S, hkv, dh), torch.randn(S, hkv, dh)
+    k_pages, v_pages, table = _paged(k, v, page, 20)
+    first_needed = (S - 1 - window + 1) // page
+    table = [-1 if b < first_needed else t for b, t in enumerate(table)]
+    out = _ops().attention_generic(
+        q.reshape(1, hq * dh).to(DEV), hq, hkv, dh, k_pages, v_pages, _i32([0]), _i32([S - 1]), _i32([table]), window, dh ** -0.5
+    ).cpu()
+    torch.testing.assert_close(out, _windowed_plain(q, k, v, window), rtol=1e-5, atol=1e-5)
+
+
+def test_attention_batch_of_requests_and_strided_queries():
+    """Three requests in one launch, queries read out of a wider row (the fused q|k|v buffer)."""
+    torch.manual_seed(0)
+    hq, hkv, dh, page = 4, 2, 32, 8
+    lens = [(21, 21), (50, 1), (33, 5)]  # (tokens cached, new queries)
+    n_pages = 20
+    k_pages = torch.zeros(n_pages, hkv, page, dh)
+    v_pages = torch.zeros(n_pages, hkv, page, dh)
+    free = torch.randperm(n_pages).tolist()
+    tables, wants, qs, seq, pos = [], [], [], [], []
+    for b, (S, sq) in enumerate(lens):
+        k, v, q = torch.randn(S, hkv, dh), torch.randn(S, hkv, dh), torch.randn(sq, hq, dh)
+        table = [free.pop() for _ in range(-(-S // page))]
+        for p in range(S):
+            k_pages[table[p // page], :, p % page] = k[p]
+            v_pages[table[p // page], :, p % page] = v[p]
+        tables.append(table + [-1] * (7 - len(table)))
+        wants.append(plain.attention(q, k, v))
+        qs.append(q.reshape(sq, hq * dh))
+        seq += [b] * sq
+        pos += list(range(S - sq, S))
+    wide = torch.cat([torch.cat(qs), torch.randn(len(seq), 2 * hkv * dh)], dim=1).to(DEV)
+    out = _ops().attention_generic(wide, hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32(seq), _i32(pos), _i32(tables), 0, dh ** -0.5)
+    torch.testing.assert_close(out.cpu(), torch.cat(wants), rtol=1e-5, atol=1e-5)
+
+
+def test_attention_refuses_sizes_it_does_not_have():
+    from torchllms_amd.kernels.lib import KernelError
+
+    q = torch.zeros(1, 2 * 272, device=DEV)
+    pages = torch.zeros(2, 2, 4, 272, device=DEV)
+    with pytest.raises(KernelError, match="head_dim=272"):
+        _ops().attention_generic(q, 2, 2, 272, pages, pages, _i32([0]), _i32([0]), _i32([[0]]), 0, 1.0)
+    q = torch.zeros(1, 3 * 16, device=DEV)
+    pages = torch.zeros(2, 2, 4, 16, device=DEV)
+    with pytest.raises(KernelError, match="not a multiple"):
+        _ops().attention_generic(q, 3, 2, 16, pages, pages, _i32([0]), _i32([0]), _i32([[0]]), 0, 1.0)
+    with pytest.raises(KernelError, match="GPU"):
+        _ops().silu_mul(torch.zeros(2, 4))
+
+
+# ----------------------------------------------------------------------------- sampling
+def _sample(logits, temps, seeds, steps, top_k=None):
+    n = logits.shape[0]
+    return _ops().sample(
+        logits.to(DEV), torch.tensor(temps, dtype=torch.float32, device=DEV), torch.tensor(seeds, dtype=torch.int64, device=DEV),
+        torch.tensor(steps, dtype=torch.int64, device=DEV), None if top_k is None else _i32(top_k),
+    ).cpu()
+
+
+def test_sample_greedy_and_ties():
+    torch.manual_seed(0)
+    logits = torch.randn(5, 1003)
+    logits[2, 77] = logits[2, 900] = 9.0  # the lowest index among equal maxima
+    got = _sample(logits, [0.0] * 5, [1] * 5, [0] * 5)
+    assert got.tolist() == logits.argmax(-1).tolist() and got[2] == 77
+
+
+@pytest.mark.parametrize("vocab", [8, 301, 5000])
+def test_sample_temperature_matches_the_plain_rule(vocab):
+    torch.manual_seed(0)
+    logits = torch.randn(6, vocab) * 2
+    logits[5] = logits[0]
+    seeds, steps = [3, 3, 4, 5, 2 ** 40 + 7, 3], [0, 1, 0, 9, 2 ** 33, 0]
+    got = _sample(logits, [0.7] * 6, seeds, steps)
+    for r in range(6):
+        u = _ops().philox_uniform(seeds[r], steps[r], vocab, DEV).cpu()
+        assert (u > 0).all() and (u < 1).all()
+        want = plain.sample_with_exponentials(logits[r], 0.7, -torch.log(u))
+        assert got[r] == want
+    assert got[0] == got[5]  # same seed and step: same draw, whatever the row
+    # top-k: the draw comes from the k largest
+    got = _sample(logits, [1.5] * 6, seeds, steps, top_k=[3] * 6)
+    for r in range(6):
+        assert got[r] in logits[r].topk(3).indices.tolist()
+        u = _ops().philox_uniform(seeds[r], steps[r], vocab, DEV).cpu()
+        assert got[r] == plain.sample_with_exponentials(logits[r], 1.5, -torch.log(u), top_k=3)
+
+
+def test_sample_mixed_rows_and_tiny_temperature():
+    torch.manual_seed(0)
+    logits = torch.randn(4, 200)
+    got = _sample(logits, [0.0, 1e-7, 0.9, 0.0], [5, 6, 7, 8], [0, 0, 0, 0])
+    assert got[0] == logits[0].argmax() and got[1] == logits[1].argmax() and got[3] == logits[3].argmax()
+
+
+def test_sample_frequencies_follow_softmax():
+    logits = torch.tensor([1.0, 0.0, -1.0, 2.0, 0.5, -3.0])
+    n = 20000
+    got = _sample(logits.expand(n, 6).contiguous(), [0.7] * n, [123] * n, list(range(n)))
+    freq = torch.bincount(got.long(), minlength=6).float()
+    expect = torch.softmax(logits / 0.7, -1) * n
+    chi2 = ((freq - expect) ** 2 / expect).sum().item()
+    assert chi2 < 20.5  # 5 degrees of freedom, p = 0.001
+    u = _ops().philox_uniform(9, 0, 100000, DEV).cpu()
+    assert abs(u.mean().item() - 0.5) < 0.005 and abs(u.var().item() - 1 / 12) < 0.002

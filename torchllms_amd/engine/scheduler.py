@@ -1,0 +1,276 @@
+"""Continuous-batching scheduler: admits requests, cuts prompts into portions under a token
+budget, decodes, finishes and frees, and decides what happens when pages run out.
+
+The reference has no scheduler: it takes a list of prompts, sorts them by length, prefills each
+static batch in one forward and decodes in lock step until all rows are done
+(reference: torchllms/inference/llm.py:762-997, 1113-1141); when pages run out the request fails
+(torchllms/models/paged_kv.py:285-289).  What is kept from it are the rules of finishing: any-of
+stop ids with the stop token kept, the budget ``min(max_len - prompt_len, max_new_tokens)``, the
+last sampled token never fed back (llm.py:489-494, 568, 905-908).
+
+Every step is built in this order: one token for every request that is decoding; then further
+portions of prompts already started; then new requests from the waiting queue, while slots, pages
+and the token budget last.  Pages are counted before anything is committed.  When a decoding
+request cannot get the page it needs, the most recently admitted running request is preempted:
+its pages and slot are freed and it returns to the front of the waiting queue to be recomputed
+from its prompt plus everything it has generated so far.  Its sampling counter is the number of
+generated tokens, so its output is unchanged.  A request that could not fit into an empty pool
+is refused when it is added.
+
+The scheduler is plain host code; it touches the cache manager's bookkeeping only.
+"""
+
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, Hashable, List, Optional, Sequence
+
+from ..cache.manager import CacheManager
+from ..sampling.params import SamplingParams
+from .layout import StepEntry
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclass
+class Request:
+    rid: Hashable
+    prompt: List[int]
+    params: SamplingParams
+    budget: int  # tokens it may still generate in total
+    output: List[int] = field(default_factory=list)
+    state: str = WAITING
+    num_computed: int = 0  # of prompt + output, how many tokens are in the cache
+    stop_reason: Optional[int] = None  # the stop token id, or None when the budget ended it
+    preemptions: int = 0
+    arrival: int = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.output
+
+    @property
+    def remaining(self) -> int:
+        """Tokens not yet in the cache (the last generated token included)."""
+        return len(self.prompt) + len(self.output) - self.num_computed
+
+    @property
+    def finished(self) -> bool:
+        return self.state == FINISHED
+
+
+@dataclass
+class ScheduledEntry:
+    request: Request
+    tokens: List[int]
+    samples: bool  # the portion reaches the request's end: its last logits are sampled from
+
+
+@dataclass
+class StepPlan:
+    entries: List[ScheduledEntry] = field(default_factory=list)
+    preempted: List[Request] = field(default_factory=list)
+
+    @property
+    def n_tokens(self) -> int:
+        return sum(len(e.tokens) for e in self.entries)
+
+    def step_entries(self) -> List[StepEntry]:
+        return [StepEntry(e.request.rid, e.tokens, [len(e.tokens) - 1] if e.samples else []) for e in self.entries]
+
+
+class Scheduler:
+    def __init__(
+        self,
+        cache: CacheManager,
+        max_num_seqs: int,
+        max_num_batched_tokens: int,
+        max_model_len: int,
+        prefill_chunk: Optional[int] = None,
+    ):
+        if max_num_batched_tokens < 1 or max_num_seqs < 1:
+            raise ValueError("max_num_seqs and max_num_batched_tokens must be at least 1")
+        self.cache = cache
+        self.max_num_seqs = min(max_num_seqs, cache.max_seqs)
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.max_model_len = max_model_len
+        self.prefill_chunk = prefill_chunk or max_num_batched_tokens
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []  # in order of admission
+        self._arrivals = 0
+        self.stats = {"steps": 0, "tokens": 0, "preemptions": 0, "finished": 0}
+
+    # ------------------------------------------------------------------ intake
+    def add(self, rid: Hashable, prompt: Sequence[int], params: SamplingParams) -> Request:
+        """Queue a request.  Budget: ``min(max_model_len - len(prompt), max_new_tokens)``
+        (reference: llm.py:489-494); below 1 the request finishes at once with no tokens."""
+        prompt = [int(t) for t in prompt]
+        if not prompt:
+            raise ValueError(f"request {rid!r}: empty prompt")
+        budget = self.max_model_len - len(prompt)
+        if params.max_new_tokens is not None:
+            budget = min(budget, params.max_new_tokens)
+        req = Request(rid=rid, prompt=prompt, params=params, budget=max(budget, 0), arrival=self._arrivals)
+        self._arrivals += 1
+        if req.budget < 1:
+            req.state = FINISHED
+            return req
+        # the longest it can get: all but the last generated token sit in the cache
+        longest = len(prompt) + req.budget - 1
+        for pool in self.cache.pools:
+            if self.cache.blocks_for(longest) > pool.num_pages:
+                raise ValueError(
+                    f"request {rid!r}: {longest} tokens need {self.cache.blocks_for(longest)} pages, "
+                    f"the pool has {pool.num_pages}; it could never finish"
+                )
+        self.waiting.append(req)
+        return req
+
+    @property
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    # ------------------------------------------------------------------ planning
+    def _pages_for(self, req: Request, n_new: int) -> int:
+        if self.cache.has(req.rid):
+            return self.cache.new_pages_needed(req.rid, n_new)
+        return self.cache.blocks_for(n_new)
+
+    def _preempt(self, req: Request, plan: StepPlan) -> None:
+        self.cache.free(req.rid)
+        self.running.remove(req)
+        req.state = WAITING
+        req.num_computed = 0
+        req.preemptions += 1
+        self.stats["preemptions"] += 1
+        self.waiting.appendleft(req)
+        plan.preempted.append(req)
+
+    def schedule(self) -> StepPlan:
+        """Decide the next step.  Pages are counted here and taken by ``Engine.step``."""
+        plan = StepPlan()
+        budget = self.max_num_batched_tokens
+        free = [pool.free_count for pool in self.cache.pools]
+
+        def fits(pages: int) -> bool:
+            return all(f >= pages for f in free)
+
+        def take(pages: int) -> None:
+            for g in range(len(free)):
+                free[g] -= pages
+
+        # (1) one token for every decoding request, oldest first; make room by preempting the youngest
+        decoding = [r for r in self.running if r.remaining == 1]
+        i = 0
+        while i < len(decoding) and budget > 0:
+            req = decoding[i]
+            if req not in self.running:  # preempted a moment ago
+                i += 1
+                continue
+            pages = self._pages_for(req, 1)
+            while not fits(pages):
+                victim = self.running[-1]
+                was_planned = [e for e in plan.entries if e.request is victim]
+                for e in was_planned:  # give back what this step had counted for it
+                    plan.entries.remove(e)
+                    budget += len(e.tokens)
+                self._preempt(victim, plan)
+                counted = sum(self._pages_for(e.request, len(e.tokens)) for e in plan.entries)
+                for g in range(len(free)):
+                    free[g] = self.cache.pools[g].free_count - counted
+                if victim is req:
+                    break
+            if req in self.running:
+                plan.entries.append(ScheduledEntry(req, [req.tokens[-1]], samples=True))
+                take(pages)
+                budget -= 1
+            i += 1
+
+        # (2) prompts already started, in order of admission
+        for req in self.running:
+            if budget <= 0:
+                break
+            if req.remaining <= 1 or any(e.request is req for e in plan.entries):
+                continue
+            n = min(req.remaining, budget, self.prefill_chunk)
+            while n > 0 and not fits(self._pages_for(req, n)):
+                n = self._shrink(req, n, free)
+            if n <= 0:
+                continue
+            self._add_portion(plan, req, n)
+            take(self._pages_for(req, n))
+            budget -= n
+
+        # (3) new requests, first come first served; nothing overtakes the head of the queue
+        while self.waiting and budget > 0 and len(self.running) < self.max_num_seqs and self.cache.free_slots > 0:
+            req = self.waiting[0]
+            if req in plan.preempted:
+                break  # it lost its pages in this very step; it starts again in a later one
+            n = min(req.remaining, budget, self.prefill_chunk)
+            while n > 0 and not fits(self._pages_for(req, n)):
+                n = self._shrink(req, n, free)
+            if n <= 0:
+                break
+            self.waiting.popleft()
+            self.cache.admit(req.rid)
+            req.state = RUNNING
+            self.running.append(req)
+            self._add_portion(plan, req, n)
+            take(self._pages_for(req, n))
+            budget -= n
+
+        if not plan.entries and self.has_work:
+            raise RuntimeError(
+                "scheduler is stuck: work is queued but nothing fits (pool too small for the head of the queue?)"
+            )
+        return plan
+
+    def _shrink(self, req: Request, n: int, free: List[int]) -> int:
+        """The largest portion below ``n`` that the free pages hold (0: none)."""
+        have = max(min(free), 0) if free else 0
+        held = self.cache.num_tokens(req.rid) if self.cache.has(req.rid) else 0
+        room = (self.cache.blocks_for(held) + have) * self.cache.page_size - held
+        return max(min(n - 1, room), 0)
+
+    def _add_portion(self, plan: StepPlan, req: Request, n: int) -> None:
+        toks = req.tokens[req.num_computed : req.num_computed + n]
+        plan.entries.append(ScheduledEntry(req, toks, samples=(n == req.remaining)))
+
+    # ------------------------------------------------------------------ after the step
+    def update(self, plan: StepPlan, sampled: Sequence[int]) -> List[Request]:
+        """Book the step: ``sampled`` holds one token for every entry with ``samples``, in order.
+        Returns the requests that finished; their pages and slots are free again."""
+        done: List[Request] = []
+        it = iter(sampled)
+        for e in plan.entries:
+            req = e.request
+            req.num_computed += len(e.tokens)
+            if not e.samples:
+                continue
+            tok = int(next(it))
+            req.output.append(tok)
+            if tok in req.params.stop_token_ids:
+                req.stop_reason = tok
+                self._finish(req, done)
+            elif len(req.output) >= req.budget:
+                self._finish(req, done)
+        self.stats["steps"] += 1
+        self.stats["tokens"] += plan.n_tokens
+        return done
+
+    def _finish(self, req: Request, done: List[Request]) -> None:
+        req.state = FINISHED
+        self.running.remove(req)
+        self.cache.free(req.rid)
+        self.stats["finished"] += 1
+        done.append(req)
+
+    def abort(self, req: Request) -> None:
+        """Drop a request wherever it is; what it holds is given back."""
+        if req.state == RUNNING:
+            self.running.remove(req)
+            self.cache.free(req.rid)
+        elif req.state == WAITING and req in self.waiting:
+            self.waiting.remove(req)
+        req.state = FINISHED

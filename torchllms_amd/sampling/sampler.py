@@ -1,0 +1,40 @@
+"""Chooses next tokens from a step's logits with the sampling kernel."""
+
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from ..kernels import ops
+from .params import SamplingParams
+
+
+class Sampler:
+    """``sampler(logits, params, steps)`` -> one token id per row.
+
+    Row i is drawn with ``params[i]`` at generator counter ``steps[i]`` (the number of tokens the
+    request has generated so far), so the same request gives the same tokens whatever else is in
+    the batch and however often it was preempted.
+    """
+
+    def __call__(self, logits: torch.Tensor, params: Sequence[SamplingParams], steps: Sequence[int]) -> List[int]:
+        n = logits.shape[0]
+        if n == 0:
+            return []
+        if len(params) != n or len(steps) != n:
+            raise ValueError("one SamplingParams and one step counter per logits row")
+        dev = logits.device
+        temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32, device=dev)
+        seeds = torch.tensor([_as_i64(p.seed) for p in params], dtype=torch.int64, device=dev)
+        counters = torch.tensor([int(s) for s in steps], dtype=torch.int64, device=dev)
+        top_k = None
+        if any(p.top_k for p in params):
+            top_k = torch.tensor([p.top_k or 0 for p in params], dtype=torch.int32, device=dev)
+        return ops.sample(logits, temperature, seeds, counters, top_k).tolist()
+
+
+def _as_i64(x: int) -> int:
+    """A seed of up to 64 bits as the signed integer with the same bits."""
+    x &= (1 << 64) - 1
+    return x - (1 << 64) if x >= (1 << 63) else x
