@@ -1,0 +1,239 @@
+"""Decode and prefill throughput of the engine on one MI355X, Llama-3.1-8B layer sizes, random
+bfloat16 weights, synthetic token ids.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
+
+A step is one decode step of the whole batch: ``Engine.step`` on one token per request followed by
+the sampling kernel and the copy of the chosen tokens to the host, as generation does it.  The
+requests' earlier context is not computed: their pages are filled with random keys and values,
+which costs a decode step the same reads.  One JSON line is printed: ``value`` is decoded tokens a
+second at the default batch; ``prefill`` times one 2,048-token prompt; ``roofline`` sets the decode
+step's unavoidable reads (every weight once, the live requests' cache) against HBM's 8 TB/s;
+``points`` holds decode at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_GBS = 8000.0  # MI355X HBM3E, published
+PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # dense MFMA, published
+
+# BASELINE.json configs[2]: Llama-3.1-8B shape
+LLAMA_8B = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=4096, num_hidden_layers=32, num_attention_heads=32,
+    num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=128256, rms_norm_eps=1e-5,
+    rope_theta=500000.0, max_position_embeddings=131072, tie_word_embeddings=False,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+)
+
+
+def parse_args(argv=None):
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=32)
+    p.add_argument("--warmup", type=int, default=4)
+    p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--context", type=int, default=8192)
+    p.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (both numbers are reported)")
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    p.add_argument("--prefill-tokens", type=int, default=2048)
+    p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
+    p.add_argument("--page-size", type=int, default=16)
+    return p.parse_args(argv)
+
+
+def weight_bytes(engine) -> int:
+    """Bytes of every tensor a decode step reads once: all layers, final norm, output matrix; of the
+    embedding table only the rows of the batch (counted by the caller)."""
+    total = 0
+    seen = set()
+    m = engine.model
+
+    def add(t):
+        if t is not None and t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            nonlocal total
+            total += t.numel() * t.element_size()
+
+    for b in m.blocks:
+        for part in (b.mixer, b.feed_forward, b.mixer_norm, b.ffn_norm):
+            for v in vars(part).values():
+                if hasattr(v, "data_ptr"):
+                    add(v)
+    add(m.final_norm.weight)
+    add(m.head.weight)
+    return total
+
+
+def fill_context(engine, rids, n_tokens, seed=0):
+    """Give every request ``n_tokens`` cached tokens without computing them: pages are claimed and
+    filled with random keys and values."""
+    import torch
+
+    for rid in rids:
+        engine.admit(rid)
+        engine.cache.extend(rid, n_tokens)
+        engine.cache.advance(rid, n_tokens)
+    g = torch.Generator(device=engine.device).manual_seed(seed)
+    for pages in list(engine.cache.k_pages) + list(engine.cache.v_pages):
+        flat = pages.view(-1)
+        chunk = 1 << 28
+        for lo in range(0, flat.numel(), chunk):
+            flat[lo : lo + chunk].normal_(0.0, 1.0, generator=g)
+
+
+def decode_run(engine, sampler, batch, context, steps, warmup, vocab):
+    """Time ``steps`` decode steps of ``batch`` requests whose context ends at ``context`` tokens."""
+    import torch
+
+    from torchllms_amd.engine import StepEntry
+    from torchllms_amd.sampling import SamplingParams
+
+    rids = [f"d{i}" for i in range(batch)]
+    start = context - (steps + warmup) - 1
+    fill_context(engine, rids, start)
+    params = [SamplingParams(temperature=0.0, seed=i) for i in range(batch)]
+    tokens = [(7 * i + 3) % vocab for i in range(batch)]
+
+    def one_step(k):
+        nonlocal tokens
+        logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(rids, tokens)])
+        tokens = sampler(logits, params, [k] * batch)
+
+    for k in range(warmup):
+        one_step(k)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        one_step(warmup + k)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    mean_ctx = start + warmup + (steps + 1) / 2
+    for r in rids:
+        engine.free(r)
+    return dt / steps, mean_ctx
+
+
+def prefill_run(engine, n_tokens, vocab, repeats=3):
+    import torch
+
+    from torchllms_amd.engine import StepEntry
+
+    toks = torch.randint(0, vocab, (n_tokens,), generator=torch.Generator().manual_seed(1)).tolist()
+    times = []
+    for i in range(repeats + 1):
+        engine.admit("p")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([StepEntry("p", toks, [n_tokens - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.free("p")
+    times = sorted(times[1:])  # the first run warms up
+    return times[len(times) // 2]
+
+
+def prefill_flops(cfg, n_layers, T):
+    """Multiply-adds x 2 of one prompt of T tokens: projections, causal attention (half the square),
+    feed-forward, and the output matrix for the one wanted row."""
+    D, Hq, Hkv, dh, F, V = cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.intermediate_size, cfg.vocab_size
+    per_token = 2 * D * (Hq + 2 * Hkv) * dh + 2 * Hq * dh * D + 3 * 2 * D * F
+    attn = 2 * 2 * Hq * dh * (T * (T + 1) / 2)
+    return n_layers * (T * per_token + attn) + 2 * D * V
+
+
+def main(argv=None) -> int:
+    args = parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
+        return 2
+    import torch
+
+    from torchllms_amd.cache.manager import CacheManager
+    from torchllms_amd.config import LlamaConfig
+    from torchllms_amd.engine import Engine
+    from torchllms_amd.sampling import Sampler
+
+    full_layers = LLAMA_8B["num_hidden_layers"]
+    n_layers = args.layers or full_layers
+    cfg = LlamaConfig.from_dict(dict(LLAMA_8B, num_hidden_layers=n_layers))
+    batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
+    max_batch = max(batches)
+    pages_per_req = -(-args.context // args.page_size) + 1
+    engine = Engine.from_random(
+        cfg, seed=0, dtype=args.dtype, draw_on_device=True, page_size=args.page_size,
+        num_pages=max_batch * pages_per_req, max_seqs=max_batch, max_model_len=args.context,
+    )
+    sampler = Sampler()
+    elt = 2 if args.dtype == "bfloat16" else 4
+    wbytes = weight_bytes(engine)
+    kv_per_token = 2 * n_layers * cfg.num_key_value_heads * cfg.head_dim * elt
+
+    results = {}
+    for b in batches:
+        steps = args.steps if b == args.batch else max(args.steps // 2, 4)
+        sec, mean_ctx = decode_run(engine, sampler, b, args.context, steps, args.warmup, cfg.vocab_size)
+        step_bytes = wbytes + b * cfg.hidden_size * elt + b * mean_ctx * kv_per_token
+        results[b] = dict(sec=sec, tps=b / sec, bytes=step_bytes)
+
+    pre_sec = prefill_run(engine, args.prefill_tokens, cfg.vocab_size)
+    flops = prefill_flops(cfg, n_layers, args.prefill_tokens)
+
+    main_r = results[args.batch]
+    achieved = main_r["bytes"] / main_r["sec"] / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8, Llama-3.1-8B shape (plus batch 1/64 and prefill tok/s at 2048 tokens)",
+        "value": round(main_r["tps"], 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_r["sec"] * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: random-init weights, random token ids, cache of earlier context filled with random values",
+        "config": {
+            "model": "Llama-3.1-8B shape",
+            "global_batch": args.batch,
+            "seq_len": args.context,
+            "parallelism": "single GPU",
+            "n_layers": n_layers,
+            "n_layers_full": full_layers,
+            "hidden_size": cfg.hidden_size,
+            "n_heads": cfg.num_attention_heads,
+            "n_kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim,
+            "intermediate_size": cfg.intermediate_size,
+            "vocab_size": cfg.vocab_size,
+            "page_size": args.page_size,
+            "prefill_tokens": args.prefill_tokens,
+            "rope": "llama3 factor 8 theta 5e5",
+        },
+        "prefill": {
+            "value": round(args.prefill_tokens / pre_sec, 1),
+            "tokens": args.prefill_tokens,
+            "ms": round(pre_sec * 1e3, 3),
+            "frac": round(flops / pre_sec / (PEAK_TFLOPS[args.dtype] * 1e12), 4),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_GBS, 4),
+        },
+        "points": {f"decode_b{b}": round(r["tps"], 2) for b, r in results.items() if b != args.batch},
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,123 @@
+"""Generation through the Python entry point and the command line, on the GPU."""
+
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+from .helpers import TINY, make_folder, random_tokens, read_folder
+from .plain import llama as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
+
+
+@pytest.fixture(scope="module")
+def model_b(tmp_path_factory):
+    folder = make_folder(tmp_path_factory.mktemp("gen") / "B", TINY["B"], seed=5, dtype=torch.bfloat16, sharpen=True)
+    cfg, weights = read_folder(folder)
+    return folder, cfg, weights
+
+
+def plain_greedy(weights, cfg, prompt, n, stop=()):
+    toks = list(prompt)
+    for _ in range(n):
+        nxt = int(plain.forward(weights, cfg, toks, torch.float32)[-1].argmax())
+        toks.append(nxt)
+        if nxt in stop:
+            break
+    return toks[len(prompt):]
+
+
+def test_greedy_generation_matches_the_plain_model(model_b):
+    from torchllms_amd.inference import LLM
+
+    folder, cfg, weights = model_b
+    prompts = [random_tokens(n, cfg["vocab_size"], 40 + n) for n in (5, 17, 1, 32)]
+    llm = LLM(str(folder), precision="float32", max_len=128, max_bsz=3, page_size=8)
+    results = llm.generate(prompt_token_ids=prompts, temperature=0.0, max_new_tokens=12)
+    for p, r in zip(prompts, results):
+        assert r.token_ids == plain_greedy(weights, cfg, p, 12) and r.stop_reason is None and r.text == ""
+    # a stop token ends the request and is kept
+    want = plain_greedy(weights, cfg, prompts[1], 12)
+    stop = want[4]
+    r = llm.generate(prompt_token_ids=[prompts[1]], max_new_tokens=12, stop_token_ids=[stop])[0]
+    cut = want.index(stop) + 1
+    assert r.token_ids == want[:cut] and r.stop_reason == stop
+    llm.engine.cache.check_invariants()
+    assert llm.engine.cache.live == []
+
+
+def test_bfloat16_greedy_picks_tokens_the_plain_model_rates_highest(model_b):
+    from torchllms_amd.inference import LLM
+
+    folder, cfg, weights = model_b
+    prompt = random_tokens(20, cfg["vocab_size"], 77)
+    llm = LLM(str(folder), precision="bfloat16", max_len=128, max_bsz=2)
+    got = llm.generate(prompt_token_ids=[prompt], max_new_tokens=16)[0].token_ids
+    assert len(got) == 16
+    toks = prompt + got
+    logits32 = plain.forward(weights, cfg, toks, torch.float32)
+    logits16 = plain.forward(weights, cfg, toks, torch.bfloat16).float()
+    slack = 2 * (logits16 - logits32).abs().max().item()
+    for i, tok in enumerate(got):
+        row = logits32[len(prompt) - 1 + i]
+        assert row[tok] >= row.max() - slack, f"token {i}: chose {tok}, plain model prefers {int(row.argmax())}"
+
+
+def test_seeded_sampling_does_not_depend_on_batch_mates(model_b):
+    from torchllms_amd.inference import LLM
+
+    folder, cfg, _ = model_b
+    prompts = [random_tokens(n, cfg["vocab_size"], 60 + n) for n in (1, 9, 40, 100)]
+    llm = LLM(str(folder), precision="float32", max_len=160, max_bsz=4, max_num_batched_tokens=24)
+    together = llm.generate(prompt_token_ids=prompts, temperature=0.7, max_new_tokens=24, seed=1234)
+    assert llm.last_stats["steps"] > 24  # prompts were fed in 24-token portions beside decoding
+    for i, p in enumerate(prompts):
+        alone = llm.generate(prompt_token_ids=[p], temperature=0.7, max_new_tokens=24, seed=1234 + i)[0]
+        assert alone.token_ids == together[i].token_ids
+    other = llm.generate(prompt_token_ids=prompts, temperature=0.7, max_new_tokens=24, seed=99)
+    assert [r.token_ids for r in other] != [r.token_ids for r in together]
+    greedy = llm.generate(prompt_token_ids=prompts, temperature=0.0, max_new_tokens=24)
+    assert [r.token_ids for r in greedy] != [r.token_ids for r in together]
+
+
+def test_preemption_on_the_gpu_changes_nothing(model_b):
+    from torchllms_amd.inference import LLM
+
+    folder, cfg, _ = model_b
+    prompts = [random_tokens(n, cfg["vocab_size"], 80 + n) for n in (30, 25, 28, 21)]
+    ample = LLM(str(folder), precision="float32", max_len=96, max_bsz=4, page_size=8)
+    want = ample.generate(prompt_token_ids=prompts, temperature=0.8, max_new_tokens=30, seed=7)
+    tight = LLM(str(folder), precision="float32", max_len=96, max_bsz=4, page_size=8, num_pages=20)  # 160 places for 224 tokens
+    got = tight.generate(prompt_token_ids=prompts, temperature=0.8, max_new_tokens=30, seed=7)
+    assert tight.last_stats["preemptions"] > 0
+    assert [r.token_ids for r in got] == [r.token_ids for r in want]
+    tight.engine.cache.check_invariants()
+
+
+def test_generate_command_line(model_b, tmp_path):
+    folder, cfg, weights = model_b
+    prompts = [random_tokens(n, cfg["vocab_size"], 90 + n) for n in (4, 11)]
+    inp, out = tmp_path / "in.jsonl", tmp_path / "sub" / "out.jsonl"
+    inp.write_text("".join(json.dumps({"prompt_token_ids": p, "tag": i}) + "\n" for i, p in enumerate(prompts)))
+    cmd = [
+        sys.executable, "-m", "torchllms_amd.inference.generate", "--input_path", str(inp), "--output_path", str(out),
+        "--provider_kwargs", json.dumps({"ckpt_paths": str(folder), "precision": "float32", "max_len": 64}),
+        "--generate_kwargs", json.dumps({"max_new_tokens": 5}),
+    ]
+    subprocess.run(cmd, check=True, cwd=ROOT, timeout=300)
+    recs = [json.loads(l) for l in out.read_text().splitlines()]
+    assert [r["tag"] for r in recs] == [0, 1]
+    for p, r in zip(prompts, recs):
+        assert r["completion_token_ids"] == plain_greedy(weights, cfg, p, 5)
+
+
+def test_smoke_entry():
+    sys.path.insert(0, str(ROOT))
+    import __graft_entry__
+
+    __graft_entry__.smoke()

@@ -1,0 +1,167 @@
+"""A toy architecture defined here, in the test: a mixer with state of its own beside attention
+layers (one of them windowed), an execution order that runs a layer twice and lets a run read
+another run's cache.  It is registered, built from random weights and stepped through the engine
+in portions and mixed batches without any change to the framework's files, and compared with a
+plain whole-sequence computation written here."""
+
+from dataclasses import dataclass
+from typing import Dict, Tuple
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from . import schedules
+from .helpers import random_tokens
+from .plain import llama as plain
+from .test_gpu_engine import run_trace
+
+pytestmark = pytest.mark.gpu
+
+HIDDEN, STATE, VOCAB, HEADS, KV, DH, FFN, WINDOW = 40, 24, 97, 4, 2, 16, 56, 6
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    decay: float = 0.8
+    architectures: Tuple[str, ...] = ("ToyHybridForCausalLM",)
+
+
+def _register():
+    from torchllms_amd.config import ArchSpec, register_architecture
+    from torchllms_amd.config.spec import LayerRun, LayerSpec, ModelSpec, PartSpec
+    from torchllms_amd.parts import MIXERS, Mixer, ParamSpec, StateNeed
+    from torchllms_amd.weights import NameRule
+
+    if "toy_decay" not in MIXERS:
+
+        @MIXERS.register("toy_decay")
+        class DecayMixer(Mixer):
+            """s_t = decay * s_{t-1} + W_in x_t ;  y_t = W_out s_t.  The state s lives in the
+            request's slot, so it carries over from one step to the next."""
+
+            def __init__(self, hidden_size, state_size, decay):
+                self.hidden_size, self.state_size, self.decay = hidden_size, state_size, decay
+
+            def param_specs(self):
+                return {"w_in.weight": ParamSpec((self.state_size, self.hidden_size)),
+                        "w_out.weight": ParamSpec((self.hidden_size, self.state_size))}
+
+            def cache_need(self):
+                return StateNeed(shape=(self.state_size,), dtype="float32")
+
+            def bind(self, tensors):
+                self.w_in, self.w_out = tensors["w_in.weight"], tensors["w_out.weight"]
+
+            def forward(self, x, ctx, cache):
+                u = F.linear(x.float(), self.w_in.float())
+                states = torch.empty_like(u)
+                lay = ctx.host
+                for row in range(lay.n_seqs):
+                    s = cache.tensor[int(lay.slot_ids[row])]
+                    for t in range(int(lay.qo_indptr[row]), int(lay.qo_indptr[row + 1])):
+                        s.mul_(self.decay).add_(u[t])
+                        states[t] = s
+                return F.linear(states, self.w_out.float()).to(x.dtype)
+
+    def spec(cfg: ToyConfig) -> ModelSpec:
+        rope = PartSpec("rope", dict(head_dim=DH, rotary_dim=DH, theta=100.0, scaling=None))
+        norm = PartSpec("rmsnorm", dict(size=HIDDEN, eps=1e-5))
+        ffn = PartSpec("swiglu", dict(hidden_size=HIDDEN, intermediate_size=FFN))
+
+        def attn(window):
+            return PartSpec("attention", dict(hidden_size=HIDDEN, num_heads=HEADS, num_kv_heads=KV, head_dim=DH, qkv_bias=False,
+                                              softmax_scale=DH ** -0.5, window=window, position=rope))
+
+        mixers = [attn(0), PartSpec("toy_decay", dict(hidden_size=HIDDEN, state_size=STATE, decay=cfg.decay)), attn(WINDOW)]
+        layers = [LayerSpec(f"layers.{i}", "pre_norm", m, ffn, norm, norm) for i, m in enumerate(mixers)]
+        order = [LayerRun(0), LayerRun(1), LayerRun(2), LayerRun(1), LayerRun(0, cache_from=0)]
+        return ModelSpec("ToyHybridForCausalLM", HIDDEN, VOCAB, 512, PartSpec("embedding", dict(vocab_size=VOCAB, hidden_size=HIDDEN)),
+                         layers, order, norm, PartSpec("lm_head", dict(vocab_size=VOCAB, hidden_size=HIDDEN, tied=True)))
+
+    def rules(cfg):
+        names = ["embed.weight", "final_norm.weight"]
+        per_layer = ["mixer_norm.weight", "ffn_norm.weight", "ffn.w1.weight", "ffn.w2.weight", "ffn.w3.weight",
+                     "mixer.wq.weight", "mixer.wk.weight", "mixer.wv.weight", "mixer.wo.weight",
+                     "mixer.w_in.weight", "mixer.w_out.weight"]
+        return [NameRule(n, n) for n in names] + [NameRule("layers.{}." + n, "layers.{}." + n) for n in per_layer]
+
+    return register_architecture(ArchSpec("ToyHybridForCausalLM", lambda d: ToyConfig(**d), spec, rules))
+
+
+def plain_toy(w: Dict[str, torch.Tensor], cfg: ToyConfig, tokens):
+    """The same model over a whole sequence, no cache, no engine."""
+    S = len(tokens)
+    pos = torch.arange(S)
+    f = plain.rope_inverse_frequencies(DH, 100.0, None)
+    h = w["embed.weight"][torch.tensor(tokens)]
+    kept = {}
+
+    def attn(run, layer, x, window, borrow=None):
+        p = f"layers.{layer}.mixer."
+        q = plain.rope_rotate_interleaved(F.linear(x, w[p + "wq.weight"]).view(S, HEADS, DH), pos, f)
+        if borrow is None:
+            k = plain.rope_rotate_interleaved(F.linear(x, w[p + "wk.weight"]).view(S, KV, DH), pos, f)
+            v = F.linear(x, w[p + "wv.weight"]).view(S, KV, DH)
+            kept[run] = (k, v)
+        else:
+            k, v = kept[borrow]
+        rows = []
+        for i in range(S):
+            lo = max(i - window + 1, 0) if window else 0
+            rows.append(plain.attention(q[i : i + 1], k[lo : i + 1], v[lo : i + 1]))
+        return F.linear(torch.cat(rows), w[p + "wo.weight"])
+
+    def decay(layer, x):
+        p = f"layers.{layer}.mixer."
+        u = F.linear(x, w[p + "w_in.weight"])
+        s = torch.zeros(STATE)
+        out = []
+        for t in range(S):
+            s = cfg.decay * s + u[t]
+            out.append(s)
+        return F.linear(torch.stack(out), w[p + "w_out.weight"])
+
+    runs = [(0, None), (1, None), (2, None), (1, None), (0, 0)]
+    for run, (layer, borrow) in enumerate(runs):
+        p = f"layers.{layer}."
+        x = plain.rms_norm(h, w[p + "mixer_norm.weight"], 1e-5)
+        h = h + (decay(layer, x) if layer == 1 else attn(run, layer, x, WINDOW if layer == 2 else 0, borrow))
+        h = h + plain.swiglu(plain.rms_norm(h, w[p + "ffn_norm.weight"], 1e-5), w[p + "ffn.w1.weight"], w[p + "ffn.w3.weight"], w[p + "ffn.w2.weight"])
+    return F.linear(plain.rms_norm(h, w["final_norm.weight"], 1e-5), w["embed.weight"])
+
+
+def test_toy_architecture_is_registered_built_and_stepped():
+    from torchllms_amd.engine import Engine
+    from torchllms_amd.parts import Model
+    from torchllms_amd.weights import random_tensors
+
+    arch = _register()
+    cfg = ToyConfig()
+    expected = Model(arch.model_spec(cfg)).param_specs()
+    w = random_tensors(expected, seed=3, dtype=torch.float32, norm_jitter=0.1)
+    for name in w:  # sharper attention and a livelier state than N(0, 0.02) gives
+        if name.endswith(("wq.weight", "wk.weight")):
+            w[name] = w[name] * 15
+        if name.endswith(("w_in.weight", "w_out.weight")):
+            w[name] = w[name] * 8
+    requests = {f"t{i}": random_tokens(n, VOCAB, 500 + i) for i, n in enumerate([40, 70, 33, 55])}
+    traces = {"whole": schedules.whole(requests), "portions": schedules.portions(requests), "mixed": schedules.mixed(requests)}
+    pool_tokens = max(schedules.max_live_tokens(t) for t in traces.values())
+    eng = Engine(arch, cfg, {k: v.to("cuda:0") for k, v in w.items()}, torch.float32, page_size=4,
+                 num_pages=-(-pool_tokens // 4), max_seqs=4, max_model_len=512)
+    # groups: full attention (runs 0 and the borrower's source), windowed attention, and state slots for two runs
+    assert sorted((g.window, g.run_ids) for g in eng.cache.groups) == [(0, (0,)), (WINDOW, (2,))]
+    assert [(s.run_ids, s.shape) for s in eng.cache.states] == [((1, 3), (STATE,))]
+    truth = {rid: plain_toy(w, cfg, t) for rid, t in requests.items()}
+    for name, steps in traces.items():
+        got = run_trace(eng, steps)
+        for (rid, pos), row in got.items():
+            assert (row - truth[rid][pos]).abs().max().item() < 5e-5, f"{name}: {rid} position {pos}"
+    # the windowed group gave pages back while requests were still running
+    eng.admit("w")
+    from torchllms_amd.engine import StepEntry
+
+    eng.step([StepEntry("w", random_tokens(30, VOCAB, 9))])
+    assert sum(p >= 0 for p in eng.cache.block_table("w", 1)) <= 3 < sum(p >= 0 for p in eng.cache.block_table("w", 0))
+    eng.free("w")

@@ -1,0 +1,208 @@
+"""The scheduler's decisions and the generation loop, on the CPU with a fake engine.
+
+The fake engine keeps the real cache manager's books and answers, for a token at position p, with
+logits whose argmax is (p + 1) % VOCAB, as the reference's own fake model does.  Vectors marked
+(ref) restate reference: torchllms/inference/test_prefix_cache_wiring.py:257-555.
+"""
+
+import random
+
+import pytest
+import torch
+
+from torchllms_amd.cache import CacheGroupSpec, CacheManager
+from torchllms_amd.engine.scheduler import Scheduler
+from torchllms_amd.inference.llm import GenerationLoop
+from torchllms_amd.sampling import SamplingParams
+
+VOCAB = 32
+
+
+class FakeEngine:
+    def __init__(self, num_pages=64, page_size=4, max_seqs=4, window=0):
+        self.cache = CacheManager([CacheGroupSpec("kv0", (0,), 1, 4, window)], [], page_size, num_pages, max_seqs)
+        self.calls = []  # per step: list of (rid, first position, n tokens)
+
+    def step(self, entries):
+        need = sum(self.cache.new_pages_needed(e.rid, len(e.tokens)) for e in entries)
+        assert need <= self.cache.free_pages(), "the scheduler planned a step the pool cannot hold"
+        rows, call = [], []
+        for e in entries:
+            start = self.cache.extend(e.rid, len(e.tokens))
+            call.append((e.rid, start, len(e.tokens)))
+            for w in e.want:
+                row = torch.zeros(VOCAB)
+                row[(start + w + 1) % VOCAB] = 1.0
+                rows.append(row)
+        for e in entries:
+            self.cache.advance(e.rid, len(e.tokens))
+        self.cache.check_invariants()
+        self.calls.append(call)
+        return torch.stack(rows) if rows else torch.zeros(0, VOCAB)
+
+
+def greedy(logits, params, steps):
+    return logits.argmax(-1).tolist() if len(params) else []
+
+
+def generate(prompts, max_new_tokens=None, stop=(), engine=None, max_num_seqs=4, budget=64, max_model_len=256, chunk=None):
+    engine = engine or FakeEngine()
+    loop = GenerationLoop(engine, greedy, max_num_seqs, budget, max_model_len, chunk)
+    params = [SamplingParams(max_new_tokens=max_new_tokens, stop_token_ids=stop) for _ in prompts]
+    reqs = loop.run(prompts, params)
+    assert engine.cache.live == [] and engine.cache.free_pages() == engine.cache.pools[0].num_pages
+    return reqs, engine, loop
+
+
+def test_single_request_token_stream_and_call_count():  # (ref)
+    reqs, eng, _ = generate([[5, 6, 7, 8, 9]], max_new_tokens=6)
+    assert reqs[0].output == [5, 6, 7, 8, 9, 10] and reqs[0].stop_reason is None
+    assert len(eng.calls) == 6 and eng.calls[0][0][2] == 5 and all(c[0][2] == 1 for c in eng.calls[1:])
+
+
+def test_zero_budget_runs_nothing():  # (ref)
+    reqs, eng, _ = generate([[5, 6, 7]], max_new_tokens=0)
+    assert reqs[0].output == [] and reqs[0].stop_reason is None and eng.calls == []
+
+
+def test_stop_ids_are_alternatives_and_the_stop_token_is_kept():  # (ref)
+    reqs, _, _ = generate([[5, 6, 7, 8, 9]], max_new_tokens=10, stop=(7, 6))
+    assert reqs[0].output == [5, 6] and reqs[0].stop_reason == 6
+    reqs, eng, _ = generate([[5, 6, 7, 8, 9]], max_new_tokens=10, stop=(5,))
+    assert reqs[0].output == [5] and reqs[0].stop_reason == 5 and len(eng.calls) == 1
+    reqs, _, _ = generate([[5, 6, 7, 8, 9]], max_new_tokens=4, stop=(99,))
+    assert reqs[0].stop_reason is None and len(reqs[0].output) == 4
+    reqs, _, _ = generate([[5, 6, 7, 8, 9]], max_new_tokens=10, stop=(8, 6))
+    assert reqs[0].output == [5, 6] and reqs[0].stop_reason == 6
+
+
+def test_batched_equals_single_per_row_and_order_is_kept():  # (ref: lengths 3, 6, 2)
+    prompts = [[1, 2, 3], [1, 2, 3, 4, 5, 6], [7, 8]]
+    together, _, _ = generate(prompts, max_new_tokens=5)
+    for p, r in zip(prompts, together):
+        alone, _, _ = generate([p], max_new_tokens=5)
+        assert r.output == alone[0].output == [(len(p) + i) % VOCAB for i in range(5)]
+    # rows that finish at different times, one with no budget at all
+    loop_reqs, _, _ = generate(prompts, max_new_tokens=None, max_model_len=7)
+    assert [len(r.output) for r in loop_reqs] == [4, 1, 5]
+
+
+def test_context_length_bounds_the_budget():
+    reqs, _, _ = generate([[1] * 10], max_new_tokens=100, max_model_len=13)
+    assert len(reqs[0].output) == 3
+    reqs, eng, _ = generate([[1] * 13], max_new_tokens=100, max_model_len=13)
+    assert reqs[0].output == [] and eng.calls == []
+
+
+def test_empty_prompt_and_impossible_requests_are_refused():
+    eng = FakeEngine(num_pages=4, page_size=4)
+    s = Scheduler(eng.cache, 4, 64, 256)
+    with pytest.raises(ValueError, match="empty prompt"):
+        s.add("a", [], SamplingParams(max_new_tokens=3))
+    with pytest.raises(ValueError, match="could never finish"):
+        s.add("b", [1] * 10, SamplingParams(max_new_tokens=8))  # 17 tokens in the cache > 16 places
+    s.add("c", [1] * 10, SamplingParams(max_new_tokens=7))  # 16 tokens: fits exactly
+
+
+def test_token_budget_and_order_inside_a_step():
+    eng = FakeEngine(num_pages=64, page_size=4, max_seqs=4)
+    loop = GenerationLoop(eng, greedy, 4, 8, 256)
+    seen = []
+    prompts = [[1] * 3, [1] * 19, [1] * 6, [1] * 2]
+    loop.run(prompts, [SamplingParams(max_new_tokens=6) for _ in prompts], on_step=lambda plan: seen.append(plan))
+    assert all(p.n_tokens <= 8 for p in seen)
+    # the 19-token prompt was cut into portions; a portion may be as small as the budget leaves
+    portions = [n for call in eng.calls for rid, start, n in call if rid[2] == 1 and start < 19]
+    assert sum(portions) == 19 and max(portions) <= 8 and len(portions) >= 3
+    for p in seen:
+        kinds = [len(e.tokens) == 1 and e.samples and len(e.request.output) > 0 for e in p.entries]
+        # decoding requests come first, then portions of prompts
+        assert kinds == sorted(kinds, reverse=True)
+    mixed = [p for p in seen if any(len(e.tokens) > 1 for e in p.entries) and any(len(e.tokens) == 1 for e in p.entries)]
+    assert mixed, "no step held a portion of a prompt beside a decoded token"
+
+
+def test_prefill_chunk_limits_a_portion():
+    reqs, eng, _ = generate([[1] * 23], max_new_tokens=2, budget=64, chunk=5)
+    sizes = [c[0][2] for c in eng.calls]
+    assert sizes == [5, 5, 5, 5, 3, 1]
+    assert reqs[0].output == [23, 24]
+
+
+def test_requests_queue_for_slots():
+    prompts = [[1] * (2 + i) for i in range(9)]
+    reqs, eng, loop = generate(prompts, max_new_tokens=4, max_num_seqs=2)
+    assert all(len(c) <= 2 for c in eng.calls)
+    assert [r.output for r in reqs] == [[(2 + i + k) % VOCAB for k in range(4)] for i in range(9)]
+    assert loop.scheduler.stats["finished"] == 9
+
+
+def test_preemption_gives_the_same_tokens_as_an_ample_pool():
+    prompts = [[1] * 9, [1] * 7, [1] * 11, [1] * 5]
+    ample, _, _ = generate(prompts, max_new_tokens=14)
+    tight_engine = FakeEngine(num_pages=12, page_size=4, max_seqs=4)  # 48 places for 32 + 4 * 13 tokens
+    tight, _, loop = generate(prompts, max_new_tokens=14, engine=tight_engine)
+    assert loop.scheduler.stats["preemptions"] > 0
+    assert [r.output for r in tight] == [r.output for r in ample]
+    assert any(r.preemptions for r in tight)
+    # the oldest request is never the victim
+    assert tight[0].preemptions == 0
+
+
+def test_a_lone_request_that_outgrows_the_pool_is_caught_at_add():
+    eng = FakeEngine(num_pages=3, page_size=4)
+    loop = GenerationLoop(eng, greedy, 4, 64, 256)
+    with pytest.raises(ValueError, match="could never finish"):
+        loop.run([[1] * 8], [SamplingParams(max_new_tokens=10)])
+    assert eng.cache.live == []
+
+
+def test_failure_gives_everything_back():
+    eng = FakeEngine()
+
+    def broken(logits, params, steps):
+        if len(eng.calls) >= 3:
+            raise RuntimeError("sampler died")
+        return greedy(logits, params, steps)
+
+    loop = GenerationLoop(eng, broken, 4, 64, 256)
+    with pytest.raises(RuntimeError, match="sampler died"):
+        loop.run([[1, 2, 3], [4, 5]], [SamplingParams(max_new_tokens=9)] * 2)
+    assert eng.cache.live == [] and eng.cache.free_pages() == 64
+    eng.cache.check_invariants()
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_workloads_finish_with_right_tokens(seed):
+    rng = random.Random(seed)
+    n = rng.randint(3, 12)
+    prompts = [[1] * rng.randint(1, 30) for _ in range(n)]
+    news = [rng.randint(1, 20) for _ in range(n)]
+    page = rng.choice([2, 4, 8])
+    longest = max(len(p) + m for p, m in zip(prompts, news))
+    eng = FakeEngine(num_pages=-(-longest // page) + rng.randint(0, 6), page_size=page, max_seqs=rng.randint(1, 4))
+    loop = GenerationLoop(eng, greedy, rng.randint(1, 4), rng.choice([1, 2, 5, 16, 64]), 256, rng.choice([None, 3, 7]))
+    params = [SamplingParams(max_new_tokens=m) for m in news]
+    reqs = loop.run(prompts, params)
+    for p, m, r in zip(prompts, news, reqs):
+        assert r.output == [(len(p) + k) % VOCAB for k in range(m)]
+    assert eng.cache.live == []
+    eng.cache.check_invariants()
+
+
+def test_sampling_counter_survives_preemption():
+    """The sampler sees (seed, number of tokens generated so far): recomputation after a preemption
+    asks for the same draws again."""
+    asked = []
+
+    def recording(logits, params, steps):
+        asked.extend((p.seed, s) for p, s in zip(params, steps))
+        return greedy(logits, params, steps)
+
+    eng = FakeEngine(num_pages=6, page_size=4, max_seqs=2)
+    loop = GenerationLoop(eng, recording, 2, 64, 256)
+    loop.run([[1] * 6, [1] * 6], [SamplingParams(max_new_tokens=10, seed=s) for s in (11, 22)])
+    assert loop.scheduler.stats["preemptions"] > 0
+    for seed in (11, 22):
+        steps = [s for sd, s in asked if sd == seed]
+        assert steps == list(range(10))  # each draw asked for exactly once, in order

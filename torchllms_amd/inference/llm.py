@@ -1,0 +1,188 @@
+"""``LLM``: load a model folder and generate from prompts, conversations or token ids.
+
+The constructor and ``generate`` keep the reference's argument names and meanings where it has
+them (reference: torchllms/inference/llm.py:95-109 constructor, 693-760 and 1076-1152 generate,
+63-77 ``GenerationResult``).  Behind them sits this engine's continuous-batching scheduler in
+place of the reference's one-prompt-at-a-time loop and static batches, so ``batched`` and
+``batch_size`` are accepted and only bound how many requests run at once.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from pathlib import Path
+from typing import Any, Dict, List, Optional, Sequence, Union
+
+from ..messages.templates import ChatTemplate, FileTokenizer, get_template, tokenize_conversation
+from ..sampling.params import SamplingParams
+
+
+@dataclass
+class GenerationResult:
+    """``token_ids`` includes the stop token when generation stopped on one; ``text`` is decoded
+    without special tokens; ``stop_reason`` is the stop token id, or None when the token budget
+    or the context length ended generation (reference: llm.py:63-77)."""
+
+    text: str
+    token_ids: List[int]
+    stop_reason: Optional[int]
+
+
+class GenerationLoop:
+    """Drives scheduler, step function and sampler until every request is done.  It needs an
+    object with ``step(entries) -> logits`` and ``cache``, and a sampler
+    ``(logits, params, steps) -> token ids``; nothing else."""
+
+    def __init__(self, engine, sampler, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
+                 prefill_chunk: Optional[int] = None):
+        from ..engine.scheduler import Scheduler
+
+        self.engine = engine
+        self.sampler = sampler
+        self.scheduler = Scheduler(engine.cache, max_num_seqs, max_num_batched_tokens, max_model_len, prefill_chunk)
+
+    def run(self, prompts: Sequence[Sequence[int]], params: Sequence[SamplingParams], on_step=None):
+        """Generate for every prompt; returns the finished ``Request`` objects in input order."""
+        sched = self.scheduler
+        requests = [sched.add(("gen", id(self), i), p, sp) for i, (p, sp) in enumerate(zip(prompts, params))]
+        try:
+            while sched.has_work:
+                plan = sched.schedule()
+                logits = self.engine.step(plan.step_entries())
+                sampling = [e.request for e in plan.entries if e.samples]
+                tokens = self.sampler(logits, [r.params for r in sampling], [len(r.output) for r in sampling])
+                sched.update(plan, tokens)
+                if on_step is not None:
+                    on_step(plan)
+        except BaseException:
+            # whatever happens, give pages and slots back (reference: llm.py:602-617)
+            for r in requests:
+                if not r.finished:
+                    sched.abort(r)
+            raise
+        return requests
+
+
+class LLM:
+    def __init__(
+        self,
+        ckpt_paths: Union[str, Path, Sequence[Union[str, Path]]],
+        template_config: Optional[str] = None,
+        eos_ids: Optional[List[int]] = None,
+        max_len: int = 4096,
+        max_bsz: int = 4,
+        device: str = "cuda",
+        precision: Optional[str] = "bfloat16",
+        model_kwargs: Optional[Dict[str, Any]] = None,
+        batched: bool = True,
+        page_size: int = 16,
+        kv_memory_gb: Optional[float] = None,
+        num_pages: Optional[int] = None,
+        max_num_batched_tokens: int = 2048,
+        tokenizer=None,
+        seed: int = 0,
+    ):
+        """``ckpt_paths``: the model folder (config.json + safetensors), or a list whose first
+        entry is that folder or a file in it.  ``precision``: "bfloat16" or "float32"; None takes
+        config.json's ``torch_dtype``.  ``max_len`` bounds prompt + generated tokens of a request,
+        ``max_bsz`` the requests running at once.  ``model_kwargs`` may override ``max_seq_len``
+        (reference: throughput_bench.py:1057-1060)."""
+        from ..engine.engine import Engine
+        from ..sampling.sampler import Sampler
+
+        first = ckpt_paths if isinstance(ckpt_paths, (str, Path)) else list(ckpt_paths)[0]
+        folder = Path(first)
+        if folder.is_file():
+            folder = folder.parent
+        self.folder = folder
+        if device == "cuda":
+            device = "cuda:0"
+        model_kwargs = dict(model_kwargs or {})
+        if precision is None:
+            import json
+
+            with open(folder / "config.json") as f:
+                precision = json.load(f).get("torch_dtype", "bfloat16")
+        if "max_seq_len" in model_kwargs:
+            max_len = min(max_len, int(model_kwargs.pop("max_seq_len")))
+        if model_kwargs:
+            raise ValueError(f"unknown model_kwargs {sorted(model_kwargs)}")
+        self.engine = Engine.from_folder(
+            folder, dtype=precision, device=device, page_size=page_size, num_pages=num_pages,
+            kv_memory_gb=kv_memory_gb, max_seqs=max_bsz, max_model_len=max_len,
+        )
+        self.max_len = self.engine.max_model_len
+        self.max_bsz = max_bsz
+        self.batched = batched
+        self.device = device
+        self.seed = seed
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.template: Optional[ChatTemplate] = get_template(template_config)
+        if tokenizer is None and (folder / "tokenizer.json").is_file():
+            tokenizer = FileTokenizer(folder / "tokenizer.json")
+        self.tokenizer = tokenizer
+        if self.template is not None and self.template.stop_token_ids:
+            eos_ids = list(self.template.stop_token_ids)  # reference: llm.py:188-189
+        if eos_ids is None:
+            eos = self.engine.config.eos_token_id
+            eos_ids = [] if eos is None else (list(eos) if isinstance(eos, (list, tuple)) else [eos])
+        self.eos_ids = list(eos_ids)
+        self.sampler = Sampler()
+
+    # ------------------------------------------------------------------ text <-> ids
+    def _need_tokenizer(self):
+        if self.tokenizer is None:
+            raise ValueError("this model folder has no tokenizer.json: pass prompt_token_ids, or a tokenizer to LLM()")
+        return self.tokenizer
+
+    def tokenize_conversation(self, conversation) -> List[int]:
+        tok = self._need_tokenizer()
+        if self.template is None:
+            raise ValueError("conversations need a template_config (for instance 'llama3_instruct')")
+        return tokenize_conversation(conversation, tok, self.template, add_generation_prompt=True)
+
+    # ------------------------------------------------------------------ generation
+    def generate(
+        self,
+        prompts: Optional[List[str]] = None,
+        conversations: Optional[List[List[Dict[str, str]]]] = None,
+        temperature: float = 0.0,
+        max_new_tokens: Optional[int] = None,
+        batch_size: int = 0,
+        disable_tqdm: bool = True,
+        prompt_token_ids: Optional[List[List[int]]] = None,
+        top_k: Optional[int] = None,
+        stop_token_ids: Optional[Sequence[int]] = None,
+        seed: Optional[int] = None,
+    ) -> List[GenerationResult]:
+        """Exactly one of ``prompts`` (texts, encoded without added special tokens),
+        ``conversations`` (lists of role/content messages) and ``prompt_token_ids``.  Results come
+        back in input order.  ``batch_size`` > 0 bounds the requests running at once below
+        ``max_bsz``.  Request i is sampled with seed ``seed + i``."""
+        given = [x is not None for x in (prompts, conversations, prompt_token_ids)]
+        if sum(given) != 1:
+            raise ValueError("give exactly one of prompts, conversations, prompt_token_ids")
+        if conversations is not None:
+            ids = [self.tokenize_conversation(c) for c in conversations]
+        elif prompts is not None:
+            tok = self._need_tokenizer()
+            ids = [tok.encode(p) for p in prompts]
+        else:
+            ids = [list(p) for p in prompt_token_ids]
+        stops = tuple(self.eos_ids if stop_token_ids is None else stop_token_ids)
+        base = self.seed if seed is None else seed
+        params = [
+            SamplingParams(temperature=temperature, top_k=top_k, max_new_tokens=max_new_tokens, stop_token_ids=stops, seed=base + i)
+            for i in range(len(ids))
+        ]
+        live = self.max_bsz if not batch_size else min(batch_size, self.max_bsz)
+        if not self.batched:
+            live = 1
+        loop = GenerationLoop(self.engine, self.sampler, live, self.max_num_batched_tokens, self.max_len)
+        finished = loop.run(ids, params)
+        self.last_stats = dict(loop.scheduler.stats)
+        out = []
+        for r in finished:
+            text = self.tokenizer.decode(r.output) if self.tokenizer is not None else ""
+            out.append(GenerationResult(text=text, token_ids=list(r.output), stop_reason=r.stop_reason))
+        return out
