@@ -428,3 +428,116 @@ def test_sample_frequencies_follow_softmax():
     assert chi2 < 20.5  # 5 degrees of freedom, p = 0.001
     u = _ops().philox_uniform(9, 0, 100000, DEV).cpu()
     assert abs(u.mean().item() - 0.5) < 0.005 and abs(u.var().item() - 1 / 12) < 0.002
+
+
+# ----------------------------------------------------------------------------- decode attention (MFMA, split-KV)
+def _decode(q, k, v, page, window=0, split_size=None, n_pages=None):
+    """The decode kernel for one token (the last position of the request) with bfloat16 inputs."""
+    hq, dh = q.shape[1], q.shape[2]
+    S, hkv, _ = k.shape
+    n_pages = n_pages or (-(-S // page) + 3)
+    k_pages, v_pages, table = _paged(k.bfloat16(), v.bfloat16(), page, n_pages, dtype=torch.bfloat16)
+    qkv = q.reshape(1, hq * dh).bfloat16().to(DEV).contiguous()
+    lo = max(S - window, 0) if window else 0
+    longest = S - (lo // 16) * 16
+    out = _ops().attention_decode(
+        qkv, hq, hkv, dh, k_pages, v_pages, _i32([0]), _i32([S - 1]), _i32([table]), window, dh ** -0.5, longest, split_size=split_size
+    )
+    return out.float().cpu()
+
+
+@pytest.mark.parametrize(
+    "hq, hkv, dh, page, S, split",
+    [
+        (32, 8, 128, 16, 2000, None), (32, 8, 128, 16, 2000, 64), (32, 8, 128, 16, 2000, 4096), (8, 1, 32, 16, 300, 64),
+        (4, 4, 64, 8, 100, None), (6, 2, 64, 4, 77, 64), (16, 1, 128, 32, 513, 128), (8, 1, 256, 16, 200, 64),
+        (5, 5, 32, 12, 130, 64), (6, 3, 128, 1, 65, 64), (2, 2, 64, 16, 1, None), (4, 1, 128, 16, 16, None), (4, 1, 128, 16, 17, None),
+    ],
+)
+def test_attention_decode(hq, hkv, dh, page, S, split):
+    torch.manual_seed(0)
+    q = (torch.randn(1, hq, dh) * 2).bfloat16().float()
+    k = torch.randn(S, hkv, dh).bfloat16().float()
+    v = torch.randn(S, hkv, dh).bfloat16().float()
+    got = _decode(q, k, v, page, split_size=split)
+    want = plain.attention(q, k, v)
+    torch.testing.assert_close(got, want, rtol=2 ** -7, atol=2 ** -7)
+
+
+def test_attention_decode_finds_a_far_key_among_thousands():
+    torch.manual_seed(0)
+    hq, hkv, dh, page, S = 8, 2, 128, 16, 3000
+    k = torch.randn(S, hkv, dh) * 0.1
+    v = torch.randn(S, hkv, dh)
+    for far in (0, 1, 15, 16, 17, 63, 64, 255, 256, 1000, 2047, 2048, 2998, 2999):
+        kk = k.clone()
+        direction = torch.randn(dh)
+        direction /= direction.norm()
+        kk[far] = direction * 12
+        qq = (direction * 12 * math.sqrt(dh) / 4).expand(1, hq, dh).clone()
+        got = _decode(qq, kk, v, page, split_size=256).view(hq, dh)
+        want = v[far].bfloat16().float().repeat_interleave(hq // hkv, dim=0)
+        assert (got - want).abs().max().item() < 2e-2, f"key {far}"
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 64, 100])
+def test_attention_decode_window(window):
+    torch.manual_seed(0)
+    hq, hkv, dh, page, S = 4, 2, 64, 8, 230
+    q = torch.randn(1, hq, dh).bfloat16().float()
+    k = (torch.randn(S, hkv, dh) * 0.3).bfloat16().float()
+    v = torch.randn(S, hkv, dh).bfloat16().float()
+    torch.testing.assert_close(_decode(q, k, v, page, window=window, split_size=64), _windowed_plain(q, k, v, window), rtol=2 ** -7, atol=2 ** -7)
+    # the key just outside the window matches the query and must stay unseen
+    direction = torch.ones(dh) / math.sqrt(dh)
+    qq = (direction * 40).expand(1, hq, dh).clone()
+    kk = k.clone()
+    kk[S - 1 - window] = direction * 10
+    got = _decode(qq, kk, v, page, window=window, split_size=64)
+    torch.testing.assert_close(got, _windowed_plain(qq, kk.bfloat16().float(), v, window), rtol=2 ** -6, atol=2 ** -6)
+    # pages before the window are released (-1 in the block table) and must not be touched
+    k_pages, v_pages, table = _paged(k.bfloat16(), v.bfloat16(), page, 40, dtype=torch.bfloat16)
+    first_needed = (S - window) // page
+    table = [-1 if blk < first_needed else pg for blk, pg in enumerate(table)]
+    out = _ops().attention_decode(
+        q.reshape(1, hq * dh).bfloat16().to(DEV), hq, hkv, dh, k_pages, v_pages, _i32([0]), _i32([S - 1]), _i32([table]), window, dh ** -0.5, window + 15
+    )
+    torch.testing.assert_close(out.float().cpu(), _windowed_plain(q, k, v, window), rtol=2 ** -7, atol=2 ** -7)
+
+
+def test_attention_decode_batch_with_different_lengths():
+    torch.manual_seed(0)
+    hq, hkv, dh, page = 32, 8, 128, 16
+    lens = [1, 700, 64, 33, 1024, 250]
+    n_pages = sum(-(-n // page) for n in lens) + 5
+    k_pages = torch.full((n_pages, hkv, page, dh), 30.0, dtype=torch.bfloat16)
+    v_pages = torch.full((n_pages, hkv, page, dh), -30.0, dtype=torch.bfloat16)
+    free = torch.randperm(n_pages).tolist()
+    tables, wants, qs = [], [], []
+    for S in lens:
+        k, v, q = torch.randn(S, hkv, dh).bfloat16(), torch.randn(S, hkv, dh).bfloat16(), torch.randn(1, hq, dh).bfloat16()
+        table = [free.pop() for _ in range(-(-S // page))]
+        for pos in range(S):
+            k_pages[table[pos // page], :, pos % page] = k[pos]
+            v_pages[table[pos // page], :, pos % page] = v[pos]
+        tables.append(table + [-1] * (64 - len(table)))
+        wants.append(plain.attention(q.float(), k.float(), v.float()))
+        qs.append(q.reshape(1, hq * dh))
+    # queries sit in a wider row, as in the fused q|k|v buffer
+    wide = torch.cat([torch.cat(qs), torch.randn(len(lens), 2 * hkv * dh).bfloat16()], dim=1).to(DEV)
+    for split in (None, 64, 512):
+        out = _ops().attention_decode(
+            wide, hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32(list(range(len(lens)))), _i32([n - 1 for n in lens]),
+            _i32(tables), 0, dh ** -0.5, max(lens), split_size=split,
+        )
+        torch.testing.assert_close(out.float().cpu(), torch.cat(wants), rtol=2 ** -7, atol=2 ** -7)
+
+
+def test_attention_decode_says_what_it_takes():
+    ops = _ops()
+    assert ops.decode_attention_supported(torch.bfloat16, 32, 8, 128)
+    assert not ops.decode_attention_supported(torch.float32, 32, 8, 128)
+    assert not ops.decode_attention_supported(torch.bfloat16, 6, 3, 48)
+    assert not ops.decode_attention_supported(torch.bfloat16, 16, 1, 256)
+    assert ops.plan_decode_splits(8, 8, 8192) == (512, 16)
+    assert ops.plan_decode_splits(64, 8, 40) == (64, 1)

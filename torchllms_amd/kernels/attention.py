@@ -26,7 +26,26 @@ def paged_attention(
 ) -> torch.Tensor:
     """Attention of this step's queries (first Hq * dh columns of ``qkv``) over their requests'
     cached keys and values; returns [n_tokens, Hq * dh]."""
-    return ops.attention_generic(
-        qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq, ctx.positions,
-        ctx.block_tables[group], window, scale,
+    n = qkv.shape[0]
+    n_dec = ctx.host.n_decode
+    fast_decode = n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
+    if not fast_decode:
+        return ops.attention_generic(
+            qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq, ctx.positions,
+            ctx.block_tables[group], window, scale,
+        )
+    out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    # rows with a single new token come first in the batch: they take the split-KV decode kernel
+    longest = int(ctx.host.positions[:n_dec].max()) + 1
+    if window > 0:
+        longest = min(longest, window + 15)
+    ops.attention_decode(
+        qkv[:n_dec], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[:n_dec], ctx.positions[:n_dec],
+        ctx.block_tables[group], window, scale, longest, out=out[:n_dec],
     )
+    if n_dec < n:
+        ops.attention_generic(
+            qkv[n_dec:], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[n_dec:], ctx.positions[n_dec:],
+            ctx.block_tables[group], window, scale, out=out[n_dec:],
+        )
+    return out

@@ -184,8 +184,10 @@ def build_variant(kind: str, value: int, force: bool = False) -> Path:
     return build_library(variant_name(kind, value), [v["source"]], defines=[f"-D{v['macro']}={value}"], force=force)
 
 
+register_variant("attn_decode", "attention_decode.hip", "TL_HEAD_DIM")
+
 #: sizes compiled ahead of time by ``build_all`` (tests, the smoke run and the benchmark use these)
-PREBUILT_VARIANTS: Dict[str, Iterable[int]] = {}
+PREBUILT_VARIANTS: Dict[str, Iterable[int]] = {"attn_decode": (32, 64, 128)}
 
 
 def build_all(force: bool = False) -> List[Path]:

@@ -11,7 +11,7 @@ from typing import Optional
 
 import torch
 
-from .lib import KernelError, check, core
+from .lib import KernelError, check, core, variant
 
 F32, BF16 = 0, 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -255,4 +255,89 @@ def philox_uniform(seed: int, step: int, n: int, device) -> torch.Tensor:
     """The uniforms the sampler draws for (seed, step) at indices 0..n-1."""
     out = torch.empty((n,), dtype=torch.float32, device=device)
     check(core().tl_philox_uniform(seed & (2**64 - 1), step & (2**64 - 1), out.data_ptr(), n, _stream()))
+    return out
+
+
+# ----------------------------------------------------------------------------- decode attention (bfloat16, MFMA)
+_P, _I, _F = __import__("ctypes").c_void_p, __import__("ctypes").c_int, __import__("ctypes").c_float
+_DECODE_SIGNATURES = {
+    "tl_attn_decode": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P],
+}
+DECODE_HEAD_DIMS = (32, 64, 128, 256)
+_DECODE_BLOCK_KEYS = 64  # keys one block pass covers (4 waves x 16): splits are multiples of it
+
+
+def decode_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: int, head_dim: int) -> bool:
+    """Whether the MFMA decode kernel takes these sizes (else the plain kernel runs)."""
+    if dtype != torch.bfloat16 or head_dim not in DECODE_HEAD_DIMS or n_q_heads % n_kv_heads:
+        return False
+    return n_q_heads // n_kv_heads <= (16 if head_dim <= 128 else 8)
+
+
+def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, target_blocks: int = 1024):
+    """``(split_size, n_splits)`` for a decode launch whose longest visible key range (counted from
+    its 16-aligned start) is ``longest``: enough splits to fill the GPU, none shorter than 64 keys."""
+    pairs = max(n_tokens * n_kv_heads, 1)
+    want = max(-(-target_blocks // pairs), 1)
+    split = -(-max(longest, 1) // want)
+    split = max(-(-split // _DECODE_BLOCK_KEYS) * _DECODE_BLOCK_KEYS, _DECODE_BLOCK_KEYS)
+    return split, max(-(-max(longest, 1) // split), 1)
+
+
+def attention_decode(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    token_seq: torch.Tensor,
+    positions: torch.Tensor,
+    block_table: torch.Tensor,
+    window: int,
+    scale: float,
+    longest: int,
+    out: Optional[torch.Tensor] = None,
+    split_size: Optional[int] = None,
+) -> torch.Tensor:
+    """Attention of single-token queries over their requests' pages with the split-KV MFMA kernel.
+    ``longest``: an upper bound of any token's visible key range, counted from its 16-aligned first
+    visible key (position + 1 without a window)."""
+    _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
+    _i32(token_seq, "token_seq")
+    _i32(positions, "positions")
+    if qkv.dtype != torch.bfloat16:
+        raise KernelError("attention_decode takes bfloat16")
+    n = token_seq.numel()
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[0] < n or qkv.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention_decode: qkv must be row-major with a row per token and at least Hq * dh columns")
+    if positions.numel() != n:
+        raise KernelError("attention_decode: one position per token")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("attention_decode: block_table must be an int32 matrix")
+    page_size = k_pages.shape[2]
+    for pg in (k_pages, v_pages):
+        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+            raise KernelError("attention_decode: pages must be contiguous [pages, Hkv, page_size, dh] bfloat16")
+    if out is None:
+        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    if split_size is None:
+        split_size, n_splits = plan_decode_splits(n, n_kv_heads, longest)
+    else:
+        n_splits = max(-(-max(longest, 1) // split_size), 1)
+    ws_o = ws_ml = None
+    if n_splits > 1:
+        ws_o = torch.empty((n * n_q_heads * n_splits * head_dim,), dtype=torch.float32, device=qkv.device)
+        ws_ml = torch.empty((n * n_q_heads * n_splits * 2,), dtype=torch.float32, device=qkv.device)
+    lib = variant("attn_decode", head_dim, _DECODE_SIGNATURES)
+    check(
+        lib.tl_attn_decode(
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
+            n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), split_size, n_splits,
+            _ptr(ws_o), _ptr(ws_ml), _stream(),
+        ),
+        lib,
+        "tl_variant_last_error",
+    )
     return out
