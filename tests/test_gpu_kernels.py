@@ -541,3 +541,43 @@ def test_attention_decode_says_what_it_takes():
     assert not ops.decode_attention_supported(torch.bfloat16, 16, 1, 256)
     assert ops.plan_decode_splits(8, 8, 8192) == (512, 16)
     assert ops.plan_decode_splits(64, 8, 40) == (64, 1)
+
+
+# ----------------------------------------------------------------------------- skinny matrix product (decode)
+@pytest.mark.parametrize(
+    "m, n, k",
+    [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 14336), (16, 1000, 256), (17, 300, 96), (33, 257, 688), (64, 2048, 1024),
+     (3, 16, 8), (5, 31, 136), (64, 128256 // 8, 512)],
+)
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_skinny(m, n, k, out_dtype):
+    torch.manual_seed(0)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) * 0.05).bfloat16()
+    got = _ops().gemm_skinny(x.to(DEV), w.to(DEV), out_dtype).float().cpu()
+    want = x.double() @ w.double().T
+    tol = (1e-4 if out_dtype == torch.float32 else 2 ** -8) * want.abs().max().item() + 1e-5
+    assert (got.double() - want).abs().max().item() <= tol
+    for waves in (1, 2, 4, 8):
+        alt = _ops().gemm_skinny(x.to(DEV), w.to(DEV), out_dtype, waves=waves).float().cpu()
+        assert (alt.double() - want).abs().max().item() <= tol, f"waves={waves}"
+
+
+def test_gemm_skinny_rows_in_a_wider_buffer_and_limits():
+    from torchllms_amd.kernels.lib import KernelError
+
+    torch.manual_seed(0)
+    wide = torch.randn(6, 512).bfloat16().to(DEV)
+    x = wide[:, :256]  # row stride 512
+    w = torch.randn(40, 256).bfloat16().to(DEV)
+    got = _ops().linear(x, w).float().cpu()
+    torch.testing.assert_close(got, (x.float() @ w.float().T).cpu(), rtol=2 ** -7, atol=0.1)
+    with pytest.raises(KernelError, match="exceeds 64"):
+        _ops().gemm_skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
+    with pytest.raises(KernelError, match="multiple of 8"):
+        _ops().gemm_skinny(torch.zeros(2, 12, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV))
+    # sizes the kernel does not take go to the library
+    odd = _ops().linear(torch.ones(2, 12, dtype=torch.bfloat16, device=DEV), torch.ones(4, 12, dtype=torch.bfloat16, device=DEV))
+    assert odd.float().cpu().tolist() == [[12.0] * 4] * 2
+    big = _ops().linear(torch.ones(70, 16, dtype=torch.bfloat16, device=DEV), torch.ones(4, 16, dtype=torch.bfloat16, device=DEV), out_dtype=torch.float32)
+    assert big.dtype == torch.float32 and big.shape == (70, 4)

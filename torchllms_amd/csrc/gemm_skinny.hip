@@ -1,0 +1,164 @@
+// C[M, N] = A[M, K] * W[N, K]^T for few rows (M <= 64), bfloat16 inputs, 32-bit accumulation:
+// the matrix products of decode steps, whose cost is reading W once from HBM.
+//
+//   * a block owns a strip of 16 output columns (16 rows of W); its waves split K between them and
+//     add their partial sums through LDS in a fixed order (no atomics).
+//   * C^T[16 columns x 16 rows of A] by MFMA 16x16x16 bf16: the A operand is W exactly as it lies in
+//     memory (a lane loads 64 contiguous bytes of its row per step, four lanes cover 256 bytes), the B
+//     operand is A, read through the cache with the same addressing.  M > 16 takes up to four MFMA
+//     column blocks that reuse each W load.
+//   * the result leaves as bfloat16 or as 32-bit (logits).
+#include "common.h"
+
+namespace {
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+union Pack16 {
+  uint4 u;
+  short4_t s[2];
+};
+
+constexpr int kStrip = 16;   // output columns per block
+constexpr int kStepK = 128;  // k covered by one wave step: 4 lane groups x 32 contiguous elements
+
+// MB: MFMA column blocks (M <= 16 * MB).  WAVES: waves per block = splits of K.
+template <int MB, int WAVES, typename OutT>
+__global__ void __launch_bounds__(WAVES* kWave)
+gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
+                   OutT* __restrict__ C, int ldc, int M, int N, int K) {
+  __shared__ float red[WAVES][MB][kWave][4];
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int n16 = lane % 16;
+  const int g4 = lane / 16;
+  const int n0 = blockIdx.x * kStrip;
+
+  // this wave's share of K, in whole steps
+  const int steps_total = (K + kStepK - 1) / kStepK;
+  const int steps_per_wave = (steps_total + WAVES - 1) / WAVES;
+  const int step_lo = wave * steps_per_wave;
+  const int step_hi = min(step_lo + steps_per_wave, steps_total);
+
+  const int wrow = min(n0 + n16, N - 1);  // rows past N are clamped; their results are not stored
+  const bf16_t* wp = W + (size_t)wrow * ldw + 32 * g4;
+  const bf16_t* ap[MB];
+  bool arow_ok[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int m = 16 * b + n16;
+    arow_ok[b] = m < M;
+    ap[b] = A + (size_t)(arow_ok[b] ? m : 0) * lda + 32 * g4;
+  }
+
+  float4_t acc[MB];
+#pragma unroll
+  for (int b = 0; b < MB; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  for (int st = step_lo; st < step_hi; ++st) {
+    const int k0 = st * kStepK;  // this lane reads k0 + 32 g4 + (0..31)
+    Pack16 w[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 32 * g4 + 8 * u;
+      w[u].u = (k < K) ? *reinterpret_cast<const uint4*>(wp + k0 + 8 * u) : zero;
+    }
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+      Pack16 a[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int k = k0 + 32 * g4 + 8 * u;
+        a[u].u = (arow_ok[b] && k < K) ? *reinterpret_cast<const uint4*>(ap[b] + k0 + 8 * u) : zero;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w[u].s[0], a[u].s[0], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w[u].s[1], a[u].s[1], acc[b], 0, 0, 0);
+      }
+    }
+  }
+
+  // acc[b][i] = C^T[n0 + 4 g4 + i][16 b + n16]; add the waves' shares in wave order
+  if (WAVES > 1) {
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wave][b][lane][i] = acc[b][i];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float s = red[0][b][lane][i];
+#pragma unroll
+        for (int w2 = 1; w2 < WAVES; ++w2) s += red[w2][b][lane][i];
+        acc[b][i] = s;
+      }
+  }
+#pragma unroll
+  for (int b = 0; b < MB; ++b) {
+    const int m = 16 * b + n16;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * g4 + i;
+      if (n < N) C[(size_t)m * ldc + n] = from_f32<OutT>(acc[b][i]);
+    }
+  }
+}
+
+template <int MB, int WAVES>
+int launch(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N, int K,
+           int out_dtype, hipStream_t stream) {
+  const dim3 grid((N + kStrip - 1) / kStrip);
+  if (out_dtype == TL_BF16)
+    gemm_skinny_kernel<MB, WAVES, bf16_t><<<grid, WAVES * kWave, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K);
+  else
+    gemm_skinny_kernel<MB, WAVES, float><<<grid, WAVES * kWave, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, M, N, K);
+  return tl_check_launch("gemm_skinny");
+}
+
+template <int MB>
+int launch_waves(int waves, const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N,
+                 int K, int out_dtype, hipStream_t stream) {
+  switch (waves) {
+    case 1: return launch<MB, 1>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+    case 2: return launch<MB, 2>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+    case 4: return launch<MB, 4>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+    default: return launch<MB, 8>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+  }
+}
+
+}  // namespace
+
+// A [M, K] and W [N, K] bfloat16, row-major with leading dimensions lda / ldw (multiples of 8, bases
+// 16-byte aligned); C [M, N] bfloat16 (out_dtype 1) or 32-bit (out_dtype 0).  M <= 64, K a multiple of 8.
+// waves = 0 picks the number of K splits from the sizes.
+TL_EXPORT int tl_gemm_skinny(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
+                             int K, int out_dtype, int waves, hipStream_t stream) {
+  TL_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
+  if (M > 64) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_skinny: M=%d exceeds 64", M);
+  if (K % 8) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_skinny: K=%d is not a multiple of 8", K);
+  TL_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_skinny: leading dimensions too small");
+  TL_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0,
+             "gemm_skinny: rows must start on 16-byte boundaries");
+  TL_REQUIRE(out_dtype == TL_BF16 || out_dtype == TL_F32, "gemm_skinny: out_dtype must be 0 or 1");
+  if (M == 0) return TL_OK;
+  if (waves == 0) {
+    // enough waves to keep loads in flight on 256 CUs: about 4096 in all, at least one step each
+    const int strips = (N + kStrip - 1) / kStrip;
+    const int steps = (K + kStepK - 1) / kStepK;
+    waves = 1;
+    while (waves < 8 && strips * waves < 4096 && steps >= 2 * waves * 2) waves *= 2;
+  }
+  TL_REQUIRE(waves == 1 || waves == 2 || waves == 4 || waves == 8, "gemm_skinny: waves must be 1, 2, 4 or 8");
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  if (M <= 16) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
+  if (M <= 32) return launch_waves<2>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
+  return launch_waves<4>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
+}

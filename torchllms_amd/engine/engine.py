@@ -60,6 +60,7 @@ class Engine:
         max_seqs: int = 8,
         max_model_len: Optional[int] = None,
         device="cuda:0",
+        use_graphs: bool = True,
     ):
         """``tensors``: the model's tensors under the parts' own names, on ``device``.
         Pool size: ``num_pages`` pages per group, else what ``kv_memory_gb`` holds, else room for
@@ -84,6 +85,12 @@ class Engine:
         self.cache = CacheManager(groups, states, page_size, num_pages, max_seqs, dtype=dtype, device=self.device)
         self.steps_run = 0
         self.tokens_run = 0
+        # decode steps are replayed from HIP graphs when every mixer's launches are fixed by the
+        # step's shape alone
+        from .graphs import DecodeGraphs
+
+        graph_safe = all(getattr(b.mixer, "graph_safe", False) for b in self.model.blocks)
+        self.graphs = DecodeGraphs(self) if (use_graphs and graph_safe) else None
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -165,8 +172,11 @@ class Engine:
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         layout = self.plan(entries)
-        ctx = upload(layout, self.device)
-        logits = self.model.forward(ctx, self.cache)
+        if self.graphs is not None and layout.n_decode == layout.n_seqs:
+            logits = self.graphs.run(layout)
+        else:
+            ctx = upload(layout, self.device)
+            logits = self.model.forward(ctx, self.cache)
         for e in entries:
             self.cache.advance(e.rid, len(e.tokens))
         self.steps_run += 1

@@ -1,0 +1,97 @@
+"""Decode steps recorded as HIP graphs.
+
+A decode step launches a few hundred small kernels; issued one by one from Python they take
+longer to launch than to run.  A step whose every request brings exactly one token has a fixed
+shape, so its launches are recorded once into a HIP graph and replayed: the step's plan is copied
+into buffers at fixed addresses, the graph runs, and the logits appear in a fixed tensor.  (The
+reference reaches for ``torch.compile(mode="reduce-overhead")`` here:
+torchllms/inference/llm.py:202-283.)
+
+A graph is keyed by what fixes its launches: the number of requests, the number of wanted logit
+rows, and a power-of-two cap on the context length, which bounds the block tables' width and the
+number of key splits of the decode attention.  No memset node is recorded: buffers are written by
+kernels only.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, Tuple
+
+import torch
+
+from .context import make_context, pack_into, section_offsets, section_shapes
+from .layout import StepLayout
+
+MIN_CONTEXT_CAP = 512
+
+
+def context_cap(max_kv_len: int) -> int:
+    cap = MIN_CONTEXT_CAP
+    while cap < max_kv_len:
+        cap *= 2
+    return cap
+
+
+class DecodeGraph:
+    def __init__(self, engine, layout: StepLayout, cap: int):
+        self.engine = engine
+        self.cap = cap
+        width = -(-cap // engine.page_size)
+        n_groups = len(layout.block_tables)
+        self.shapes = section_shapes(layout.n_tokens, layout.n_seqs, layout.logit_rows.size, [width] * n_groups)
+        self.offsets, total = section_offsets(self.shapes)
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=engine.device)
+        self.copied = torch.cuda.Event()
+        self.graph = None
+        self.logits = None
+        self.replays = 0
+
+    def _load(self, layout: StepLayout) -> None:
+        if self.replays or self.graph is not None:
+            self.copied.synchronize()  # the pinned buffer is free again
+        pack_into(self.host_np, layout, self.shapes, self.offsets)
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+    def first_run(self, layout: StepLayout) -> torch.Tensor:
+        """Run the step eagerly (this is the step's real execution), then record the same launches."""
+        self._load(layout)
+        ctx = make_context(layout, self.dev, self.shapes, self.offsets, decode_longest=self.cap)
+        logits = self.engine.model.forward(ctx, self.engine.cache)
+        result = logits.clone()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.logits = self.engine.model.forward(ctx, self.engine.cache)
+        self.graph = graph
+        self.ctx = ctx
+        return result
+
+    def replay(self, layout: StepLayout) -> torch.Tensor:
+        self._load(layout)
+        self.graph.replay()
+        self.replays += 1
+        return self.logits.clone()
+
+
+class DecodeGraphs:
+    """The engine's recorded decode steps, by (requests, wanted rows, context cap)."""
+
+    def __init__(self, engine, max_graphs: int = 32):
+        self.engine = engine
+        self.max_graphs = max_graphs
+        self.graphs: Dict[Tuple[int, int, int], DecodeGraph] = {}
+
+    def run(self, layout: StepLayout) -> torch.Tensor:
+        cap = context_cap(layout.max_kv_len)
+        key = (layout.n_seqs, int(layout.logit_rows.size), cap)
+        g = self.graphs.get(key)
+        if g is None:
+            if len(self.graphs) >= self.max_graphs:
+                self.graphs.pop(next(iter(self.graphs)))
+            g = DecodeGraph(self.engine, layout, cap)
+            self.graphs[key] = g
+            return g.first_run(layout)
+        return g.replay(layout)

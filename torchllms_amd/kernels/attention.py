@@ -36,7 +36,10 @@ def paged_attention(
         )
     out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
     # rows with a single new token come first in the batch: they take the split-KV decode kernel
-    longest = int(ctx.host.positions[:n_dec].max()) + 1
+    if ctx.decode_longest is not None:
+        longest = ctx.decode_longest
+    else:
+        longest = int(ctx.host.positions[:n_dec].max()) + 1
     if window > 0:
         longest = min(longest, window + 15)
     ops.attention_decode(

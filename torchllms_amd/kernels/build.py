@@ -32,6 +32,7 @@ CORE_SOURCES = [
     "elementwise.hip",
     "attention_generic.hip",
     "gemm_f32.hip",
+    "gemm_skinny.hip",
     "sampling.hip",
 ]
 HEADERS = ["common.h"]

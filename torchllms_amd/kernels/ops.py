@@ -211,13 +211,49 @@ def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """``x @ w.T``.  float32: the 32-bit kernel above.  bfloat16: the BLAS library's matrix product
-    (the reference uses its library's here as well: torchllms/models/networks.py:474-493)."""
+SKINNY_MAX_ROWS = 64
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0) -> torch.Tensor:
+    """``x @ w.T`` for at most 64 rows of bfloat16 ``x`` with the weight-streaming MFMA kernel;
+    the result is bfloat16 or float32."""
+    _gpu(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("gemm_skinny takes bfloat16 tensors")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelError(f"gemm_skinny: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
+    m, k = x.shape
+    n = w.shape[0]
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    check(
+        core().tl_gemm_skinny(
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k,
+            dtype_code(out_dtype), waves, _stream(),
+        )
+    )
+    return out
+
+
+def skinny_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (
+        x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
+        and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+    )
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16 with at most 64 rows (decode): the
+    weight-streaming MFMA kernel.  bfloat16 with more rows (prefill): the BLAS library's matrix
+    product, as the reference uses its library's (torchllms/models/networks.py:474-493).
+    ``out_dtype`` float32 asks for 32-bit results from bfloat16 inputs (logits)."""
     if x.dtype == torch.float32:
         return gemm_f32(x, w)
     _gpu(x, w)
-    return torch.nn.functional.linear(x, w)
+    out_dtype = out_dtype or x.dtype
+    if skinny_supported(x, w):
+        return gemm_skinny(x, w, out_dtype)
+    y = torch.nn.functional.linear(x, w)
+    return y if y.dtype == out_dtype else y.to(out_dtype)
 
 
 def sample(

@@ -23,6 +23,9 @@ class Attention(Mixer):
     projections and reads the cache of the run named by the execution order.
     """
 
+    #: every launch is fixed by the step's shape: a decode step may be recorded in a HIP graph
+    graph_safe = True
+
     def __init__(
         self,
         hidden_size: int,

@@ -53,4 +53,4 @@ class LMHead(Head):
         self.weight = embedding.weight
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.linear(x, self.weight).float()
+        return ops.linear(x, self.weight, out_dtype=torch.float32)
