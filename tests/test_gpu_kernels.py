@@ -546,8 +546,8 @@ def test_attention_decode_says_what_it_takes():
 # ----------------------------------------------------------------------------- skinny matrix product (decode)
 @pytest.mark.parametrize(
     "m, n, k",
-    [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 14336), (16, 1000, 256), (17, 300, 96), (33, 257, 688), (64, 2048, 1024),
-     (3, 16, 8), (5, 31, 136), (64, 128256 // 8, 512)],
+    [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 14336), (16, 1000, 256), (16, 300, 96), (9, 257, 688), (13, 2048, 1024),
+     (3, 16, 8), (5, 31, 136), (16, 128256 // 8, 512)],
 )
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_skinny(m, n, k, out_dtype):
@@ -574,6 +574,8 @@ def test_gemm_skinny_rows_in_a_wider_buffer_and_limits():
     torch.testing.assert_close(got, (x.float() @ w.float().T).cpu(), rtol=2 ** -7, atol=0.1)
     with pytest.raises(KernelError, match="exceeds 64"):
         _ops().gemm_skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
+    many = _ops().gemm_skinny(torch.ones(40, 64, dtype=torch.bfloat16, device=DEV), torch.ones(24, 64, dtype=torch.bfloat16, device=DEV))
+    assert many.float().cpu().tolist() == [[64.0] * 24] * 40  # up to 64 rows through four column blocks
     with pytest.raises(KernelError, match="multiple of 8"):
         _ops().gemm_skinny(torch.zeros(2, 12, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV))
     # sizes the kernel does not take go to the library
@@ -581,3 +583,88 @@ def test_gemm_skinny_rows_in_a_wider_buffer_and_limits():
     assert odd.float().cpu().tolist() == [[12.0] * 4] * 2
     big = _ops().linear(torch.ones(70, 16, dtype=torch.bfloat16, device=DEV), torch.ones(4, 16, dtype=torch.bfloat16, device=DEV), out_dtype=torch.float32)
     assert big.dtype == torch.float32 and big.shape == (70, 4)
+
+
+# ----------------------------------------------------------------------------- prefill attention (MFMA)
+def _prefill(rows, hq, hkv, dh, page, window=0, seed=0):
+    """Run the prefill kernel on a batch: ``rows`` = [(tokens cached after the step, new queries)].
+    Returns (got, want): outputs for all new tokens, row after row."""
+    torch.manual_seed(seed)
+    n_pages = sum(-(-S // page) for S, _ in rows) + 4
+    k_pages = torch.full((n_pages, hkv, page, dh), 40.0, dtype=torch.bfloat16)
+    v_pages = torch.full((n_pages, hkv, page, dh), -40.0, dtype=torch.bfloat16)
+    free = torch.randperm(n_pages).tolist()
+    width = max(-(-S // page) for S, _ in rows)
+    tables, wants, qs, qo, kv = [], [], [], [0], []
+    for S, sq in rows:
+        k = (torch.randn(S, hkv, dh) * 0.5).bfloat16()
+        v = torch.randn(S, hkv, dh).bfloat16()
+        q = (torch.randn(sq, hq, dh) * 2).bfloat16()
+        table = [free.pop() for _ in range(-(-S // page))]
+        for pos in range(S):
+            k_pages[table[pos // page], :, pos % page] = k[pos]
+            v_pages[table[pos // page], :, pos % page] = v[pos]
+        tables.append(table + [-1] * (width - len(table)))
+        wants.append(_windowed_plain(q.float(), k.float(), v.float(), window) if window else plain.attention(q.float(), k.float(), v.float()))
+        qs.append(q.reshape(sq, hq * dh))
+        qo.append(qo[-1] + sq)
+        kv.append(S)
+    ops = _ops()
+    n = qo[-1]
+    wide = torch.cat([torch.cat(qs), torch.randn(n, 2 * hkv * dh).bfloat16()], dim=1).to(DEV)
+    qpt = ops.prefill_queries_per_tile(hq, hkv, dh)
+    trow, tq0 = ops.prefill_tiles(qo, 0, len(rows), qpt)
+    out = torch.zeros(n, hq * dh, dtype=torch.bfloat16, device=DEV)
+    ops.attention_prefill(wide, hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32(qo), _i32(kv), _i32(tables), _i32(trow), _i32(tq0),
+                          window, dh ** -0.5, out)
+    return out.float().cpu(), torch.cat(wants)
+
+
+@pytest.mark.parametrize(
+    "hq, hkv, dh, page, rows",
+    [
+        (32, 8, 128, 16, [(300, 300)]),
+        (32, 8, 128, 16, [(77, 77), (500, 2), (130, 64), (33, 33)]),
+        (8, 1, 32, 16, [(200, 200), (65, 3)]),
+        (4, 4, 64, 8, [(150, 150)]),
+        (6, 2, 64, 4, [(90, 31), (40, 40)]),
+        (16, 1, 128, 32, [(129, 129)]),
+        (4, 1, 256, 16, [(100, 100), (70, 5)]),
+        (5, 5, 32, 12, [(61, 61)]),
+        (2, 2, 64, 16, [(1, 1), (2, 2), (17, 16)]),
+    ],
+)
+def test_attention_prefill(hq, hkv, dh, page, rows):
+    got, want = _prefill(rows, hq, hkv, dh, page)
+    torch.testing.assert_close(got, want, rtol=2 ** -6, atol=2 ** -6)
+
+
+@pytest.mark.parametrize("window", [1, 7, 64, 100])
+def test_attention_prefill_window(window):
+    got, want = _prefill([(260, 260), (300, 40)], 4, 2, 64, 8, window=window)
+    torch.testing.assert_close(got, want, rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_attention_prefill_sharp_scores_find_the_right_key():
+    """Each query matches exactly one key (its own position minus a fixed distance): a kernel that
+    mixes up tiles, pages or the causal edge returns another key's value."""
+    hq, hkv, dh, page, S = 8, 2, 128, 16, 400
+    torch.manual_seed(0)
+    dirs = torch.randn(S, dh)
+    dirs /= dirs.norm(dim=-1, keepdim=True)
+    v = torch.randn(S, hkv, dh).bfloat16()
+    ops = _ops()
+    for dist in (0, 1, 63, 64, 200):
+        k = (dirs * 12)[:, None, :].expand(S, hkv, dh).bfloat16()
+        tgt = (torch.arange(S) - dist).clamp(min=0)
+        q = (dirs[tgt] * 12 * math.sqrt(dh) / 4)[:, None, :].expand(S, hq, dh).bfloat16()
+        n_pages = -(-S // page) + 2
+        k_pages, v_pages, table = _paged(k, v, page, n_pages, dtype=torch.bfloat16)
+        qpt = ops.prefill_queries_per_tile(hq, hkv, dh)
+        trow, tq0 = ops.prefill_tiles([0, S], 0, 1, qpt)
+        out = torch.zeros(S, hq * dh, dtype=torch.bfloat16, device=DEV)
+        ops.attention_prefill(q.reshape(S, hq * dh).to(DEV), hq, hkv, dh, k_pages, v_pages, _i32([0, S]), _i32([S]), _i32([table]),
+                              _i32(trow), _i32(tq0), 0, dh ** -0.5, out)
+        want = v[tgt].float().repeat_interleave(hq // hkv, dim=1).reshape(S, hq * dh)
+        err = (out.float().cpu() - want).abs().amax(dim=1)
+        assert err.max().item() < 3e-2, f"distance {dist}: first bad query {int((err >= 3e-2).nonzero()[0])}"

@@ -43,7 +43,10 @@ typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kTile = 16;             // keys per tile = MFMA M
-constexpr int kWaves = 4;
+#ifndef TL_DECODE_WAVES
+#define TL_DECODE_WAVES 4
+#endif
+constexpr int kWaves = TL_DECODE_WAVES;
 constexpr int kKLoads = DH / 32;      // 16-byte loads a lane makes of its key row
 constexpr int kLPR = DH / 8;          // lanes that cover one value row with 16-byte loads
 constexpr int kRPI = kWave / kLPR;    // value rows one load instruction covers
@@ -135,12 +138,17 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
     return pages + ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH;
   };
 
-  Pack16 kcur[kKLoads], knext[kKLoads];
-  Pack16 vcur[kVLoads], vnext[kVLoads];
-  auto load_tile = [&](int base, Pack16* kd, Pack16* vd) {
+  // Rolling prefetch: the keys of tile t+1 are requested as soon as the MFMAs of tile t have read
+  // their registers, the values of tile t+1 as soon as P.V of tile t is done, so one set of
+  // registers per operand keeps a load in flight at all times.
+  Pack16 kreg[kKLoads];
+  Pack16 vreg[kVLoads];
+  auto load_k = [&](int base, Pack16* kd) {
     const bf16_t* kr = row_ptr(a.k_pages, clamp_key(base + n16));
 #pragma unroll
     for (int u = 0; u < kKLoads; ++u) kd[u].u = *reinterpret_cast<const uint4*>(kr + 32 * u + 8 * g4);
+  };
+  auto load_v = [&](int base, Pack16* vd) {
 #pragma unroll
     for (int j = 0; j < kVLoads; ++j) {
       const bf16_t* vr = row_ptr(a.v_pages, clamp_key(base + j * kRPI + vrow));
@@ -149,18 +157,21 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
   };
 
   int base = split_begin + wave * kTile;
-  if (base <= split_end) load_tile(base, kcur, vcur);
+  if (base <= split_end) {
+    load_k(base, kreg);
+    load_v(base, vreg);
+  }
   for (; base <= split_end; base += kWaves * kTile) {
     const int next = base + kWaves * kTile;
-    if (next <= split_end) load_tile(next, knext, vnext);
 
     // scores S^T[key][head]
     float4_t c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int u = 0; u < kKLoads; ++u) {
-      c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kcur[u].s[0], qreg[u].s[0], c, 0, 0, 0);
-      c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kcur[u].s[1], qreg[u].s[1], c, 0, 0, 0);
+      c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].s[0], qreg[u].s[0], c, 0, 0, 0);
+      c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].s[1], qreg[u].s[1], c, 0, 0, 0);
     }
+    if (next <= split_end) load_k(next, kreg);
     float s[4];
     float tmax = -INFINITY;
 #pragma unroll
@@ -204,7 +215,7 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
       const int kt = j * kRPI + vrow;  // key within the tile
       float vf[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vf[e] = bf16_bits_to_f32(vcur[j].h[e]);
+      for (int e = 0; e < 8; ++e) vf[e] = bf16_bits_to_f32(vreg[j].h[e]);
 #pragma unroll
       for (int h = 0; h < RP; ++h) {
         const float ph = p_lds[wave][kt][h];
@@ -215,10 +226,7 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
-#pragma unroll
-    for (int u = 0; u < kKLoads; ++u) kcur[u] = knext[u];
-#pragma unroll
-    for (int j = 0; j < kVLoads; ++j) vcur[j] = vnext[j];
+    if (next <= split_end) load_v(next, vreg);
   }
 
   // wave-level reductions: sums over the four row groups; outputs over the value-row lanes
@@ -281,19 +289,43 @@ __global__ void __launch_bounds__(kWave) attn_decode_merge_kernel(DecodeArgs a, 
   const int lo_al = lo & ~(kTile - 1);
   const int n_valid = min((p - lo_al) / a.split_size + 1, a.n_splits);
   const size_t slot0 = ((size_t)t * n_q_heads + qh) * a.n_splits;
+  // lane s (and s + 64, ...) reads the statistics of split s; the maximum is reduced over the wave
   float M = -INFINITY;
-  for (int s = 0; s < n_valid; ++s) M = fmaxf(M, a.ws_ml[(slot0 + s) * 2]);
+  for (int s = lane; s < n_valid; s += kWave) M = fmaxf(M, a.ws_ml[(slot0 + s) * 2]);
+  M = wave_max(M);
   float L = 0.f;
-  float o[DH / kWave > 0 ? DH / kWave : 1];
+  for (int s = lane; s < n_valid; s += kWave)
+    L += a.ws_ml[(slot0 + s) * 2 + 1] * __builtin_amdgcn_exp2f(a.ws_ml[(slot0 + s) * 2] - M);
+  L = wave_sum(L);
+  constexpr int NC = (DH + kWave - 1) / kWave;
+  float o[NC];
 #pragma unroll
-  for (int c = 0; c < (DH + kWave - 1) / kWave; ++c) o[c] = 0.f;
-  for (int s = 0; s < n_valid; ++s) {
-    const float f = __builtin_amdgcn_exp2f(a.ws_ml[(slot0 + s) * 2] - M);
-    L += a.ws_ml[(slot0 + s) * 2 + 1] * f;
+  for (int c = 0; c < NC; ++c) o[c] = 0.f;
+  int s = 0;
+  for (; s + 4 <= n_valid; s += 4) {  // four splits' loads in flight at a time
+    float f[4], v[4][NC];
 #pragma unroll
-    for (int c = 0; c < (DH + kWave - 1) / kWave; ++c) {
+    for (int u = 0; u < 4; ++u) {
+      f[u] = a.ws_ml[(slot0 + s + u) * 2];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int d = lane + c * kWave;
+        v[u][c] = d < DH ? a.ws_o[(slot0 + s + u) * DH + d] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float w = __builtin_amdgcn_exp2f(f[u] - M);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) o[c] += v[u][c] * w;
+    }
+  }
+  for (; s < n_valid; ++s) {
+    const float w = __builtin_amdgcn_exp2f(a.ws_ml[(slot0 + s) * 2] - M);
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
       const int d = lane + c * kWave;
-      if (d < DH) o[c] += a.ws_o[(slot0 + s) * DH + d] * f;
+      if (d < DH) o[c] += a.ws_o[(slot0 + s) * DH + d] * w;
     }
   }
 #pragma unroll

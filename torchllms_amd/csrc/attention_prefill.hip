@@ -1,0 +1,325 @@
+// Causal attention of prompt portions over paged bfloat16 keys and values (the cached prefix and
+// the portion itself, which the step has already written into the pages): the prefill kernel.
+//
+//   * a block of 4 waves takes a tile of consecutive queries of one request and one kv head, with
+//     all query heads that share it: its 128 MFMA columns are (query, head) pairs, so a key or value
+//     is fetched once for the whole group.
+//   * keys and values stream through LDS in tiles of 64 keys.  Keys lie there as in the page, values
+//     transposed (channel-major), so that both are MFMA A operands that a lane reads with one
+//     contiguous LDS load.
+//   * scores are computed transposed, S^T[key][column] = K Q^T, by MFMA 16x16x16 bf16; their output
+//     layout is exactly the B-operand layout of P^T in O^T[channel][column] = V^T P^T, so the
+//     probabilities never leave their registers.  Softmax statistics are 32-bit, per column.
+//   * every column has its own causal limit (its query's position) and window start.
+//
+// Compiled once per head size (-DTL_HEAD_DIM=32|64|128|256).
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+
+#ifndef TL_HEAD_DIM
+#error "compile with -DTL_HEAD_DIM=<head size>"
+#endif
+
+static thread_local char g_variant_error[512] = "";
+static int variant_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_variant_error, sizeof(g_variant_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+TL_EXPORT const char* tl_variant_last_error() { return g_variant_error; }
+
+namespace {
+
+constexpr int DH = TL_HEAD_DIM;
+static_assert(DH == 32 || DH == 64 || DH == 128 || DH == 256, "prefill kernel: head size 32, 64, 128 or 256");
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * kWave;
+constexpr int NC = DH <= 128 ? 2 : 1;        // MFMA column blocks per wave
+constexpr int kCols = kWaves * NC * 16;      // columns per block
+constexpr int KT = DH <= 128 ? 64 : 32;       // keys per LDS tile
+constexpr int KL = DH / 32;                  // 16-byte pieces of a key row per lane
+constexpr int DT = DH / 16;                  // channel tiles of the output
+constexpr int kKPitch = DH + 8;              // bf16 elements per key row in LDS
+constexpr int kVPitch = KT + 8;              // bf16 elements per channel row in LDS
+constexpr int kChunksPerRow = DH / 8;        // 16-byte chunks in a key/value row
+constexpr int kLoadsPerThread = KT * kChunksPerRow / kThreads;
+static_assert(KT * kChunksPerRow % kThreads == 0, "tile does not divide over the block");
+
+struct PrefillArgs {
+  const bf16_t* q;
+  int q_stride;
+  bf16_t* out;
+  int out_stride;
+  const bf16_t* k_pages;
+  const bf16_t* v_pages;
+  const int32_t* qo_indptr;   // [rows + 1] first token of each row in this launch's token numbering
+  const int32_t* kv_lens;     // [rows] tokens of the request after this step
+  const int32_t* block_table;
+  int bt_stride;
+  const int32_t* tile_row;    // [tiles] row of each query tile
+  const int32_t* tile_q0;     // [tiles] first query of the tile, counted from the row's first new token
+  int n_kv_heads;
+  int group;
+  int page_size;
+  int page_shift;
+  int window;
+  float scale_log2e;
+};
+
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+// 16 bytes as they come from memory; the two halves are MFMA operands
+struct Pack16 {
+  u32x4_t u;
+  __device__ __forceinline__ short4_t half(int e) const {
+    return __builtin_bit_cast(short4_t, e == 0 ? u32x2_t{u[0], u[1]} : u32x2_t{u[2], u[3]});
+  }
+};
+
+__device__ __forceinline__ uint32_t bf16_bits(float x) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x));
+}
+// two floats -> two bfloat16 in one 32-bit word (first in the low half)
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) { return bf16_bits(a) | (bf16_bits(b) << 16); }
+
+template <int RP>
+__global__ void __launch_bounds__(kThreads) attn_prefill_kernel(PrefillArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[KT * kKPitch];
+  __shared__ __attribute__((aligned(16))) bf16_t vt_lds[DH * kVPitch];
+  constexpr int QB = kCols / RP;  // queries per block
+
+  const int tile = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int n16 = lane % 16;
+  const int g4 = lane / 16;
+  const int R = a.group;
+
+  const int row = a.tile_row[tile];
+  const int q0 = a.tile_q0[tile];
+  const int tok0 = a.qo_indptr[row];
+  const int q_len = a.qo_indptr[row + 1] - tok0;
+  const int kv_len = a.kv_lens[row];
+  const int pos0 = kv_len - q_len;  // position of the row's first new token
+  const int32_t* bt = a.block_table + (size_t)row * a.bt_stride;
+  const size_t head_elems = (size_t)a.page_size * DH;
+
+  auto window_lo = [&](int pos) { return (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0; };
+  const int q_last = min(q0 + QB, q_len) - 1;       // last query of the tile
+  const int key_lo = window_lo(pos0 + q0);          // first key any column sees
+  const int key_hi = pos0 + q_last;                 // last key any column sees
+  const int tile_begin = key_lo & ~(KT - 1);
+
+  // this lane's columns: col -> (query, head)
+  int col_pos[NC], col_lo[NC], col_tok[NC], col_head[NC];
+  bool col_ok[NC];
+  Pack16 qreg[NC][KL];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int col = 16 * (wave * NC + i) + n16;
+    const int ql = q0 + col / RP;
+    const int hh = col % RP;
+    col_ok[i] = ql < q_len && hh < R;
+    col_tok[i] = tok0 + (col_ok[i] ? ql : q0);
+    col_head[i] = kvh * R + (col_ok[i] ? hh : 0);
+    // a column that stands for nothing sees every key with a zero query: finite, never stored
+    col_pos[i] = col_ok[i] ? pos0 + ql : 0x3fffffff;
+    col_lo[i] = col_ok[i] ? window_lo(pos0 + ql) : 0;
+    const bf16_t* qrow = a.q + (size_t)col_tok[i] * a.q_stride + (size_t)col_head[i] * DH;
+#pragma unroll
+    for (int u = 0; u < KL; ++u) {
+      qreg[i][u].u = *reinterpret_cast<const u32x4_t*>(qrow + 32 * u + 8 * g4);
+      if (!col_ok[i]) qreg[i][u].u = u32x4_t{0u, 0u, 0u, 0u};
+    }
+  }
+  // range of keys this wave's columns can see at all (tiles outside it are skipped)
+  int wave_hi = -1, wave_lo = 0x3fffffff;
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int p_ok = col_ok[i] ? col_pos[i] : -1;
+    const int l_ok = col_ok[i] ? col_lo[i] : 0x3fffffff;
+    wave_hi = max(wave_hi, p_ok);
+    wave_lo = min(wave_lo, l_ok);
+  }
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    wave_hi = max(wave_hi, __shfl_xor(wave_hi, off, kWave));
+    wave_lo = min(wave_lo, __shfl_xor(wave_lo, off, kWave));
+  }
+
+  float m_run[NC], l_part[NC];
+  float4_t acc[NC][DT];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    m_run[i] = -INFINITY;
+    l_part[i] = 0.f;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[i][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // global -> registers for one tile of keys and values; keys outside the visible range are
+  // clamped into it (their scores are masked), so no load touches a page the request does not hold
+  Pack16 kst[kLoadsPerThread], vst[kLoadsPerThread];
+  auto fetch = [&](int base) {
+#pragma unroll
+    for (int j = 0; j < kLoadsPerThread; ++j) {
+      const int id = threadIdx.x + j * kThreads;
+      int key = base + id / kChunksPerRow;
+      key = key < key_lo ? key_lo : (key > key_hi ? key_hi : key);
+      const int blk = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
+      const int off = a.page_shift >= 0 ? key & (a.page_size - 1) : key % a.page_size;
+      const size_t at = ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH + 8 * (id % kChunksPerRow);
+      kst[j].u = *reinterpret_cast<const u32x4_t*>(a.k_pages + at);
+      vst[j].u = *reinterpret_cast<const u32x4_t*>(a.v_pages + at);
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int j = 0; j < kLoadsPerThread; ++j) {
+      const int id = threadIdx.x + j * kThreads;
+      const int key = id / kChunksPerRow;
+      const int dc = id % kChunksPerRow;
+      *reinterpret_cast<u32x4_t*>(&k_lds[key * kKPitch + 8 * dc]) = kst[j].u;
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        reinterpret_cast<uint16_t*>(vt_lds)[(8 * dc + e) * kVPitch + key] = (uint16_t)(vst[j].u[e / 2] >> (16 * (e & 1)));
+    }
+  };
+
+  fetch(tile_begin);
+  for (int base = tile_begin; base <= key_hi; base += KT) {
+    __syncthreads();  // the previous tile has been read by every wave
+    stash();
+    __syncthreads();
+    if (base + KT <= key_hi) fetch(base + KT);  // in flight while this tile is computed
+
+    if (base > wave_hi || base + KT - 1 < wave_lo) continue;  // nothing here for this wave's columns
+#pragma unroll
+    for (int sub = 0; sub < KT / 16; ++sub) {
+      const int kb = base + 16 * sub;
+      if (kb > wave_hi || kb + 15 < wave_lo) continue;
+      Pack16 ka[KL];
+#pragma unroll
+      for (int u = 0; u < KL; ++u)
+        ka[u].u = *reinterpret_cast<const u32x4_t*>(&k_lds[(16 * sub + n16) * kKPitch + 32 * u + 8 * g4]);
+      short4_t pb[NC];
+#pragma unroll
+      for (int i = 0; i < NC; ++i) {
+        float4_t c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < KL; ++u) {
+          c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[u].half(0), qreg[i][u].half(0), c, 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[u].half(1), qreg[i][u].half(1), c, 0, 0, 0);
+        }
+        float s[4];
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = kb + 4 * g4 + r;
+          const bool valid = key >= col_lo[i] && key <= col_pos[i];
+          s[r] = valid ? c[r] * a.scale_log2e : -INFINITY;
+          tmax = fmaxf(tmax, s[r]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+        const float m_new = fmaxf(m_run[i], tmax);
+        // a column may not have met a visible key yet: then nothing is rescaled and nothing added
+        const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run[i] - m_new);
+        float pr[4];
+        float psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          pr[r] = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s[r] - m_new);
+          psum += pr[r];
+        }
+        l_part[i] = l_part[i] * alpha + psum;
+        m_run[i] = m_new;
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha;
+        pb[i] = __builtin_bit_cast(short4_t, u32x2_t{pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3])});
+      }
+      // O^T[channel][column] += V^T[channel][key] P^T[key][column]
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        const short4_t va = *reinterpret_cast<const short4_t*>(&vt_lds[(16 * t + n16) * kVPitch + 16 * sub + 4 * g4]);
+#pragma unroll
+        for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb[i], acc[i][t], 0, 0, 0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    float l = l_part[i];
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (!col_ok[i]) continue;
+    const float inv = 1.0f / l;
+    bf16_t* orow = a.out + (size_t)col_tok[i] * a.out_stride + (size_t)col_head[i] * DH;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      const uint2 o = make_uint2(pack_bf16x2(acc[i][t][0] * inv, acc[i][t][1] * inv),
+                                 pack_bf16x2(acc[i][t][2] * inv, acc[i][t][3] * inv));
+      *reinterpret_cast<uint2*>(orow + 16 * t + 4 * g4) = o;
+    }
+  }
+}
+
+}  // namespace
+
+TL_EXPORT int tl_attn_prefill_head_dim() { return DH; }
+
+// Columns of one block: a tile holds tl_attn_prefill_block_cols() / RP queries, RP = the number of
+// query heads per kv head rounded up to a power of two.
+TL_EXPORT int tl_attn_prefill_block_cols() { return kCols; }
+
+// q: element (t, h, d) at q + t*q_stride + h*DH + d, token t counted as in qo_indptr; out likewise.
+// Pages [page][Hkv][page_size][DH].  Row r holds tokens qo_indptr[r]..qo_indptr[r+1]-1, which are the
+// last positions of a request of kv_lens[r] tokens.  tile_row / tile_q0 list the query tiles (see above).
+TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
+                              const void* v_pages, const int32_t* qo_indptr, const int32_t* kv_lens,
+                              const int32_t* block_table, int bt_stride, const int32_t* tile_row,
+                              const int32_t* tile_q0, int n_tiles, int n_q_heads, int n_kv_heads, int head_dim,
+                              int page_size, int window, float scale, hipStream_t stream) {
+  if (head_dim != DH) return variant_fail(TL_ERR_ARG, "attn_prefill: built for head_dim %d, called with %d", DH, head_dim);
+  if (n_tiles < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || page_size <= 0 || bt_stride <= 0 || window < 0)
+    return variant_fail(TL_ERR_ARG, "attn_prefill: bad sizes");
+  if (n_q_heads % n_kv_heads) return variant_fail(TL_ERR_ARG, "attn_prefill: %d query heads are not a multiple of %d kv heads", n_q_heads, n_kv_heads);
+  const int R = n_q_heads / n_kv_heads;
+  if (R > 16) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: %d query heads per kv head exceed 16", R);
+  if (n_kv_heads > 65535) return variant_fail(TL_ERR_ARG, "attn_prefill: grid out of range");
+  if (q_stride % 8 || ((uintptr_t)q % 16) || out_stride % 4 || ((uintptr_t)out % 8))
+    return variant_fail(TL_ERR_ARG, "attn_prefill: queries need 16-byte aligned rows, outputs 8-byte aligned rows");
+  if (n_tiles == 0) return TL_OK;
+  PrefillArgs a;
+  a.q = (const bf16_t*)q; a.q_stride = q_stride; a.out = (bf16_t*)out; a.out_stride = out_stride;
+  a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
+  a.qo_indptr = qo_indptr; a.kv_lens = kv_lens; a.block_table = block_table; a.bt_stride = bt_stride;
+  a.tile_row = tile_row; a.tile_q0 = tile_q0;
+  a.n_kv_heads = n_kv_heads; a.group = R; a.page_size = page_size; a.window = window;
+  a.page_shift = -1;
+  for (int sh = 0; sh < 31; ++sh)
+    if ((1 << sh) == page_size) a.page_shift = sh;
+  a.scale_log2e = scale * 1.4426950408889634f;
+  dim3 grid(n_tiles, n_kv_heads);
+  if (R == 1) attn_prefill_kernel<1><<<grid, kThreads, 0, stream>>>(a);
+  else if (R == 2) attn_prefill_kernel<2><<<grid, kThreads, 0, stream>>>(a);
+  else if (R <= 4) attn_prefill_kernel<4><<<grid, kThreads, 0, stream>>>(a);
+  else if (R <= 8) attn_prefill_kernel<8><<<grid, kThreads, 0, stream>>>(a);
+  else attn_prefill_kernel<16><<<grid, kThreads, 0, stream>>>(a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return variant_fail(TL_ERR_HIP, "attn_prefill: %s", hipGetErrorString(e));
+  return TL_OK;
+}

@@ -94,6 +94,67 @@ rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ delta, const int32
   }
 }
 
+// Fast path: rows whose length is a multiple of the 16-byte vector and at most kNormThreads * 4 vectors
+// long are read with 16-byte loads and kept in registers between the two passes.
+template <typename T, typename WT>
+__global__ void __launch_bounds__(kNormThreads)
+rmsnorm_vec_kernel(const T* __restrict__ x, const T* __restrict__ delta, const int32_t* __restrict__ rows,
+                   const WT* __restrict__ weight, T* __restrict__ h_out, T* __restrict__ y, int hidden,
+                   float eps) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int MAXV = 4;
+  __shared__ float scratch[kNormThreads / kWave];
+  const int r = blockIdx.x;
+  const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+  const int n_vec = hidden / VEC;
+  const uint4* xr = reinterpret_cast<const uint4*>(x + s * hidden);
+  const uint4* dr = delta ? reinterpret_cast<const uint4*>(delta + s * hidden) : nullptr;
+  union V { uint4 u; T e[VEC]; };
+  float v[MAXV][VEC];
+  V xin[MAXV], din[MAXV];
+#pragma unroll
+  for (int it = 0; it < MAXV; ++it) {
+    const int c = threadIdx.x + it * kNormThreads;
+    if (c < n_vec) {
+      xin[it].u = xr[c];
+      if (dr) din[it].u = dr[c];
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < MAXV; ++it) {
+    const int c = threadIdx.x + it * kNormThreads;
+    if (c < n_vec) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float f = to_f32(xin[it].e[e]);
+        if (dr) f = to_f32(from_f32<T>(f + to_f32(din[it].e[e])));
+        v[it][e] = f;
+        ss += f * f;
+      }
+    }
+  }
+  ss = block_sum<kNormThreads / kWave>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+  uint4* yr = reinterpret_cast<uint4*>(y + (size_t)r * hidden);
+  uint4* hr = h_out ? reinterpret_cast<uint4*>(h_out + (size_t)r * hidden) : nullptr;
+#pragma unroll
+  for (int it = 0; it < MAXV; ++it) {
+    const int c = threadIdx.x + it * kNormThreads;
+    if (c < n_vec) {
+      V out, hs;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        hs.e[e] = from_f32<T>(v[it][e]);
+        const float n = to_f32(from_f32<T>(v[it][e] * inv));
+        out.e[e] = from_f32<T>(n * to_f32(weight[c * VEC + e]));
+      }
+      yr[c] = out.u;
+      if (hr) hr[c] = hs.u;
+    }
+  }
+}
+
 TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, const void* weight,
                          int weight_dtype, void* h_out, void* y, int n_rows, int hidden, float eps,
                          int dtype, hipStream_t stream) {
@@ -102,6 +163,23 @@ TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, 
   TL_REQUIRE((size_t)hidden * sizeof(float) <= 160 * 1024 - 1024, "rmsnorm: hidden=%d does not fit LDS", hidden);
   if (n_rows == 0) return TL_OK;
   const size_t lds = (size_t)hidden * sizeof(float);
+  const int vec = dtype == TL_F32 ? 4 : 8;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && (!delta || (uintptr_t)delta % 16 == 0) &&
+                       (!h_out || (uintptr_t)h_out % 16 == 0);
+  if (hidden % vec == 0 && hidden / vec <= kNormThreads * 4 && aligned) {
+    if (dtype == TL_F32 && weight_dtype == TL_F32)
+      rmsnorm_vec_kernel<float, float><<<n_rows, kNormThreads, 0, stream>>>(
+          (const float*)x, (const float*)delta, rows, (const float*)weight, (float*)h_out, (float*)y, hidden, eps);
+    else if (dtype == TL_BF16 && weight_dtype == TL_BF16)
+      rmsnorm_vec_kernel<bf16_t, bf16_t><<<n_rows, kNormThreads, 0, stream>>>(
+          (const bf16_t*)x, (const bf16_t*)delta, rows, (const bf16_t*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps);
+    else if (dtype == TL_BF16 && weight_dtype == TL_F32)
+      rmsnorm_vec_kernel<bf16_t, float><<<n_rows, kNormThreads, 0, stream>>>(
+          (const bf16_t*)x, (const bf16_t*)delta, rows, (const float*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps);
+    else
+      return tl_fail(TL_ERR_ARG, "rmsnorm: unsupported dtypes x=%d weight=%d", dtype, weight_dtype);
+    return tl_check_launch("rmsnorm");
+  }
 #define TL_NORM_LAUNCH(T, WT)                                                                       \
   do {                                                                                              \
     if (lds > 48 * 1024) {                                                                          \
@@ -148,15 +226,18 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_k
   const int off = slot >= 0 ? slot % page_size : 0;
   const bool store = k_pages != nullptr && slot >= 0;
 
-  // queries and keys: one thread per (head, pair)
+  // queries and keys: a thread owns one pair index and walks over heads, so the angle's cosine and
+  // sine are formed once per (token, pair)
   const int n_rot_heads = n_q_heads + n_kv_heads;
-  for (int w = threadIdx.x; w < n_rot_heads * half; w += blockDim.x) {
-    const int h = w / half;
-    const int i = w % half;
-    T* head = base + (size_t)h * head_dim;
+  const int lanes_per_head = half;                       // threads that cover the pairs of one head
+  const int head_groups = blockDim.x / lanes_per_head > 0 ? blockDim.x / lanes_per_head : 1;
+  for (int i = threadIdx.x % lanes_per_head; i < half; i += blockDim.x) {
+    const int hgrp = threadIdx.x / lanes_per_head;
+    if (hgrp >= head_groups) continue;
     int i0, i1;
-    float x0, x1;
-    if (i < rot_half) {
+    float c = 1.f, sn = 0.f;
+    const bool rotates = i < rot_half;
+    if (rotates) {
       if (pairing == 0) {
         i0 = 2 * i;
         i1 = 2 * i + 1;
@@ -164,31 +245,32 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_k
         i0 = i;
         i1 = i + rot_half;
       }
-      const float a0 = to_f32(head[i0]);
-      const float a1 = to_f32(head[i1]);
       const float ang = pos * inv_freq[i];
-      const float c = cosf(ang);
-      const float s = sinf(ang);
-      x0 = a0 * c - a1 * s;
-      x1 = a1 * c + a0 * s;
+      c = cosf(ang);
+      sn = sinf(ang);
     } else {
       // channels beyond rotary_dim pass unchanged
       i0 = rotary_dim + 2 * (i - rot_half);
       i1 = i0 + 1;
-      x0 = to_f32(head[i0]);
-      x1 = to_f32(head[i1]);
     }
-    const T r0 = from_f32<T>(x0);
-    const T r1 = from_f32<T>(x1);
-    if (h < n_q_heads || k_pages == nullptr) {
-      head[i0] = r0;
-      head[i1] = r1;
-    }
-    if (h >= n_q_heads && store) {
-      const int kh = h - n_q_heads;
-      T* dst = k_pages + (((size_t)page * n_kv_heads + kh) * page_size + off) * head_dim;
-      dst[i0] = r0;
-      dst[i1] = r1;
+    for (int h = hgrp; h < n_rot_heads; h += head_groups) {
+      T* head = base + (size_t)h * head_dim;
+      const float a0 = to_f32(head[i0]);
+      const float a1 = to_f32(head[i1]);
+      const float x0 = rotates ? a0 * c - a1 * sn : a0;
+      const float x1 = rotates ? a1 * c + a0 * sn : a1;
+      const T r0 = from_f32<T>(x0);
+      const T r1 = from_f32<T>(x1);
+      if (h < n_q_heads || k_pages == nullptr) {
+        head[i0] = r0;
+        head[i1] = r1;
+      }
+      if (h >= n_q_heads && store) {
+        const int kh = h - n_q_heads;
+        T* dst = k_pages + (((size_t)page * n_kv_heads + kh) * page_size + off) * head_dim;
+        dst[i0] = r0;
+        dst[i1] = r1;
+      }
     }
   }
   // values

@@ -15,8 +15,11 @@ namespace {
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
 union Pack16 {
   uint4 u;
+  u32x4_t v;
   short4_t s[2];
 };
 
@@ -56,29 +59,65 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
 #pragma unroll
   for (int b = 0; b < MB; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  const uint4 zero = make_uint4(0, 0, 0, 0);
-  for (int st = step_lo; st < step_hi; ++st) {
-    const int k0 = st * kStepK;  // this lane reads k0 + 32 g4 + (0..31)
-    Pack16 w[4];
+  // Loads never branch: addresses past K are clamped into the row and the A side is zeroed by a
+  // mask, so out-of-range products vanish.  Two stages: the loads of step s+1 are issued before the
+  // MFMAs of step s.
+  const int kmax = K - 8;  // last 16-byte piece of a row
+  auto load_w = [&](int st, Pack16* w) {
+    const int k0 = st * kStepK + 32 * g4;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int k = k0 + 32 * g4 + 8 * u;
-      w[u].u = (k < K) ? *reinterpret_cast<const uint4*>(wp + k0 + 8 * u) : zero;
+      const int k = min(k0 + 8 * u, kmax);
+      w[u].v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp - 32 * g4 + k));
     }
+  };
+  auto load_a = [&](int st, int b, Pack16* a) {
+    const int k0 = st * kStepK + 32 * g4;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 8 * u;
+      const uint4 v = *reinterpret_cast<const uint4*>(ap[b] - 32 * g4 + min(k, kmax));
+      const uint32_t keep = (arow_ok[b] && k < K) ? 0xFFFFFFFFu : 0u;
+      a[u].u = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
+    }
+  };
+
+  Pack16 w0[4], w1[4];
+  Pack16 a0[MB][4], a1[MB][4];
+  auto load = [&](int st, Pack16* w, Pack16 (*a)[4]) {
+    load_w(st, w);
+#pragma unroll
+    for (int b = 0; b < MB; ++b) load_a(st, b, a[b]);
+  };
+  auto mma = [&](const Pack16* w, const Pack16 (*a)[4]) {
 #pragma unroll
     for (int b = 0; b < MB; ++b) {
-      Pack16 a[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const int k = k0 + 32 * g4 + 8 * u;
-        a[u].u = (arow_ok[b] && k < K) ? *reinterpret_cast<const uint4*>(ap[b] + k0 + 8 * u) : zero;
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w[u].s[0], a[u].s[0], acc[b], 0, 0, 0);
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w[u].s[1], a[u].s[1], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w[u].s[0], a[b][u].s[0], acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(w[u].s[1], a[b][u].s[1], acc[b], 0, 0, 0);
       }
     }
+  };
+  // Rows of W lie a power of two apart, so blocks that walk K in step would all press on the same
+  // memory channels at once; every block therefore starts its walk at a different step and wraps
+  // around.  Two steps per trip so that both buffers are named statically (they stay in registers).
+  const int nst = step_hi - step_lo;
+  const int rot = nst > 0 ? (int)((blockIdx.x * 5u + wave * 3u) % (unsigned)nst) : 0;
+  auto step_of = [&](int i) {
+    int s = i + rot;
+    if (s >= nst) s -= nst;
+    return step_lo + s;
+  };
+  int i = 0;
+  if (i < nst) load(step_of(i), w0, a0);
+  while (i < nst) {
+    if (i + 1 < nst) load(step_of(i + 1), w1, a1);
+    mma(w0, a0);
+    if (i + 1 >= nst) break;
+    if (i + 2 < nst) load(step_of(i + 2), w0, a0);
+    mma(w1, a1);
+    i += 2;
   }
 
   // acc[b][i] = C^T[n0 + 4 g4 + i][16 b + n16]; add the waves' shares in wave order

@@ -33,6 +33,8 @@ class StepContext:
     block_tables: List[torch.Tensor] = field(default_factory=list)
     slot_mappings: List[torch.Tensor] = field(default_factory=list)
     decode_longest: Optional[int] = None
+    #: what kernels derive from the plan once per step and share between layers
+    scratch: dict = field(default_factory=dict)
 
     @property
     def n_tokens(self) -> int:

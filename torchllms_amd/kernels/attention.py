@@ -29,26 +29,48 @@ def paged_attention(
     n = qkv.shape[0]
     n_dec = ctx.host.n_decode
     fast_decode = n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
-    if not fast_decode:
+    fast_prefill = n_dec < n and ops.prefill_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
+    if not fast_decode and not fast_prefill:
         return ops.attention_generic(
             qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq, ctx.positions,
             ctx.block_tables[group], window, scale,
         )
     out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
     # rows with a single new token come first in the batch: they take the split-KV decode kernel
-    if ctx.decode_longest is not None:
-        longest = ctx.decode_longest
-    else:
-        longest = int(ctx.host.positions[:n_dec].max()) + 1
-    if window > 0:
-        longest = min(longest, window + 15)
-    ops.attention_decode(
-        qkv[:n_dec], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[:n_dec], ctx.positions[:n_dec],
-        ctx.block_tables[group], window, scale, longest, out=out[:n_dec],
-    )
+    if n_dec > 0:
+        if fast_decode:
+            if ctx.decode_longest is not None:
+                longest = ctx.decode_longest
+            else:
+                longest = int(ctx.host.positions[:n_dec].max()) + 1
+            if window > 0:
+                longest = min(longest, window + 15)
+            ops.attention_decode(
+                qkv[:n_dec], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[:n_dec],
+                ctx.positions[:n_dec], ctx.block_tables[group], window, scale, longest, out=out[:n_dec],
+            )
+        else:
+            ops.attention_generic(
+                qkv[:n_dec], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[:n_dec],
+                ctx.positions[:n_dec], ctx.block_tables[group], window, scale, out=out[:n_dec],
+            )
+    # rows that bring a portion of a prompt take the tiled MFMA kernel
     if n_dec < n:
-        ops.attention_generic(
-            qkv[n_dec:], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[n_dec:], ctx.positions[n_dec:],
-            ctx.block_tables[group], window, scale, out=out[n_dec:],
-        )
+        if fast_prefill:
+            qpt = ops.prefill_queries_per_tile(n_q_heads, n_kv_heads, head_dim)
+            tiles = ctx.scratch.get(("prefill_tiles", qpt))
+            if tiles is None:
+                rows, q0s = ops.prefill_tiles(ctx.host.qo_indptr, n_dec, ctx.host.n_seqs, qpt)
+                both = torch.tensor([rows, q0s], dtype=torch.int32).to(qkv.device)
+                tiles = (both[0], both[1])
+                ctx.scratch[("prefill_tiles", qpt)] = tiles
+            ops.attention_prefill(
+                qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.qo_indptr, ctx.kv_lens,
+                ctx.block_tables[group], tiles[0], tiles[1], window, scale, out,
+            )
+        else:
+            ops.attention_generic(
+                qkv[n_dec:], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[n_dec:],
+                ctx.positions[n_dec:], ctx.block_tables[group], window, scale, out=out[n_dec:],
+            )
     return out

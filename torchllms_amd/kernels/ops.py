@@ -211,7 +211,11 @@ def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 16
+#: the weight-streaming kernel is used for matrices up to this many elements; measured on MI355X, the
+#: BLAS library's kernels stream larger matrices faster (3.9-5.8 TB/s against 2.7-3.3 TB/s), while on
+#: smaller ones (4096 x 4096: 13 us against 20 us) its launch and tail costs make it the slower one
+SKINNY_MAX_ELEMENTS = 1 << 24
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0) -> torch.Tensor:
@@ -237,13 +241,14 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
 def skinny_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
     return (
         x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
+        and w.shape[0] * w.shape[1] <= SKINNY_MAX_ELEMENTS
         and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
     )
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16 with at most 64 rows (decode): the
-    weight-streaming MFMA kernel.  bfloat16 with more rows (prefill): the BLAS library's matrix
+    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16: the weight-streaming MFMA kernel for
+    few rows and small matrices (see ``SKINNY_MAX_ELEMENTS``), else the BLAS library's matrix
     product, as the reference uses its library's (torchllms/models/networks.py:474-493).
     ``out_dtype`` float32 asks for 32-bit results from bfloat16 inputs (logits)."""
     if x.dtype == torch.float32:
@@ -372,6 +377,90 @@ def attention_decode(
             token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
             n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), split_size, n_splits,
             _ptr(ws_o), _ptr(ws_ml), _stream(),
+        ),
+        lib,
+        "tl_variant_last_error",
+    )
+    return out
+
+
+# ----------------------------------------------------------------------------- prefill attention (bfloat16, MFMA)
+_PREFILL_SIGNATURES = {
+    "tl_attn_prefill": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+}
+PREFILL_HEAD_DIMS = (32, 64, 128, 256)
+
+
+def prefill_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: int, head_dim: int) -> bool:
+    """Whether the MFMA prefill kernel takes these sizes (else the plain kernel runs)."""
+    return dtype == torch.bfloat16 and head_dim in PREFILL_HEAD_DIMS and n_q_heads % n_kv_heads == 0 and n_q_heads // n_kv_heads <= 16
+
+
+def prefill_queries_per_tile(n_q_heads: int, n_kv_heads: int, head_dim: int) -> int:
+    """Queries one block of the prefill kernel covers: its MFMA columns (128, or 64 at head size 256)
+    divided by the group size rounded up to a power of two."""
+    group = n_q_heads // n_kv_heads
+    rp = 1
+    while rp < group:
+        rp *= 2
+    return (128 if head_dim <= 128 else 64) // rp
+
+
+def prefill_tiles(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int):
+    """Host lists ``(tile_row, tile_q0)`` that cut rows ``first_row .. n_rows-1`` into query tiles."""
+    rows, q0s = [], []
+    for r in range(first_row, n_rows):
+        q_len = int(qo_indptr[r + 1]) - int(qo_indptr[r])
+        for q0 in range(0, q_len, queries_per_tile):
+            rows.append(r)
+            q0s.append(q0)
+    return rows, q0s
+
+
+def attention_prefill(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    qo_indptr: torch.Tensor,
+    kv_lens: torch.Tensor,
+    block_table: torch.Tensor,
+    tile_row: torch.Tensor,
+    tile_q0: torch.Tensor,
+    window: int,
+    scale: float,
+    out: torch.Tensor,
+) -> torch.Tensor:
+    """Causal attention of the rows named by the tile lists (see ``prefill_tiles``) with the MFMA
+    prefill kernel.  Token t of ``qkv`` / ``out`` is token t of ``qo_indptr``'s numbering."""
+    _gpu(qkv, k_pages, v_pages, qo_indptr, kv_lens, block_table, tile_row, tile_q0, out)
+    for t, what in ((qo_indptr, "qo_indptr"), (kv_lens, "kv_lens"), (tile_row, "tile_row"), (tile_q0, "tile_q0")):
+        _i32(t, what)
+    if qkv.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise KernelError("attention_prefill takes bfloat16")
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention_prefill: qkv must be row-major with at least Hq * dh columns")
+    if out.dim() != 2 or out.stride(1) != 1 or out.shape[0] != qkv.shape[0] or out.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention_prefill: out must be row-major [tokens, >= Hq * dh]")
+    if tile_row.numel() != tile_q0.numel():
+        raise KernelError("attention_prefill: tile lists differ in length")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("attention_prefill: block_table must be an int32 matrix")
+    if kv_lens.numel() != block_table.shape[0] or qo_indptr.numel() != kv_lens.numel() + 1:
+        raise KernelError("attention_prefill: qo_indptr, kv_lens and block_table disagree about the rows")
+    page_size = k_pages.shape[2]
+    for pg in (k_pages, v_pages):
+        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+            raise KernelError("attention_prefill: pages must be contiguous [pages, Hkv, page_size, dh] bfloat16")
+    lib = variant("attn_prefill", head_dim, _PREFILL_SIGNATURES)
+    check(
+        lib.tl_attn_prefill(
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            qo_indptr.data_ptr(), kv_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+            tile_row.data_ptr(), tile_q0.data_ptr(), tile_row.numel(), n_q_heads, n_kv_heads, head_dim, page_size,
+            window, float(scale), _stream(),
         ),
         lib,
         "tl_variant_last_error",
