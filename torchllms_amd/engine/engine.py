@@ -90,7 +90,7 @@ class Engine:
         from .graphs import DecodeGraphs
 
         graph_safe = all(getattr(b.mixer, "graph_safe", False) for b in self.model.blocks)
-        self.graphs = DecodeGraphs(self) if (use_graphs and graph_safe) else None
+        self.graphs = DecodeGraphs(self.model, self.cache, self.device, page_size) if (use_graphs and graph_safe) else None
 
     # ------------------------------------------------------------------ construction
     @classmethod

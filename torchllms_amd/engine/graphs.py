@@ -15,6 +15,7 @@ kernels only.
 
 from __future__ import annotations
 
+import gc
 from typing import Dict, Tuple
 
 import torch
@@ -33,16 +34,21 @@ def context_cap(max_kv_len: int) -> int:
 
 
 class DecodeGraph:
-    def __init__(self, engine, layout: StepLayout, cap: int):
-        self.engine = engine
+    """One recorded decode step.  It refers to the model and the cache, never to the engine that
+    owns it: a reference cycle would leave the graph to the cyclic garbage collector, which may
+    run, and destroy the graph, in the middle of somebody else's stream capture."""
+
+    def __init__(self, model, cache, device, page_size: int, layout: StepLayout, cap: int):
+        self.model = model
+        self.cache = cache
         self.cap = cap
-        width = -(-cap // engine.page_size)
+        width = -(-cap // page_size)
         n_groups = len(layout.block_tables)
         self.shapes = section_shapes(layout.n_tokens, layout.n_seqs, layout.logit_rows.size, [width] * n_groups)
         self.offsets, total = section_offsets(self.shapes)
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
         self.host_np = self.host.numpy()
-        self.dev = torch.zeros(total, dtype=torch.int32, device=engine.device)
+        self.dev = torch.zeros(total, dtype=torch.int32, device=device)
         self.copied = torch.cuda.Event()
         self.graph = None
         self.logits = None
@@ -59,12 +65,21 @@ class DecodeGraph:
         """Run the step eagerly (this is the step's real execution), then record the same launches."""
         self._load(layout)
         ctx = make_context(layout, self.dev, self.shapes, self.offsets, decode_longest=self.cap)
-        logits = self.engine.model.forward(ctx, self.engine.cache)
+        logits = self.model.forward(ctx, self.cache)
         result = logits.clone()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            self.logits = self.engine.model.forward(ctx, self.engine.cache)
+        # nothing may be destroyed while the stream is capturing: collect garbage now and keep the
+        # collector off until the capture has ended
+        gc.collect()
+        gc_was_on = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                self.logits = self.model.forward(ctx, self.cache)
+        finally:
+            if gc_was_on:
+                gc.enable()
         self.graph = graph
         self.ctx = ctx
         return result
@@ -79,8 +94,11 @@ class DecodeGraph:
 class DecodeGraphs:
     """The engine's recorded decode steps, by (requests, wanted rows, context cap)."""
 
-    def __init__(self, engine, max_graphs: int = 32):
-        self.engine = engine
+    def __init__(self, model, cache, device, page_size: int, max_graphs: int = 32):
+        self.model = model
+        self.cache = cache
+        self.device = device
+        self.page_size = page_size
         self.max_graphs = max_graphs
         self.graphs: Dict[Tuple[int, int, int], DecodeGraph] = {}
 
@@ -91,7 +109,7 @@ class DecodeGraphs:
         if g is None:
             if len(self.graphs) >= self.max_graphs:
                 self.graphs.pop(next(iter(self.graphs)))
-            g = DecodeGraph(self.engine, layout, cap)
+            g = DecodeGraph(self.model, self.cache, self.device, self.page_size, layout, cap)
             self.graphs[key] = g
             return g.first_run(layout)
         return g.replay(layout)
