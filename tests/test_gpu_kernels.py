@@ -540,7 +540,8 @@ def test_attention_decode_says_what_it_takes():
     assert not ops.decode_attention_supported(torch.bfloat16, 6, 3, 48)
     assert not ops.decode_attention_supported(torch.bfloat16, 16, 1, 256)
     assert ops.plan_decode_splits(8, 8, 8192) == (512, 16)
-    assert ops.plan_decode_splits(64, 8, 40) == (64, 1)
+    assert ops.plan_decode_splits(64, 8, 40) == (256, 1)
+    assert ops.plan_decode_splits(1, 8, 8192) == (256, 32)
 
 
 # ----------------------------------------------------------------------------- skinny matrix product (decode)

@@ -1,5 +1,6 @@
 // Attention of single new tokens over their requests' paged bfloat16 keys and values: the decode
-// kernel.  The work is reading the cache, so the design goal is to keep many wide loads in flight:
+// kernel.  The work is reading the cache, so the design goal is to keep many wide loads in flight
+// with few registers per wave (more resident waves = more bytes in flight):
 //
 //   * grid (split, kv head, token): the keys of one (token, kv head) are cut into splits of
 //     `split_size` keys so that a small batch still fills 256 CUs; a second kernel merges the
@@ -8,13 +9,16 @@
 //     that share the kv head are handled together, so keys and values are read once for the group.
 //   * scores: S^T[16 keys x 16 heads] by MFMA 16x16x16 bf16, A = the key rows exactly as they lie
 //     in the page (each lane loads 16-byte pieces of one row), B = the queries, kept in registers.
-//   * softmax statistics in 32-bit on the MFMA's output layout; the probabilities cross to the
-//     value layout through a small per-wave LDS buffer.
-//   * values: each lane loads 16 bytes (8 channels) of a value row; P.V accumulates in 32-bit
-//     registers on the vector ALU, which has time to spare while the loads stream.
+//   * softmax statistics in 32-bit on the MFMA's output layout.  That layout (lane = head, four
+//     consecutive keys) is also the B operand layout of P^T, so the probabilities go to the second
+//     product without leaving their lane.
+//   * values: O^T[channels x heads] = V^T . P^T by MFMA.  A lane loads, from each of its four key
+//     rows, the DH/16 consecutive channels  (DH/16) * n16 ...; the A operand of output block b is
+//     channel b of the four rows (two byte permutes).  Output block b, row m is therefore channel
+//     (DH/16) * m + b: a fixed renaming that the final store undoes.
 //
-// Compiled once per head size (-DTL_HEAD_DIM=32|64|128|256); the number of query heads per kv head
-// (1..16) is a template parameter rounded up to a power of two.
+// Compiled once per head size (-DTL_HEAD_DIM=32|64|128|256); any number 1..16 of query heads per kv
+// head runs through the same kernel (unused MFMA columns compute on zero queries).
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -41,17 +45,20 @@ static_assert(DH == 32 || DH == 64 || DH == 128 || DH == 256, "decode kernel: he
 
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kTile = 16;             // keys per tile = MFMA M
 #ifndef TL_DECODE_WAVES
 #define TL_DECODE_WAVES 4
 #endif
+#ifndef TL_DECODE_MIN_WAVES
+#define TL_DECODE_MIN_WAVES (TL_HEAD_DIM <= 128 ? 4 : 2)  // blocks per CU the register budget is cut for
+#endif
 constexpr int kWaves = TL_DECODE_WAVES;
 constexpr int kKLoads = DH / 32;      // 16-byte loads a lane makes of its key row
-constexpr int kLPR = DH / 8;          // lanes that cover one value row with 16-byte loads
-constexpr int kRPI = kWave / kLPR;    // value rows one load instruction covers
-constexpr int kVLoads = kTile / kRPI; // load instructions per tile of values
-static_assert(kRPI <= kTile, "head size too small for this layout");
+constexpr int kE = DH / 16;           // channels of a value row that one lane owns = output blocks
+constexpr int kVDwords = kE / 2;      // 32-bit words a lane loads from one value row
 
 struct DecodeArgs {
   const bf16_t* q;
@@ -76,19 +83,39 @@ struct DecodeArgs {
   float* ws_ml;  // [token][q head][split][2] = running maximum (log2 domain), sum
 };
 
-union Pack16 {
-  uint4 u;
-  short4_t s[2];
-  uint16_t h[8];
+struct Pack16 {
+  u32x4_t u;
+  __device__ __forceinline__ short4_t half(int e) const {
+    return __builtin_bit_cast(short4_t, e == 0 ? u32x2_t{u[0], u[1]} : u32x2_t{u[2], u[3]});
+  }
 };
 
-__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ uint32_t bf16_bits(float x) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x));
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) { return bf16_bits(a) | (bf16_bits(b) << 16); }
 
-template <int RP>
-__global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a) {
-  __shared__ float p_lds[kWaves][kTile][RP];            // probabilities of the wave's current tile
-  __shared__ float red_o[kWaves][RP][DH];               // per-wave partial outputs for the block merge
-  __shared__ float red_m[kWaves][RP], red_l[kWaves][RP];
+// kVDwords consecutive 32-bit words from a pointer aligned to their total size
+__device__ __forceinline__ void load_value_words(const bf16_t* src, uint32_t* dst) {
+  if constexpr (kVDwords == 1) {
+    dst[0] = *reinterpret_cast<const uint32_t*>(src);
+  } else if constexpr (kVDwords == 2) {
+    const u32x2_t v = *reinterpret_cast<const u32x2_t*>(src);
+    dst[0] = v[0];
+    dst[1] = v[1];
+  } else {
+#pragma unroll
+    for (int i = 0; i < kVDwords / 4; ++i) {
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + 8 * i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[4 * i + e] = v[e];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decode_kernel(DecodeArgs a) {
+  extern __shared__ float red_o[];  // [kWaves][group][DH]: per-wave partial outputs for the block merge
+  __shared__ float red_m[kWaves][16], red_l[kWaves][16];
 
   const int split = blockIdx.x;
   const int kvh = blockIdx.y;
@@ -115,21 +142,16 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
     const bf16_t* qrow = a.q + (size_t)t * a.q_stride + ((size_t)kvh * R + (n16 < R ? n16 : 0)) * DH;
 #pragma unroll
     for (int u = 0; u < kKLoads; ++u) {
-      qreg[u].u = *reinterpret_cast<const uint4*>(qrow + 32 * u + 8 * g4);
-      if (n16 >= R) qreg[u].u = make_uint4(0, 0, 0, 0);
+      qreg[u].u = *reinterpret_cast<const u32x4_t*>(qrow + 32 * u + 8 * g4);
+      if (n16 >= R) qreg[u].u = u32x4_t{0, 0, 0, 0};
     }
   }
 
   float m_run = -INFINITY;  // running maximum of head n16 (same in the four g4 lanes)
   float l_part = 0.f;       // sum of this lane's own probabilities
-  float acc[RP][8];
+  float4_t acc[kE];         // acc[b][i]: head n16, channel kE * (4 g4 + i) + b
 #pragma unroll
-  for (int h = 0; h < RP; ++h)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
-
-  const int vrow = lane / kLPR;
-  const int dchunk = lane % kLPR;
+  for (int e = 0; e < kE; ++e) acc[e] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   auto clamp_key = [&](int key) { return key < lo ? lo : (key > p ? p : key); };
   auto row_ptr = [&](const bf16_t* pages, int key) {
@@ -139,27 +161,28 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
   };
 
   // Rolling prefetch: the keys of tile t+1 are requested as soon as the MFMAs of tile t have read
-  // their registers, the values of tile t+1 as soon as P.V of tile t is done, so one set of
-  // registers per operand keeps a load in flight at all times.
+  // their registers, the values of tile t+1 as soon as the value operands of tile t are packed, so
+  // one set of registers per operand keeps a load in flight at all times.  The prefetches are not
+  // put under a branch (a conditional load makes the compiler's wait before the next use cover both
+  // paths and so wait for the prefetch itself); past the end of the split they read clamped keys
+  // that nobody uses.
   Pack16 kreg[kKLoads];
-  Pack16 vreg[kVLoads];
-  auto load_k = [&](int base, Pack16* kd) {
+  uint32_t vreg[4][kVDwords];
+  auto load_k = [&](int base) {
     const bf16_t* kr = row_ptr(a.k_pages, clamp_key(base + n16));
 #pragma unroll
-    for (int u = 0; u < kKLoads; ++u) kd[u].u = *reinterpret_cast<const uint4*>(kr + 32 * u + 8 * g4);
+    for (int u = 0; u < kKLoads; ++u) kreg[u].u = *reinterpret_cast<const u32x4_t*>(kr + 32 * u + 8 * g4);
   };
-  auto load_v = [&](int base, Pack16* vd) {
+  auto load_v = [&](int base) {
 #pragma unroll
-    for (int j = 0; j < kVLoads; ++j) {
-      const bf16_t* vr = row_ptr(a.v_pages, clamp_key(base + j * kRPI + vrow));
-      vd[j].u = *reinterpret_cast<const uint4*>(vr + 8 * dchunk);
-    }
+    for (int j = 0; j < 4; ++j)
+      load_value_words(row_ptr(a.v_pages, clamp_key(base + 4 * g4 + j)) + kE * n16, vreg[j]);
   };
 
   int base = split_begin + wave * kTile;
   if (base <= split_end) {
-    load_k(base, kreg);
-    load_v(base, vreg);
+    load_k(base);
+    load_v(base);
   }
   for (; base <= split_end; base += kWaves * kTile) {
     const int next = base + kWaves * kTile;
@@ -168,10 +191,10 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
     float4_t c = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int u = 0; u < kKLoads; ++u) {
-      c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].s[0], qreg[u].s[0], c, 0, 0, 0);
-      c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].s[1], qreg[u].s[1], c, 0, 0, 0);
+      c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].half(0), qreg[u].half(0), c, 0, 0, 0);
+      c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].half(1), qreg[u].half(1), c, 0, 0, 0);
     }
-    if (next <= split_end) load_k(next, kreg);
+    load_k(next);  // unconditional: past the split's end the keys are clamped and unused
     float s[4];
     float tmax = -INFINITY;
 #pragma unroll
@@ -192,62 +215,33 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
       l_part = (i == 0 ? l_part * alpha : l_part) + pr[i];
     }
     m_run = m_new;
+    const short4_t pop = __builtin_bit_cast(short4_t, u32x2_t{pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3])});
 
-    // probabilities and the rescale factor go to the value layout through LDS (per wave)
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    if (n16 < RP) {
+    // O^T += V^T . P^T, block by block of 16 channels
 #pragma unroll
-      for (int i = 0; i < 4; ++i) p_lds[wave][4 * g4 + i][n16] = pr[i];
+    for (int e = 0; e < kE; ++e) {
+      const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;  // the odd or the even halves of two words
+      const uint32_t lo2 = __builtin_amdgcn_perm(vreg[1][e / 2], vreg[0][e / 2], sel);
+      const uint32_t hi2 = __builtin_amdgcn_perm(vreg[3][e / 2], vreg[2][e / 2], sel);
+      const short4_t vop = __builtin_bit_cast(short4_t, u32x2_t{lo2, hi2});
+      acc[e] = acc[e] * alpha;
+      acc[e] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop, pop, acc[e], 0, 0, 0);
     }
-    // alpha of head h sits in lanes n16 == h; every lane needs all of them
-    float alpha_h[RP];
-#pragma unroll
-    for (int h = 0; h < RP; ++h) alpha_h[h] = __shfl(alpha, h, kWave);
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-
-#pragma unroll
-    for (int h = 0; h < RP; ++h)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[h][e] *= alpha_h[h];
-#pragma unroll
-    for (int j = 0; j < kVLoads; ++j) {
-      const int kt = j * kRPI + vrow;  // key within the tile
-      float vf[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) vf[e] = bf16_bits_to_f32(vreg[j].h[e]);
-#pragma unroll
-      for (int h = 0; h < RP; ++h) {
-        const float ph = p_lds[wave][kt][h];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] = fmaf(ph, vf[e], acc[h][e]);
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-
-    if (next <= split_end) load_v(next, vreg);
+    load_v(next);
   }
 
-  // wave-level reductions: sums over the four row groups; outputs over the value-row lanes
+  // the lane's own sums join over the four row groups
   l_part += __shfl_xor(l_part, 16, kWave);
   l_part += __shfl_xor(l_part, 32, kWave);
-#pragma unroll
-  for (int off = kLPR; off < kWave; off <<= 1)
-#pragma unroll
-    for (int h = 0; h < RP; ++h)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) acc[h][e] += __shfl_xor(acc[h][e], off, kWave);
-
-  if (lane < 16 && n16 < RP) {
+  if (lane < 16) {
     red_m[wave][n16] = m_run;
     red_l[wave][n16] = l_part;
   }
-  if (vrow == 0) {
+  if (n16 < R) {
 #pragma unroll
-    for (int h = 0; h < RP; ++h)
+    for (int e = 0; e < kE; ++e)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) red_o[wave][h][8 * dchunk + e] = acc[h][e];
+      for (int i = 0; i < 4; ++i) red_o[((size_t)wave * R + n16) * DH + kE * (4 * g4 + i) + e] = acc[e][i];
   }
   __syncthreads();
 
@@ -263,7 +257,7 @@ __global__ void __launch_bounds__(kWaves* kWave) attn_decode_kernel(DecodeArgs a
     for (int w = 0; w < kWaves; ++w) {
       const float f = red_m[w][h] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(red_m[w][h] - M);
       L += red_l[w][h] * f;
-      O += red_o[w][h][d] * f;
+      O += red_o[((size_t)w * R + h) * DH + d] * f;
     }
     const int qh = kvh * R + h;
     if (a.n_splits == 1) {
@@ -353,7 +347,7 @@ TL_EXPORT int tl_attn_decode(const void* q, int q_stride, void* out, int out_str
     return variant_fail(TL_ERR_ARG, "attn_decode: bad sizes");
   if (n_q_heads % n_kv_heads) return variant_fail(TL_ERR_ARG, "attn_decode: %d query heads are not a multiple of %d kv heads", n_q_heads, n_kv_heads);
   const int R = n_q_heads / n_kv_heads;
-  constexpr int kMaxGroup = DH <= 128 ? 16 : 8;  // bounded by the block's LDS
+  constexpr int kMaxGroup = DH <= 128 ? 16 : 8;  // bounded by the block's LDS (64 KB of partial outputs)
   if (R > kMaxGroup) return variant_fail(TL_ERR_UNSUPPORTED, "attn_decode: %d query heads per kv head exceed %d at head_dim %d", R, kMaxGroup, DH);
   if (split_size <= 0 || split_size % (kWaves * kTile)) return variant_fail(TL_ERR_ARG, "attn_decode: split_size=%d must be a positive multiple of %d", split_size, kWaves * kTile);
   if (n_splits <= 0 || n_splits > 65535 || n_kv_heads > 65535 || n_tokens > 65535) return variant_fail(TL_ERR_ARG, "attn_decode: grid out of range");
@@ -372,11 +366,8 @@ TL_EXPORT int tl_attn_decode(const void* q, int q_stride, void* out, int out_str
   a.split_size = split_size; a.n_splits = n_splits; a.ws_o = ws_o; a.ws_ml = ws_ml;
   dim3 grid(n_splits, n_kv_heads, n_tokens);
   const int threads = kWaves * kWave;
-  if (R == 1) attn_decode_kernel<1><<<grid, threads, 0, stream>>>(a);
-  else if (R == 2) attn_decode_kernel<2><<<grid, threads, 0, stream>>>(a);
-  else if (R <= 4) attn_decode_kernel<4><<<grid, threads, 0, stream>>>(a);
-  else if (R <= 8) attn_decode_kernel<8><<<grid, threads, 0, stream>>>(a);
-  else if constexpr (kMaxGroup >= 16) attn_decode_kernel<16><<<grid, threads, 0, stream>>>(a);
+  const size_t lds = (size_t)kWaves * R * DH * sizeof(float);
+  attn_decode_kernel<<<grid, threads, lds, stream>>>(a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return variant_fail(TL_ERR_HIP, "attn_decode: %s", hipGetErrorString(e));
   if (n_splits > 1) {

@@ -48,7 +48,8 @@ constexpr int KT = DH <= 128 ? 64 : 32;       // keys per LDS tile
 constexpr int KL = DH / 32;                  // 16-byte pieces of a key row per lane
 constexpr int DT = DH / 16;                  // channel tiles of the output
 constexpr int kKPitch = DH + 8;              // bf16 elements per key row in LDS
-constexpr int kVPitch = KT + 8;              // bf16 elements per channel row in LDS
+constexpr int kVPitch = KT + 2;              // bf16 elements per channel row in LDS: an odd number of
+                                             // dwords, so the transposed 16-bit writes spread over the banks
 constexpr int kChunksPerRow = DH / 8;        // 16-byte chunks in a key/value row
 constexpr int kLoadsPerThread = KT * kChunksPerRow / kThreads;
 static_assert(KT * kChunksPerRow % kThreads == 0, "tile does not divide over the block");
@@ -92,12 +93,12 @@ __device__ __forceinline__ uint32_t bf16_bits(float x) {
 __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) { return bf16_bits(a) | (bf16_bits(b) << 16); }
 
 template <int RP>
-__global__ void __launch_bounds__(kThreads) attn_prefill_kernel(PrefillArgs a) {
+__global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[KT * kKPitch];
   __shared__ __attribute__((aligned(16))) bf16_t vt_lds[DH * kVPitch];
   constexpr int QB = kCols / RP;  // queries per block
 
-  const int tile = blockIdx.x;
+  const int tile = gridDim.x - 1 - blockIdx.x;  // late query tiles see the most keys: start them first
   const int kvh = blockIdx.y;
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
@@ -201,63 +202,97 @@ __global__ void __launch_bounds__(kThreads) attn_prefill_kernel(PrefillArgs a) {
     __syncthreads();  // the previous tile has been read by every wave
     stash();
     __syncthreads();
-    if (base + KT <= key_hi) fetch(base + KT);  // in flight while this tile is computed
+    fetch(base + KT);  // in flight while this tile is computed; unconditional (keys are clamped), so
+                       // that no wait has to cover a path without it
 
     if (base > wave_hi || base + KT - 1 < wave_lo) continue;  // nothing here for this wave's columns
+
+    // the tile is worked off in chunks of 32 keys: scores, softmax bookkeeping, then P.V
+    constexpr int NS = 2;
 #pragma unroll
-    for (int sub = 0; sub < KT / 16; ++sub) {
-      const int kb = base + 16 * sub;
-      if (kb > wave_hi || kb + 15 < wave_lo) continue;
+    for (int chunk = 0; chunk < KT / (16 * NS); ++chunk) {
+    const int cbase = base + 16 * NS * chunk;
+    if (cbase > wave_hi || cbase + 16 * NS - 1 < wave_lo) continue;
+    // phase 1: scores S^T[key][column], one MFMA chain per (16 keys, column block)
+    float4_t c[NC][NS];
+    bool live[NS];
+#pragma unroll
+    for (int sub = 0; sub < NS; ++sub) {
+      const int kb = cbase + 16 * sub;
+      live[sub] = !(kb > wave_hi || kb + 15 < wave_lo);
+#pragma unroll
+      for (int i = 0; i < NC; ++i) c[i][sub] = float4_t{0.f, 0.f, 0.f, 0.f};
+      if (!live[sub]) continue;
       Pack16 ka[KL];
 #pragma unroll
       for (int u = 0; u < KL; ++u)
-        ka[u].u = *reinterpret_cast<const u32x4_t*>(&k_lds[(16 * sub + n16) * kKPitch + 32 * u + 8 * g4]);
-      short4_t pb[NC];
+        ka[u].u = *reinterpret_cast<const u32x4_t*>(&k_lds[(16 * (NS * chunk + sub) + n16) * kKPitch + 32 * u + 8 * g4]);
 #pragma unroll
-      for (int i = 0; i < NC; ++i) {
-        float4_t c = {0.f, 0.f, 0.f, 0.f};
+      for (int u = 0; u < KL; ++u)
 #pragma unroll
-        for (int u = 0; u < KL; ++u) {
-          c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[u].half(0), qreg[i][u].half(0), c, 0, 0, 0);
-          c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[u].half(1), qreg[i][u].half(1), c, 0, 0, 0);
+        for (int i = 0; i < NC; ++i) {
+          c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[u].half(0), qreg[i][u].half(0), c[i][sub], 0, 0, 0);
+          c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[u].half(1), qreg[i][u].half(1), c[i][sub], 0, 0, 0);
         }
-        float s[4];
-        float tmax = -INFINITY;
+    }
+    // softmax bookkeeping once per chunk and column: mask, maximum, rescale, probabilities.
+    // Scores stay unscaled; the scale enters through one fused multiply-add per element:
+    // exp2(s * scale - m), with m the running maximum of s * scale.
+    short4_t pb[NC][NS];
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      // keys of the chunk that every lane of this column sees need no test at all
+      const bool all_seen = live[0] && live[NS - 1] && cbase >= col_lo[i] && cbase + 16 * NS - 1 <= col_pos[i];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int key = kb + 4 * g4 + r;
-          const bool valid = key >= col_lo[i] && key <= col_pos[i];
-          s[r] = valid ? c[r] * a.scale_log2e : -INFINITY;
-          tmax = fmaxf(tmax, s[r]);
+          if (!all_seen) {
+            const int key = cbase + 16 * sub + 4 * g4 + r;
+            const bool valid = live[sub] && key >= col_lo[i] && key <= col_pos[i];
+            if (!valid) c[i][sub][r] = -INFINITY;
+          }
+          tmax = fmaxf(tmax, c[i][sub][r]);
         }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-        const float m_new = fmaxf(m_run[i], tmax);
-        // a column may not have met a visible key yet: then nothing is rescaled and nothing added
-        const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m_run[i] - m_new);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      const float m_new = fmaxf(m_run[i], tmax * a.scale_log2e);  // the scale is positive
+      // a column may not have met a visible key yet: then nothing is rescaled and nothing added
+      const bool none = m_new == -INFINITY;
+      const float alpha = none ? 1.f : __builtin_amdgcn_exp2f(m_run[i] - m_new);
+      const float neg_m = none ? 0.f : -m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int sub = 0; sub < NS; ++sub) {
         float pr[4];
-        float psum = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          pr[r] = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(s[r] - m_new);
+          pr[r] = __builtin_amdgcn_exp2f(fmaf(c[i][sub][r], a.scale_log2e, neg_m));  // exp2(-inf) = 0
           psum += pr[r];
         }
-        l_part[i] = l_part[i] * alpha + psum;
-        m_run[i] = m_new;
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha;
-        pb[i] = __builtin_bit_cast(short4_t, u32x2_t{pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3])});
+        pb[i][sub] = __builtin_bit_cast(short4_t, u32x2_t{pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3])});
       }
-      // O^T[channel][column] += V^T[channel][key] P^T[key][column]
+      l_part[i] = l_part[i] * alpha + psum;
+      m_run[i] = m_new;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha;
+    }
+    // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column]
+#pragma unroll
+    for (int sub = 0; sub < NS; ++sub) {
+      if (!live[sub]) continue;
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
-        const short4_t va = *reinterpret_cast<const short4_t*>(&vt_lds[(16 * t + n16) * kVPitch + 16 * sub + 4 * g4]);
+        const uint32_t* vp = reinterpret_cast<const uint32_t*>(&vt_lds[(16 * t + n16) * kVPitch + 16 * (NS * chunk + sub) + 4 * g4]);
+        const short4_t va = __builtin_bit_cast(short4_t, u32x2_t{vp[0], vp[1]});
 #pragma unroll
-        for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb[i], acc[i][t], 0, 0, 0);
+        for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb[i][sub], acc[i][t], 0, 0, 0);
       }
     }
+    }  // chunk
   }
 
 #pragma unroll

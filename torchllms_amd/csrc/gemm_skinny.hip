@@ -38,56 +38,36 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   const int g4 = lane / 16;
   const int n0 = blockIdx.x * kStrip;
 
-  // this wave's share of K, in whole steps
-  const int steps_total = (K + kStepK - 1) / kStepK;
-  const int steps_per_wave = (steps_total + WAVES - 1) / WAVES;
-  const int step_lo = wave * steps_per_wave;
-  const int step_hi = min(step_lo + steps_per_wave, steps_total);
+  // K is walked in steps of 128; the waves of the block share the whole steps between them and the
+  // last wave also takes the partial step at the end, if there is one
+  const int steps_full = K / kStepK;
+  const int steps_per_wave = (steps_full + WAVES - 1) / WAVES;
+  const int step_lo = min(wave * steps_per_wave, steps_full);
+  const int step_hi = min(step_lo + steps_per_wave, steps_full);
 
   const int wrow = min(n0 + n16, N - 1);  // rows past N are clamped; their results are not stored
   const bf16_t* wp = W + (size_t)wrow * ldw + 32 * g4;
+  // rows of A past M are read from row 0: they only feed output columns that are never stored
   const bf16_t* ap[MB];
-  bool arow_ok[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) {
     const int m = 16 * b + n16;
-    arow_ok[b] = m < M;
-    ap[b] = A + (size_t)(arow_ok[b] ? m : 0) * lda + 32 * g4;
+    ap[b] = A + (size_t)(m < M ? m : 0) * lda + 32 * g4;
   }
 
   float4_t acc[MB];
 #pragma unroll
   for (int b = 0; b < MB; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-  // Loads never branch: addresses past K are clamped into the row and the A side is zeroed by a
-  // mask, so out-of-range products vanish.  Two stages: the loads of step s+1 are issued before the
-  // MFMAs of step s.
-  const int kmax = K - 8;  // last 16-byte piece of a row
-  auto load_w = [&](int st, Pack16* w) {
-    const int k0 = st * kStepK + 32 * g4;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int k = min(k0 + 8 * u, kmax);
-      w[u].v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(wp - 32 * g4 + k));
-    }
-  };
-  auto load_a = [&](int st, int b, Pack16* a) {
-    const int k0 = st * kStepK + 32 * g4;
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int k = k0 + 8 * u;
-      const uint4 v = *reinterpret_cast<const uint4*>(ap[b] - 32 * g4 + min(k, kmax));
-      const uint32_t keep = (arow_ok[b] && k < K) ? 0xFFFFFFFFu : 0u;
-      a[u].u = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
-    }
-  };
-
-  Pack16 w0[4], w1[4];
-  Pack16 a0[MB][4], a1[MB][4];
+  // whole steps: plain loads, nothing between a load and its use but the other stage's MFMAs
   auto load = [&](int st, Pack16* w, Pack16 (*a)[4]) {
-    load_w(st, w);
+    const int k0 = st * kStepK;
 #pragma unroll
-    for (int b = 0; b < MB; ++b) load_a(st, b, a[b]);
+    for (int u = 0; u < 4; ++u) w[u].v = *reinterpret_cast<const u32x4_t*>(wp + k0 + 8 * u);
+#pragma unroll
+    for (int b = 0; b < MB; ++b)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) a[b][u].v = *reinterpret_cast<const u32x4_t*>(ap[b] + k0 + 8 * u);
   };
   auto mma = [&](const Pack16* w, const Pack16 (*a)[4]) {
 #pragma unroll
@@ -99,6 +79,8 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
       }
     }
   };
+  Pack16 w0[4], w1[4];
+  Pack16 a0[MB][4], a1[MB][4];
   // Rows of W lie a power of two apart, so blocks that walk K in step would all press on the same
   // memory channels at once; every block therefore starts its walk at a different step and wraps
   // around.  Two steps per trip so that both buffers are named statically (they stay in registers).
@@ -109,15 +91,37 @@ gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     if (s >= nst) s -= nst;
     return step_lo + s;
   };
-  int i = 0;
-  if (i < nst) load(step_of(i), w0, a0);
-  while (i < nst) {
-    if (i + 1 < nst) load(step_of(i + 1), w1, a1);
+  // The prefetches are unconditional (past the end they repeat the last step and are ignored): a
+  // load under a branch would make the wait before the MFMAs cover both paths, that is, wait for
+  // the prefetch itself.
+  if (nst > 0) {
+    load(step_of(0), w0, a0);
+    int i = 0;
+    for (; i + 1 < nst; i += 2) {  // two steps per trip, nothing conditional inside
+      load(step_of(i + 1), w1, a1);
+      mma(w0, a0);
+      load(step_of(min(i + 2, nst - 1)), w0, a0);
+      mma(w1, a1);
+    }
+    if (i < nst) mma(w0, a0);  // an odd number of steps: the last one is already loaded
+  }
+  // the partial step: addresses past K are clamped into the row and the A side is zeroed, so the
+  // out-of-range products vanish
+  if (wave == WAVES - 1 && steps_full * kStepK < K) {
+    const int kmax = K - 8;
+    const int k0 = steps_full * kStepK + 32 * g4;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 8 * u;
+      w0[u].v = *reinterpret_cast<const u32x4_t*>(wp - 32 * g4 + min(k, kmax));
+      const uint32_t keep = k < K ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(ap[b] - 32 * g4 + min(k, kmax));
+        a0[b][u].v = u32x4_t{v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
+      }
+    }
     mma(w0, a0);
-    if (i + 1 >= nst) break;
-    if (i + 2 < nst) load(step_of(i + 2), w0, a0);
-    mma(w1, a1);
-    i += 2;
   }
 
   // acc[b][i] = C^T[n0 + 4 g4 + i][16 b + n16]; add the waves' shares in wave order

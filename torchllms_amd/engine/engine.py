@@ -61,6 +61,7 @@ class Engine:
         max_model_len: Optional[int] = None,
         device="cuda:0",
         use_graphs: bool = True,
+        tune_kernels: bool = True,
     ):
         """``tensors``: the model's tensors under the parts' own names, on ``device``.
         Pool size: ``num_pages`` pages per group, else what ``kv_memory_gb`` holds, else room for
@@ -85,6 +86,12 @@ class Engine:
         self.cache = CacheManager(groups, states, page_size, num_pages, max_seqs, dtype=dtype, device=self.device)
         self.steps_run = 0
         self.tokens_run = 0
+        if dtype == torch.bfloat16 and tune_kernels:
+            # which matrix-product kernel serves decode steps best is measured, not guessed
+            from ..kernels import ops
+
+            for shape, group in self.model.linear_weights().items():
+                ops.tune_linear(group, torch.float32 if group[0] is self.model.head.weight else torch.bfloat16)
         # decode steps are replayed from HIP graphs when every mixer's launches are fixed by the
         # step's shape alone
         from .graphs import DecodeGraphs

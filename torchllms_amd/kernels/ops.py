@@ -212,9 +212,8 @@ def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 
 SKINNY_MAX_ROWS = 16
-#: the weight-streaming kernel is used for matrices up to this many elements; measured on MI355X, the
-#: BLAS library's kernels stream larger matrices faster (3.9-5.8 TB/s against 2.7-3.3 TB/s), while on
-#: smaller ones (4096 x 4096: 13 us against 20 us) its launch and tail costs make it the slower one
+#: shapes that were never measured (see ``tune_linear``) use the weight-streaming kernel up to this
+#: many elements: small matrices are where the library's launch and tail costs weigh most
 SKINNY_MAX_ELEMENTS = 1 << 24
 
 
@@ -239,23 +238,75 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
 
 
 def skinny_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the weight-streaming kernel can take this product at all."""
     return (
-        x.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
-        and w.shape[0] * w.shape[1] <= SKINNY_MAX_ELEMENTS
+        x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
         and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
     )
 
 
+#: measured choice between the two bfloat16 kernels: (n, k, row bucket) -> True (weight-streaming
+#: kernel) / False (library).  Filled by ``tune_linear``; shapes never measured follow the size rule.
+_LINEAR_CHOICE: dict = {}
+ROW_BUCKETS = (1, 2, 4, 8, 16)
+
+
+def _row_bucket(m: int) -> int:
+    for b in ROW_BUCKETS:
+        if m <= b:
+            return b
+    return ROW_BUCKETS[-1]
+
+
+def use_skinny(x: torch.Tensor, w: torch.Tensor) -> bool:
+    if not skinny_supported(x, w):
+        return False
+    choice = _LINEAR_CHOICE.get((w.shape[0], w.shape[1], _row_bucket(x.shape[0])))
+    if choice is None:
+        return w.shape[0] * w.shape[1] <= SKINNY_MAX_ELEMENTS
+    return choice
+
+
+def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, iters: int = 6) -> None:
+    """Measure, for matrices of one shape and every row bucket, which bfloat16 kernel is faster on
+    this GPU, and remember it.  ``weights``: the model's tensors of that shape; timing rotates over
+    them, as a decode step does, so that no run is served from cache.  Shapes already measured are
+    left alone, so every engine of a process makes the same choice."""
+    weights = [w for w in weights if w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2]
+    if not weights:
+        return
+    n, k = weights[0].shape
+    if k % 8 or weights[0].stride(0) % 8:
+        return
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for bucket in ROW_BUCKETS:
+        if (n, k, bucket) in _LINEAR_CHOICE:
+            continue
+        x = torch.randn((bucket, k), device=weights[0].device, dtype=torch.float32).to(torch.bfloat16)
+        times = []
+        for fn in (lambda w: gemm_skinny(x, w, out_dtype), lambda w: torch.nn.functional.linear(x, w)):
+            for i in range(2):
+                fn(weights[i % len(weights)])
+            start.record()
+            for i in range(iters):
+                fn(weights[(i + 2) % len(weights)])
+            stop.record()
+            stop.synchronize()
+            times.append(start.elapsed_time(stop))
+        _LINEAR_CHOICE[(n, k, bucket)] = times[0] <= times[1]
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16: the weight-streaming MFMA kernel for
-    few rows and small matrices (see ``SKINNY_MAX_ELEMENTS``), else the BLAS library's matrix
-    product, as the reference uses its library's (torchllms/models/networks.py:474-493).
-    ``out_dtype`` float32 asks for 32-bit results from bfloat16 inputs (logits)."""
+    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16: for up to 16 rows (decode steps)
+    the weight-streaming MFMA kernel or the BLAS library's matrix product, whichever was measured
+    faster for the shape (``tune_linear``); for more rows the library, as the reference uses its
+    library's (torchllms/models/networks.py:474-493).  ``out_dtype`` float32 asks for 32-bit
+    results from bfloat16 inputs (logits)."""
     if x.dtype == torch.float32:
         return gemm_f32(x, w)
     _gpu(x, w)
     out_dtype = out_dtype or x.dtype
-    if skinny_supported(x, w):
+    if use_skinny(x, w):
         return gemm_skinny(x, w, out_dtype)
     y = torch.nn.functional.linear(x, w)
     return y if y.dtype == out_dtype else y.to(out_dtype)
@@ -315,13 +366,17 @@ def decode_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: i
     return n_q_heads // n_kv_heads <= (16 if head_dim <= 128 else 8)
 
 
+_DECODE_MIN_SPLIT = 256  # keys: shorter splits cost more in launch and merge than they gain in spread
+
+
 def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, target_blocks: int = 1024):
     """``(split_size, n_splits)`` for a decode launch whose longest visible key range (counted from
-    its 16-aligned start) is ``longest``: enough splits to fill the GPU, none shorter than 64 keys."""
+    its 16-aligned start) is ``longest``: enough splits for about four blocks on each of the 256
+    CUs (what the kernel's registers allow to be resident), none shorter than 256 keys."""
     pairs = max(n_tokens * n_kv_heads, 1)
     want = max(-(-target_blocks // pairs), 1)
     split = -(-max(longest, 1) // want)
-    split = max(-(-split // _DECODE_BLOCK_KEYS) * _DECODE_BLOCK_KEYS, _DECODE_BLOCK_KEYS)
+    split = max(-(-split // _DECODE_BLOCK_KEYS) * _DECODE_BLOCK_KEYS, _DECODE_MIN_SPLIT)
     return split, max(-(-max(longest, 1) // split), 1)
 
 

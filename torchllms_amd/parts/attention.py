@@ -81,6 +81,9 @@ class Attention(Mixer):
         self.wo = tensors["wo.weight"].contiguous()
         self.position.to(self.wo.device)
 
+    def linear_weights(self):
+        return [self.wqkv, self.wo]
+
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         n_kv_in_row = 0 if self.shares_kv else self.num_kv_heads
         qkv = ops.linear(x, self.wqkv)

@@ -73,6 +73,10 @@ class Part:
         if tensors:
             raise ValueError(f"{type(self).__name__} takes no tensors, got {sorted(tensors)}")
 
+    def linear_weights(self):
+        """The matrices this part multiplies activations with (for kernel selection by measurement)."""
+        return []
+
 
 class Norm(Part):
     """y = norm(x).  ``forward_add`` fuses the residual sum that precedes the norm."""

@@ -52,5 +52,8 @@ class LMHead(Head):
     def tie(self, embedding: TokenEmbedding) -> None:
         self.weight = embedding.weight
 
+    def linear_weights(self):
+        return [self.weight]
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.linear(x, self.weight, out_dtype=torch.float32)

@@ -30,6 +30,9 @@ class SwiGLU(FeedForward):
         self.w13 = torch.cat([tensors["w1.weight"], tensors["w3.weight"]], dim=0).contiguous()
         self.w2 = tensors["w2.weight"].contiguous()
 
+    def linear_weights(self):
+        return [self.w13, self.w2]
+
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
         gate_up = ops.linear(x, self.w13)
         return ops.linear(ops.silu_mul(gate_up), self.w2)

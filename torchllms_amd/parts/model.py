@@ -79,6 +79,18 @@ class Model:
         self.dtype = emb.dtype
         self.device = emb.device
 
+    def linear_weights(self):
+        """All matrices of the model, grouped by shape."""
+        groups = {}
+        parts = [self.head]
+        for b in self.blocks:
+            parts += [b.mixer, b.feed_forward]
+        for part in parts:
+            for w in part.linear_weights():
+                if w is not None:
+                    groups.setdefault(tuple(w.shape), []).append(w)
+        return groups
+
     # ------------------------------------------------------------------ cache
     def cache_needs(self) -> List[Tuple[int, object]]:
         """``(run id, need)`` for every run that owns a cache entry."""
