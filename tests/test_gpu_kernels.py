@@ -544,46 +544,67 @@ def test_attention_decode_says_what_it_takes():
     assert ops.plan_decode_splits(1, 8, 8192) == (256, 32)
 
 
-# ----------------------------------------------------------------------------- skinny matrix product (decode)
+# ----------------------------------------------------------------------------- weight-streaming matrix product (decode)
 @pytest.mark.parametrize(
     "m, n, k",
     [(1, 4096, 4096), (8, 6144, 4096), (8, 4096, 14336), (16, 1000, 256), (16, 300, 96), (9, 257, 688), (13, 2048, 1024),
-     (3, 16, 8), (5, 31, 136), (16, 128256 // 8, 512)],
+     (3, 16, 8), (5, 31, 136), (4, 40, 128), (16, 128256 // 8, 512)],
 )
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
-def test_gemm_skinny(m, n, k, out_dtype):
+def test_gemm_stream(m, n, k, out_dtype):
+    """The coalesced-fetch kernel: every row count's fetch groups, K with and without a partial
+    step, N that is no multiple of 16, every split of K."""
     torch.manual_seed(0)
     x = torch.randn(m, k).bfloat16()
     w = (torch.randn(n, k) * 0.05).bfloat16()
-    got = _ops().gemm_skinny(x.to(DEV), w.to(DEV), out_dtype).float().cpu()
     want = x.double() @ w.double().T
     tol = (1e-4 if out_dtype == torch.float32 else 2 ** -8) * want.abs().max().item() + 1e-5
-    assert (got.double() - want).abs().max().item() <= tol
-    for waves in (1, 2, 4, 8):
-        alt = _ops().gemm_skinny(x.to(DEV), w.to(DEV), out_dtype, waves=waves).float().cpu()
-        assert (alt.double() - want).abs().max().item() <= tol, f"waves={waves}"
+    for waves in (0, 1, 2, 4, 8):
+        got = _ops().gemm_stream(x.to(DEV), w.to(DEV), out_dtype, waves=waves).float().cpu()
+        assert (got.double() - want).abs().max().item() <= tol, f"waves={waves}"
 
 
-def test_gemm_skinny_rows_in_a_wider_buffer_and_limits():
+def test_gemm_stream_takes_strided_rows_and_says_its_limits():
     from torchllms_amd.kernels.lib import KernelError
 
     torch.manual_seed(0)
     wide = torch.randn(6, 512).bfloat16().to(DEV)
     x = wide[:, :256]  # row stride 512
     w = torch.randn(40, 256).bfloat16().to(DEV)
+    got = _ops().gemm_stream(x, w).float().cpu()
+    torch.testing.assert_close(got, (x.float() @ w.float().T).cpu(), rtol=2 ** -7, atol=0.1)
+    with pytest.raises(KernelError, match="exceeds 16"):
+        _ops().gemm_stream(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
+    with pytest.raises(KernelError, match="multiple of 8"):
+        _ops().gemm_stream(torch.zeros(2, 12, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV))
+
+
+def test_linear_sends_what_the_streaming_kernel_does_not_take_to_the_library():
+    torch.manual_seed(0)
+    wide = torch.randn(6, 512).bfloat16().to(DEV)
+    x = wide[:, :256]  # row stride 512
+    w = torch.randn(40, 256).bfloat16().to(DEV)
     got = _ops().linear(x, w).float().cpu()
     torch.testing.assert_close(got, (x.float() @ w.float().T).cpu(), rtol=2 ** -7, atol=0.1)
-    with pytest.raises(KernelError, match="exceeds 64"):
-        _ops().gemm_skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
-    many = _ops().gemm_skinny(torch.ones(40, 64, dtype=torch.bfloat16, device=DEV), torch.ones(24, 64, dtype=torch.bfloat16, device=DEV))
-    assert many.float().cpu().tolist() == [[64.0] * 24] * 40  # up to 64 rows through four column blocks
-    with pytest.raises(KernelError, match="multiple of 8"):
-        _ops().gemm_skinny(torch.zeros(2, 12, dtype=torch.bfloat16, device=DEV), torch.zeros(4, 12, dtype=torch.bfloat16, device=DEV))
-    # sizes the kernel does not take go to the library
     odd = _ops().linear(torch.ones(2, 12, dtype=torch.bfloat16, device=DEV), torch.ones(4, 12, dtype=torch.bfloat16, device=DEV))
     assert odd.float().cpu().tolist() == [[12.0] * 4] * 2
     big = _ops().linear(torch.ones(70, 16, dtype=torch.bfloat16, device=DEV), torch.ones(4, 16, dtype=torch.bfloat16, device=DEV), out_dtype=torch.float32)
     assert big.dtype == torch.float32 and big.shape == (70, 4)
+    assert big.cpu().tolist() == [[16.0] * 4] * 70
+
+
+def test_tune_linear_remembers_a_choice_for_every_row_bucket():
+    ops = _ops()
+    torch.manual_seed(0)
+    weights = [torch.randn(48, 64, device=DEV).bfloat16() for _ in range(2)]
+    for key in [k for k in ops._LINEAR_CHOICE if k[:2] == (48, 64)]:
+        del ops._LINEAR_CHOICE[key]
+    ops.tune_linear(weights)
+    for bucket in ops.ROW_BUCKETS:
+        assert ops._LINEAR_CHOICE[(48, 64, bucket)] in (None,) + tuple(ops.STREAM_WAVE_CHOICES)
+    x = torch.randn(5, 64, device=DEV).bfloat16()
+    got = ops.linear(x, weights[0]).float().cpu()
+    torch.testing.assert_close(got, (x.float() @ weights[0].float().T).cpu(), rtol=2 ** -7, atol=0.1)
 
 
 # ----------------------------------------------------------------------------- prefill attention (MFMA)

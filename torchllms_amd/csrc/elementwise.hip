@@ -227,7 +227,8 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_k
   const bool store = k_pages != nullptr && slot >= 0;
 
   // queries and keys: a thread owns one pair index and walks over heads, so the angle's cosine and
-  // sine are formed once per (token, pair)
+  // sine are formed once per (token, pair) and block; with few tokens the heads are spread over
+  // gridDim.y blocks so that the launch still fills the GPU
   const int n_rot_heads = n_q_heads + n_kv_heads;
   const int lanes_per_head = half;                       // threads that cover the pairs of one head
   const int head_groups = blockDim.x / lanes_per_head > 0 ? blockDim.x / lanes_per_head : 1;
@@ -253,7 +254,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_k
       i0 = rotary_dim + 2 * (i - rot_half);
       i1 = i0 + 1;
     }
-    for (int h = hgrp; h < n_rot_heads; h += head_groups) {
+    for (int h = hgrp + head_groups * blockIdx.y; h < n_rot_heads; h += head_groups * gridDim.y) {
       T* head = base + (size_t)h * head_dim;
       const float a0 = to_f32(head[i0]);
       const float a1 = to_f32(head[i1]);
@@ -276,7 +277,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_k
   // values
   if (store && v_pages != nullptr) {
     const T* vsrc = base + (size_t)(n_q_heads + n_kv_heads) * head_dim;
-    for (int w = threadIdx.x; w < n_kv_heads * head_dim; w += blockDim.x) {
+    for (int w = threadIdx.x + blockDim.x * blockIdx.y; w < n_kv_heads * head_dim; w += blockDim.x * gridDim.y) {
       const int kh = w / head_dim;
       const int d = w % head_dim;
       v_pages[(((size_t)page * n_kv_heads + kh) * page_size + off) * head_dim + d] = vsrc[w];
@@ -298,12 +299,18 @@ TL_EXPORT int tl_rope_kv_write(void* qkv, int n_tokens, int n_q_heads, int n_kv_
              "rope: pages given without slot_mapping/page_size");
   if (n_tokens == 0) return TL_OK;
   const int threads = 256;
+  // heads per block column: all of them when the tokens alone fill the GPU, one pass otherwise
+  const int head_groups = threads / (head_dim / 2) > 0 ? threads / (head_dim / 2) : 1;
+  const int passes = (n_q_heads + n_kv_heads + head_groups - 1) / head_groups;
+  int columns = 2048 / n_tokens;
+  columns = columns < 1 ? 1 : (columns > passes ? passes : columns);
+  const dim3 grid(n_tokens, columns);
   if (dtype == TL_F32)
-    rope_kv_write_kernel<float><<<n_tokens, threads, 0, stream>>>(
+    rope_kv_write_kernel<float><<<grid, threads, 0, stream>>>(
         (float*)qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, rotary_dim, pairing,
         (float*)k_pages, (float*)v_pages, slot_mapping, page_size);
   else if (dtype == TL_BF16)
-    rope_kv_write_kernel<bf16_t><<<n_tokens, threads, 0, stream>>>(
+    rope_kv_write_kernel<bf16_t><<<grid, threads, 0, stream>>>(
         (bf16_t*)qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, rotary_dim, pairing,
         (bf16_t*)k_pages, (bf16_t*)v_pages, slot_mapping, page_size);
   else
@@ -313,33 +320,48 @@ TL_EXPORT int tl_rope_kv_write(void* qkv, int n_tokens, int n_q_heads, int n_kv_
 
 // ----------------------------------------------------------------------------- SwiGLU gate
 // gate_up: [n, 2F] = gate | up.  out[n, F] = T(float(T(silu(gate))) * float(up)), silu(z) = z / (1 + e^-z).
-template <typename T>
+// A thread takes V consecutive columns of one row (V elements = 16 bytes when the row allows it).
+template <typename T, int V>
 __global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int n, int inter) {
-  const size_t total = (size_t)n * inter;
-  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (size_t)gridDim.x * blockDim.x) {
-    const size_t r = idx / inter;
-    const int c = (int)(idx % inter);
-    const float g = to_f32(gate_up[r * 2 * inter + c]);
-    const float u = to_f32(gate_up[r * 2 * inter + inter + c]);
-    const float act = to_f32(from_f32<T>(g / (1.0f + expf(-g))));
-    out[idx] = from_f32<T>(act * u);
+  const int c0 = (blockIdx.x * blockDim.x + threadIdx.x) * V;
+  if (c0 >= inter) return;
+  for (int r = blockIdx.y; r < n; r += gridDim.y) {
+    const T* gp = gate_up + (size_t)r * 2 * inter + c0;
+    T* op = out + (size_t)r * inter + c0;
+    struct alignas(sizeof(T) * V) Vec { T e[V]; };
+    const Vec g = *reinterpret_cast<const Vec*>(gp);
+    const Vec u = *reinterpret_cast<const Vec*>(gp + inter);
+    Vec o;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float gf = to_f32(g.e[i]);
+      const float act = to_f32(from_f32<T>(gf / (1.0f + expf(-gf))));
+      o.e[i] = from_f32<T>(act * to_f32(u.e[i]));
+    }
+    *reinterpret_cast<Vec*>(op) = o;
   }
+}
+
+template <typename T>
+int silu_mul_launch(const T* gate_up, T* out, int n, int inter, hipStream_t stream) {
+  constexpr int kVec = 16 / sizeof(T);
+  const bool wide = inter % kVec == 0 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  const int threads = 256;
+  const int per_block = threads * (wide ? kVec : 1);
+  const dim3 grid((inter + per_block - 1) / per_block, n < 65535 ? n : 65535);
+  if (wide)
+    silu_mul_kernel<T, kVec><<<grid, threads, 0, stream>>>(gate_up, out, n, inter);
+  else
+    silu_mul_kernel<T, 1><<<grid, threads, 0, stream>>>(gate_up, out, n, inter);
+  return tl_check_launch("silu_mul");
 }
 
 TL_EXPORT int tl_silu_mul(const void* gate_up, void* out, int n, int inter, int dtype, hipStream_t stream) {
   TL_REQUIRE(n >= 0 && inter > 0, "silu_mul: bad sizes n=%d inter=%d", n, inter);
   if (n == 0) return TL_OK;
-  const size_t total = (size_t)n * inter;
-  const int threads = 256;
-  const int blocks = (int)((total + threads - 1) / threads < 65536 ? (total + threads - 1) / threads : 65536);
-  if (dtype == TL_F32)
-    silu_mul_kernel<float><<<blocks, threads, 0, stream>>>((const float*)gate_up, (float*)out, n, inter);
-  else if (dtype == TL_BF16)
-    silu_mul_kernel<bf16_t><<<blocks, threads, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, n, inter);
-  else
-    return tl_fail(TL_ERR_ARG, "silu_mul: unknown dtype %d", dtype);
-  return tl_check_launch("silu_mul");
+  if (dtype == TL_F32) return silu_mul_launch((const float*)gate_up, (float*)out, n, inter, stream);
+  if (dtype == TL_BF16) return silu_mul_launch((const bf16_t*)gate_up, (bf16_t*)out, n, inter, stream);
+  return tl_fail(TL_ERR_ARG, "silu_mul: unknown dtype %d", dtype);
 }
 
 // ----------------------------------------------------------------------------- bias

@@ -1,0 +1,233 @@
+// C[M, N] = A[M, K] * W[N, K]^T for up to 16 rows, bfloat16 inputs, 32-bit accumulation: the matrix
+// products of decode steps, whose cost is reading W once from HBM.
+//
+// The vector memory path is bound by the cache lines an instruction touches, not by its bytes, so
+// W is fetched the coalesced way: one load instruction takes 4 rows x 256 contiguous bytes (8 cache
+// lines per KB; a load in the MFMA operand's own layout, 16 rows x 64 bytes, touches twice as many).
+// The MFMA wants the other layout (lane = row), so every wave passes its tile through a private
+// piece of LDS: written as loaded, read back as operands.  A wave's LDS instructions run in order,
+// so no barrier is needed, only fences that keep the compiler from reordering them.
+//
+//   * a block owns a strip of 16 output columns (16 rows of W); its waves split K between them and
+//     add their partial sums through LDS in a fixed order (no atomics).
+//   * C^T[16 columns x 16 rows of A] by MFMA 16x16x16 bf16: A operand = W, B operand = the rows of A,
+//     fetched and transposed the same way (only as many groups of four rows as M needs).
+//   * the LDS rows are 272 bytes apart: the 16 lanes that read one 16-byte piece of 16 different
+//     rows then fall on different banks.
+#include "common.h"
+
+namespace {
+
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kStrip = 16;    // output columns per block
+constexpr int kStepK = 128;   // k per wave step: 16 pieces of 8 elements
+constexpr int kPitch = 136;   // elements between LDS rows: 128 + 8 of padding (272 bytes)
+constexpr int kTileElems = 16 * kPitch;
+
+__device__ __forceinline__ short4_t lo_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[0], v[1]}); }
+__device__ __forceinline__ short4_t hi_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[2], v[3]}); }
+
+// MR: groups of four rows of A that are fetched (M <= 4 * MR).  WAVES: waves per block = splits of K.
+template <int MR, int WAVES, typename OutT>
+__global__ void __launch_bounds__(WAVES* kWave)
+gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
+                   OutT* __restrict__ C, int ldc, int M, int N, int K) {
+  // per wave: a tile of W [16][kPitch], then a tile of A [4 MR][kPitch] (rows past 4 MR are read as
+  // whatever the neighbour holds: they only feed output columns that are never stored)
+  extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
+  constexpr int kWaveElems = kTileElems + kTileElems;
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int n16 = lane % 16;  // operand layout: row
+  const int g4 = lane / 16;   // operand layout: piece within a group of four
+  const int q = lane / 16;    // fetch layout: row within a group of four
+  const int piece = lane % 16;  // fetch layout: 16-byte piece of the row's 256 bytes
+  const int n0 = blockIdx.x * kStrip;
+  bf16_t* w_lds = lds + (size_t)wave * kWaveElems;
+  bf16_t* a_lds = w_lds + kTileElems;
+
+  // K is walked in steps of 128; the waves of the block share the whole steps between them and the
+  // last wave also takes the partial step at the end, if there is one
+  const int steps_full = K / kStepK;
+  const int steps_per_wave = (steps_full + WAVES - 1) / WAVES;
+  const int step_lo = min(wave * steps_per_wave, steps_full);
+  const int step_hi = min(step_lo + steps_per_wave, steps_full);
+
+  // rows of W past N are clamped, rows of A past M read row 0: neither result is stored
+  const bf16_t* wsrc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) wsrc[j] = W + (size_t)min(n0 + 4 * j + q, N - 1) * ldw + 8 * piece;
+  const bf16_t* asrc[MR];
+#pragma unroll
+  for (int j = 0; j < MR; ++j) {
+    const int m = 4 * j + q;
+    asrc[j] = A + (size_t)(m < M ? m : 0) * lda + 8 * piece;
+  }
+
+  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+
+  auto fetch = [&](int st, u32x4_t* w, u32x4_t* a) {
+    const int k0 = st * kStepK;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w[j] = *reinterpret_cast<const u32x4_t*>(wsrc[j] + k0);
+#pragma unroll
+    for (int j = 0; j < MR; ++j) a[j] = *reinterpret_cast<const u32x4_t*>(asrc[j] + k0);
+  };
+  // registers in fetch layout -> LDS -> registers in operand layout -> MFMA
+  auto consume = [&](const u32x4_t* w, const u32x4_t* a) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(w_lds + (4 * j + q) * kPitch + 8 * piece) = w[j];
+#pragma unroll
+    for (int j = 0; j < MR; ++j) *reinterpret_cast<u32x4_t*>(a_lds + (4 * j + q) * kPitch + 8 * piece) = a[j];
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    u32x4_t wop[4], aop[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      wop[u] = *reinterpret_cast<const u32x4_t*>(w_lds + n16 * kPitch + 8 * (g4 + 4 * u));
+      aop[u] = *reinterpret_cast<const u32x4_t*>(a_lds + n16 * kPitch + 8 * (g4 + 4 * u));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(lo_half(wop[u]), lo_half(aop[u]), acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(hi_half(wop[u]), hi_half(aop[u]), acc, 0, 0, 0);
+    }
+  };
+
+  u32x4_t w0[4], w1[4], a0[MR], a1[MR];
+  // Rows of W lie a power of two apart, so blocks that walk K in step would all press on the same
+  // memory channels at once; every block therefore starts its walk at a different step and wraps
+  // around.  Two steps per trip so that both buffers are named statically (they stay in registers).
+  const int nst = step_hi - step_lo;
+  const int rot = nst > 0 ? (int)((blockIdx.x * 5u + wave * 3u) % (unsigned)nst) : 0;
+  auto step_of = [&](int i) {
+    int s = i + rot;
+    if (s >= nst) s -= nst;
+    return step_lo + s;
+  };
+  // The prefetches are unconditional (past the end they repeat the last step and are ignored): a
+  // load under a branch would make the wait before its use cover both paths, that is, wait for the
+  // prefetch itself.
+  if (nst > 0) {
+    fetch(step_of(0), w0, a0);
+    int i = 0;
+    for (; i + 1 < nst; i += 2) {
+      fetch(step_of(i + 1), w1, a1);
+      consume(w0, a0);
+      fetch(step_of(min(i + 2, nst - 1)), w0, a0);
+      consume(w1, a1);
+    }
+    if (i < nst) consume(w0, a0);  // an odd number of steps: the last one is already loaded
+  }
+  // the partial step: pieces past K are read from a clamped address and the A side is zeroed, so the
+  // out-of-range products vanish
+  if (wave == WAVES - 1 && steps_full * kStepK < K) {
+    const int k = steps_full * kStepK + 8 * piece;
+    const int kc = min(k, K - 8) - 8 * piece;
+    const uint32_t keep = k < K ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w0[j] = *reinterpret_cast<const u32x4_t*>(wsrc[j] + kc);
+#pragma unroll
+    for (int j = 0; j < MR; ++j) {
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(asrc[j] + kc);
+      a0[j] = u32x4_t{v[0] & keep, v[1] & keep, v[2] & keep, v[3] & keep};
+    }
+    consume(w0, a0);
+  }
+
+  // acc[i] = C^T[n0 + 4 g4 + i][n16]; add the waves' shares in wave order (the wave's own W tile in
+  // LDS serves as its slot)
+  if (WAVES > 1) {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    float* slot = reinterpret_cast<float*>(w_lds);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) slot[lane * 4 + i] = acc[i];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < WAVES; ++w2) sum += reinterpret_cast<const float*>(lds + (size_t)w2 * kWaveElems)[lane * 4 + i];
+      acc[i] = sum;
+    }
+  }
+  if (n16 < M) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = n0 + 4 * g4 + i;
+      if (n < N) C[(size_t)n16 * ldc + n] = from_f32<OutT>(acc[i]);
+    }
+  }
+}
+
+template <int MR, int WAVES, typename OutT>
+int launch_typed(const bf16_t* A, int lda, const bf16_t* W, int ldw, OutT* C, int ldc, int M, int N, int K,
+                 hipStream_t stream) {
+  const size_t lds = (size_t)WAVES * 2 * kTileElems * sizeof(bf16_t);
+  static bool raised = false;  // blocks past 64 KB of LDS have to be allowed once per kernel
+  if (lds > 64 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<MR, WAVES, OutT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "gemm_stream: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    raised = true;
+  }
+  const dim3 grid((N + kStrip - 1) / kStrip);
+  gemm_stream_kernel<MR, WAVES, OutT><<<grid, WAVES * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  return tl_check_launch("gemm_stream");
+}
+
+template <int MR, int WAVES>
+int launch(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N, int K,
+           int out_dtype, hipStream_t stream) {
+  if (out_dtype == TL_BF16) return launch_typed<MR, WAVES, bf16_t>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, stream);
+  return launch_typed<MR, WAVES, float>(A, lda, W, ldw, (float*)C, ldc, M, N, K, stream);
+}
+
+template <int MR>
+int launch_waves(int waves, const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N,
+                 int K, int out_dtype, hipStream_t stream) {
+  switch (waves) {
+    case 1: return launch<MR, 1>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+    case 2: return launch<MR, 2>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+    case 4: return launch<MR, 4>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+    default: return launch<MR, 8>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+  }
+}
+
+}  // namespace
+
+// A [M, K] and W [N, K] bfloat16, row-major with leading dimensions lda / ldw (multiples of 8, bases
+// 16-byte aligned); C [M, N] bfloat16 (out_dtype 1) or 32-bit (out_dtype 0).  M <= 16, K a multiple of 8.
+// waves = 0 picks the number of K splits from the sizes.
+TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
+                             int K, int out_dtype, int waves, hipStream_t stream) {
+  TL_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_stream: bad sizes M=%d N=%d K=%d", M, N, K);
+  if (M > 16) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream: M=%d exceeds 16", M);
+  if (K % 8) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream: K=%d is not a multiple of 8", K);
+  TL_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_stream: leading dimensions too small");
+  TL_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0,
+             "gemm_stream: rows must start on 16-byte boundaries");
+  TL_REQUIRE(out_dtype == TL_BF16 || out_dtype == TL_F32, "gemm_stream: out_dtype must be 0 or 1");
+  if (M == 0) return TL_OK;
+  if (waves == 0) {
+    // enough waves to keep loads in flight on 256 CUs: about 4096 in all, at least two steps each
+    const int strips = (N + kStrip - 1) / kStrip;
+    const int steps = (K + kStepK - 1) / kStepK;
+    waves = 1;
+    while (waves < 8 && strips * waves < 4096 && steps >= 2 * waves * 2) waves *= 2;
+  }
+  TL_REQUIRE(waves == 1 || waves == 2 || waves == 4 || waves == 8, "gemm_stream: waves must be 1, 2, 4 or 8");
+  const bf16_t* a = (const bf16_t*)A;
+  const bf16_t* w = (const bf16_t*)W;
+  if (M <= 4) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
+  if (M <= 8) return launch_waves<2>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
+  return launch_waves<4>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
+}

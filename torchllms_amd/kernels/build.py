@@ -32,7 +32,7 @@ CORE_SOURCES = [
     "elementwise.hip",
     "attention_generic.hip",
     "gemm_f32.hip",
-    "gemm_skinny.hip",
+    "gemm_stream.hip",
     "sampling.hip",
 ]
 HEADERS = ["common.h"]

@@ -211,25 +211,25 @@ def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
-SKINNY_MAX_ROWS = 16
+STREAM_MAX_ROWS = 16  # what the weight-streaming kernel takes
 #: shapes that were never measured (see ``tune_linear``) use the weight-streaming kernel up to this
 #: many elements: small matrices are where the library's launch and tail costs weigh most
-SKINNY_MAX_ELEMENTS = 1 << 24
+STREAM_MAX_ELEMENTS = 1 << 28
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0) -> torch.Tensor:
-    """``x @ w.T`` for at most 64 rows of bfloat16 ``x`` with the weight-streaming MFMA kernel;
-    the result is bfloat16 or float32."""
+def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, waves: int = 0) -> torch.Tensor:
+    """``x @ w.T`` for at most 16 rows of bfloat16 ``x`` with the kernel that fetches W coalesced
+    and transposes it through LDS; the result is bfloat16 or float32."""
     _gpu(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise KernelError("gemm_skinny takes bfloat16 tensors")
+        raise KernelError("gemm_stream takes bfloat16 tensors")
     if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1:
-        raise KernelError(f"gemm_skinny: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
+        raise KernelError(f"gemm_stream: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
     m, k = x.shape
     n = w.shape[0]
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     check(
-        core().tl_gemm_skinny(
+        core().tl_gemm_stream(
             x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k,
             dtype_code(out_dtype), waves, _stream(),
         )
@@ -237,18 +237,20 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     return out
 
 
-def skinny_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+def stream_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the weight-streaming kernel can take this product at all."""
     return (
-        x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0
+        x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[0] <= STREAM_MAX_ROWS and x.shape[1] % 8 == 0
         and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
     )
 
 
-#: measured choice between the two bfloat16 kernels: (n, k, row bucket) -> True (weight-streaming
-#: kernel) / False (library).  Filled by ``tune_linear``; shapes never measured follow the size rule.
+#: measured choice of bfloat16 kernel: (n, k, row bucket) -> number of waves (splits of K) for the
+#: weight-streaming kernel (0 = its own rule), or None for the library.  Filled by ``tune_linear``;
+#: shapes never measured follow the size rule.
 _LINEAR_CHOICE: dict = {}
 ROW_BUCKETS = (1, 2, 4, 8, 16)
+STREAM_WAVE_CHOICES = (0, 4)
 
 
 def _row_bucket(m: int) -> int:
@@ -258,20 +260,21 @@ def _row_bucket(m: int) -> int:
     return ROW_BUCKETS[-1]
 
 
-def use_skinny(x: torch.Tensor, w: torch.Tensor) -> bool:
-    if not skinny_supported(x, w):
-        return False
-    choice = _LINEAR_CHOICE.get((w.shape[0], w.shape[1], _row_bucket(x.shape[0])))
-    if choice is None:
-        return w.shape[0] * w.shape[1] <= SKINNY_MAX_ELEMENTS
-    return choice
+def stream_choice(x: torch.Tensor, w: torch.Tensor):
+    """The number of waves when the weight-streaming kernel should run this product, else None."""
+    if not stream_supported(x, w):
+        return None
+    key = (w.shape[0], w.shape[1], _row_bucket(x.shape[0]))
+    if key in _LINEAR_CHOICE:
+        return _LINEAR_CHOICE[key]
+    return 0 if w.shape[0] * w.shape[1] <= STREAM_MAX_ELEMENTS else None
 
 
 def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, iters: int = 6) -> None:
-    """Measure, for matrices of one shape and every row bucket, which bfloat16 kernel is faster on
-    this GPU, and remember it.  ``weights``: the model's tensors of that shape; timing rotates over
-    them, as a decode step does, so that no run is served from cache.  Shapes already measured are
-    left alone, so every engine of a process makes the same choice."""
+    """Measure, for matrices of one shape and every row bucket, which bfloat16 kernel and launch is
+    fastest on this GPU, and remember it.  ``weights``: the model's tensors of that shape; timing
+    rotates over them, as a decode step does, so that no run is served from cache.  Shapes already
+    measured are left alone, so every engine of a process makes the same choice."""
     weights = [w for w in weights if w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2]
     if not weights:
         return
@@ -279,21 +282,32 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, iters: int = 6
     if k % 8 or weights[0].stride(0) % 8:
         return
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def clock(fn) -> float:
+        for i in range(2):
+            fn(weights[i % len(weights)])
+        start.record()
+        for i in range(iters):
+            fn(weights[(i + 2) % len(weights)])
+        stop.record()
+        stop.synchronize()
+        return start.elapsed_time(stop)
+
     for bucket in ROW_BUCKETS:
         if (n, k, bucket) in _LINEAR_CHOICE:
             continue
         x = torch.randn((bucket, k), device=weights[0].device, dtype=torch.float32).to(torch.bfloat16)
-        times = []
-        for fn in (lambda w: gemm_skinny(x, w, out_dtype), lambda w: torch.nn.functional.linear(x, w)):
-            for i in range(2):
-                fn(weights[i % len(weights)])
-            start.record()
-            for i in range(iters):
-                fn(weights[(i + 2) % len(weights)])
-            stop.record()
-            stop.synchronize()
-            times.append(start.elapsed_time(stop))
-        _LINEAR_CHOICE[(n, k, bucket)] = times[0] <= times[1]
+
+        def library(w):
+            y = torch.nn.functional.linear(x, w)
+            return y if y.dtype == out_dtype else y.to(out_dtype)
+
+        best, best_time = None, clock(library)
+        for waves in STREAM_WAVE_CHOICES:
+            t = clock(lambda w: gemm_stream(x, w, out_dtype, waves))
+            if t < best_time:
+                best, best_time = waves, t
+        _LINEAR_CHOICE[(n, k, bucket)] = best
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -306,8 +320,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         return gemm_f32(x, w)
     _gpu(x, w)
     out_dtype = out_dtype or x.dtype
-    if use_skinny(x, w):
-        return gemm_skinny(x, w, out_dtype)
+    waves = stream_choice(x, w)
+    if waves is not None:
+        return gemm_stream(x, w, out_dtype, waves)
     y = torch.nn.functional.linear(x, w)
     return y if y.dtype == out_dtype else y.to(out_dtype)
 
