@@ -564,6 +564,22 @@ def test_gemm_stream(m, n, k, out_dtype):
         assert (got.double() - want).abs().max().item() <= tol, f"waves={waves}"
 
 
+@pytest.mark.parametrize("m, f, k", [(1, 4096, 1024), (8, 14336, 4096), (5, 100, 136), (16, 688, 96), (12, 24, 8)])
+def test_gemm_stream_glu_equals_the_product_followed_by_the_gate(m, f, k):
+    """The same roundings as the two kernels it replaces; the 32-bit sums may differ in their last
+    bit (blocks walk K from different starting steps), so single results may move by one rounding."""
+    torch.manual_seed(1)
+    x = torch.randn(m, k).bfloat16().to(DEV)
+    w = (torch.randn(2 * f, k) * 0.1).bfloat16().to(DEV)
+    for waves in (0, 1, 2, 4, 8):
+        want = _ops().silu_mul(_ops().gemm_stream(x, w, torch.bfloat16, waves=waves))
+        got = _ops().gemm_stream_glu(x, w, waves=waves)
+        torch.testing.assert_close(got.float(), want.float(), rtol=2 ** -6, atol=2 ** -8 * want.float().abs().max().item(), msg=f"waves={waves}")
+        assert (got != want).float().mean().item() < 0.05, f"waves={waves}"
+    ref = torch.nn.functional.silu(x.float() @ w[:f].float().T) * (x.float() @ w[f:].float().T)
+    torch.testing.assert_close(_ops().linear_glu(x, w).float(), ref, rtol=2 ** -6, atol=2 ** -6 * ref.abs().max().item())
+
+
 def test_gemm_stream_takes_strided_rows_and_says_its_limits():
     from torchllms_amd.kernels.lib import KernelError
 

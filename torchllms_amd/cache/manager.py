@@ -22,6 +22,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 
@@ -130,6 +131,8 @@ class RequestEntry:
     # per group: logical block -> page id, -1 where a window has passed and the page went back
     block_tables: List[List[int]] = field(default_factory=list)
     first_live_block: List[int] = field(default_factory=list)
+    # per group: the block table as an int32 array, rebuilt only after the table has changed
+    table_arrays: List[Optional[np.ndarray]] = field(default_factory=list)
 
 
 @dataclass
@@ -234,6 +237,7 @@ class CacheManager:
             slot=slot,
             block_tables=[[] for _ in self.groups],
             first_live_block=[0 for _ in self.groups],
+            table_arrays=[None for _ in self.groups],
         )
         for t in self.state_tensors:
             if t is not None:
@@ -254,6 +258,17 @@ class CacheManager:
 
     def block_table(self, rid: Hashable, group: int = 0) -> List[int]:
         return self.entry(rid).block_tables[group]
+
+    def block_table_array(self, rid: Hashable, group: int = 0) -> np.ndarray:
+        """The block table as a read-only int32 array (kept until the table changes: a step plan
+        copies rows of it instead of converting a list every step)."""
+        e = self.entry(rid)
+        arr = e.table_arrays[group]
+        if arr is None:
+            arr = np.asarray(e.block_tables[group], dtype=np.int32)
+            arr.setflags(write=False)
+            e.table_arrays[group] = arr
+        return arr
 
     # ------------------------------------------------------------------ pages
     def _first_needed_block(self, group: int, first_query_pos: int) -> int:
@@ -301,6 +316,7 @@ class CacheManager:
             extra = need_blocks - len(e.block_tables[gi])
             if extra > 0:
                 e.block_tables[gi].extend(pool.take(extra))
+                e.table_arrays[gi] = None
         e.reserved_tokens = max(e.reserved_tokens, e.num_tokens + n_new)
         return e.num_tokens
 
@@ -319,6 +335,7 @@ class CacheManager:
                 pool.give_back(passed)
                 for b in range(e.first_live_block[gi], first):
                     bt[b] = -1
+                e.table_arrays[gi] = None
             e.first_live_block[gi] = max(e.first_live_block[gi], first)
 
     def truncate(self, rid: Hashable, num_tokens: int) -> None:
@@ -335,6 +352,7 @@ class CacheManager:
             tail = [p for p in bt[keep:] if p >= 0]
             pool.give_back(tail)
             del bt[keep:]
+            e.table_arrays[gi] = None
         e.num_tokens = num_tokens
         e.reserved_tokens = num_tokens
 
@@ -396,6 +414,8 @@ class CacheManager:
             held: Dict[int, int] = {}
             for rid, e in self._requests.items():
                 bt = e.block_tables[gi]
+                if e.table_arrays[gi] is not None and e.table_arrays[gi].tolist() != bt:
+                    raise AssertionError(f"{rid!r}: the cached array of group {gi}'s block table is stale")
                 need = self.blocks_for(max(e.num_tokens, e.reserved_tokens))
                 if len(bt) < self.blocks_for(e.num_tokens):
                     raise AssertionError(f"{rid!r}: {len(bt)} blocks for {e.num_tokens} tokens")

@@ -335,6 +335,8 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   const int R = n_q_heads / n_kv_heads;
   if (R > 16) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: %d query heads per kv head exceed 16", R);
   if (n_kv_heads > 65535) return variant_fail(TL_ERR_ARG, "attn_prefill: grid out of range");
+  // the running maximum is taken over raw scores and scaled afterwards
+  if (!(scale > 0.f)) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: softmax scale %g must be positive", (double)scale);
   if (q_stride % 8 || ((uintptr_t)q % 16) || out_stride % 4 || ((uintptr_t)out % 8))
     return variant_fail(TL_ERR_ARG, "attn_prefill: queries need 16-byte aligned rows, outputs 8-byte aligned rows");
   if (n_tiles == 0) return TL_OK;

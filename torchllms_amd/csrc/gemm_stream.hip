@@ -14,6 +14,9 @@
 //     fetched and transposed the same way (only as many groups of four rows as M needs).
 //   * the LDS rows are 272 bytes apart: the 16 lanes that read one 16-byte piece of 16 different
 //     rows then fall on different banks.
+//   * gated variant (GLU): W = gate rows | up rows; a block computes the same 16 columns of both
+//     products from one fetch of A and stores silu(gate) * up, with the roundings of the unfused
+//     sequence (both products rounded to bfloat16, the activation rounded, then the product).
 #include "common.h"
 
 namespace {
@@ -32,10 +35,12 @@ __device__ __forceinline__ short4_t lo_half(u32x4_t v) { return __builtin_bit_ca
 __device__ __forceinline__ short4_t hi_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[2], v[3]}); }
 
 // MR: groups of four rows of A that are fetched (M <= 4 * MR).  WAVES: waves per block = splits of K.
-template <int MR, int WAVES, typename OutT>
+// GLU: W holds 2 N rows, gate rows then up rows; C[M, N] = silu(A gate^T) * (A up^T).
+template <int MR, int WAVES, typename OutT, bool GLU>
 __global__ void __launch_bounds__(WAVES* kWave)
 gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
                    OutT* __restrict__ C, int ldc, int M, int N, int K) {
+  constexpr int NW = GLU ? 2 : 1;  // W tiles per step
   // per wave: a tile of W [16][kPitch], then a tile of A [4 MR][kPitch] (rows past 4 MR are read as
   // whatever the neighbour holds: they only feed output columns that are never stored)
   extern __shared__ __attribute__((aligned(16))) bf16_t lds[];
@@ -58,9 +63,12 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   const int step_hi = min(step_lo + steps_per_wave, steps_full);
 
   // rows of W past N are clamped, rows of A past M read row 0: neither result is stored
-  const bf16_t* wsrc[4];
+  const bf16_t* wsrc[4 * NW];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) wsrc[j] = W + (size_t)min(n0 + 4 * j + q, N - 1) * ldw + 8 * piece;
+  for (int t = 0; t < NW; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      wsrc[4 * t + j] = W + ((size_t)t * N + min(n0 + 4 * j + q, N - 1)) * ldw + 8 * piece;
   const bf16_t* asrc[MR];
 #pragma unroll
   for (int j = 0; j < MR; ++j) {
@@ -68,40 +76,48 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     asrc[j] = A + (size_t)(m < M ? m : 0) * lda + 8 * piece;
   }
 
-  float4_t acc = {0.f, 0.f, 0.f, 0.f};
+  float4_t acc[NW];
+#pragma unroll
+  for (int t = 0; t < NW; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   auto fetch = [&](int st, u32x4_t* w, u32x4_t* a) {
     const int k0 = st * kStepK;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) w[j] = *reinterpret_cast<const u32x4_t*>(wsrc[j] + k0);
+    for (int j = 0; j < 4 * NW; ++j) w[j] = *reinterpret_cast<const u32x4_t*>(wsrc[j] + k0);
 #pragma unroll
     for (int j = 0; j < MR; ++j) a[j] = *reinterpret_cast<const u32x4_t*>(asrc[j] + k0);
   };
-  // registers in fetch layout -> LDS -> registers in operand layout -> MFMA
+  // registers in fetch layout -> LDS -> registers in operand layout -> MFMA; the second W tile of
+  // the gated variant passes through the same piece of LDS after the first (LDS runs in order)
   auto consume = [&](const u32x4_t* w, const u32x4_t* a) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-#pragma unroll
-    for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(w_lds + (4 * j + q) * kPitch + 8 * piece) = w[j];
-#pragma unroll
-    for (int j = 0; j < MR; ++j) *reinterpret_cast<u32x4_t*>(a_lds + (4 * j + q) * kPitch + 8 * piece) = a[j];
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
     u32x4_t wop[4], aop[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      wop[u] = *reinterpret_cast<const u32x4_t*>(w_lds + n16 * kPitch + 8 * (g4 + 4 * u));
-      aop[u] = *reinterpret_cast<const u32x4_t*>(a_lds + n16 * kPitch + 8 * (g4 + 4 * u));
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+    for (int t = 0; t < NW; ++t) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(lo_half(wop[u]), lo_half(aop[u]), acc, 0, 0, 0);
-      acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(hi_half(wop[u]), hi_half(aop[u]), acc, 0, 0, 0);
+      for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(w_lds + (4 * j + q) * kPitch + 8 * piece) = w[4 * t + j];
+      if (t == 0) {
+#pragma unroll
+        for (int j = 0; j < MR; ++j) *reinterpret_cast<u32x4_t*>(a_lds + (4 * j + q) * kPitch + 8 * piece) = a[j];
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        wop[u] = *reinterpret_cast<const u32x4_t*>(w_lds + n16 * kPitch + 8 * (g4 + 4 * u));
+        if (t == 0) aop[u] = *reinterpret_cast<const u32x4_t*>(a_lds + n16 * kPitch + 8 * (g4 + 4 * u));
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(lo_half(wop[u]), lo_half(aop[u]), acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(hi_half(wop[u]), hi_half(aop[u]), acc[t], 0, 0, 0);
+      }
     }
   };
 
-  u32x4_t w0[4], w1[4], a0[MR], a1[MR];
+  u32x4_t w0[4 * NW], w1[4 * NW], a0[MR], a1[MR];
   // Rows of W lie a power of two apart, so blocks that walk K in step would all press on the same
   // memory channels at once; every block therefore starts its walk at a different step and wraps
   // around.  Two steps per trip so that both buffers are named statically (they stay in registers).
@@ -133,7 +149,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     const int kc = min(k, K - 8) - 8 * piece;
     const uint32_t keep = k < K ? 0xFFFFFFFFu : 0u;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) w0[j] = *reinterpret_cast<const u32x4_t*>(wsrc[j] + kc);
+    for (int j = 0; j < 4 * NW; ++j) w0[j] = *reinterpret_cast<const u32x4_t*>(wsrc[j] + kc);
 #pragma unroll
     for (int j = 0; j < MR; ++j) {
       const u32x4_t v = *reinterpret_cast<const u32x4_t*>(asrc[j] + kc);
@@ -142,73 +158,82 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     consume(w0, a0);
   }
 
-  // acc[i] = C^T[n0 + 4 g4 + i][n16]; add the waves' shares in wave order (the wave's own W tile in
-  // LDS serves as its slot)
+  // acc[t][i] = C^T[n0 + 4 g4 + i][n16]; add the waves' shares in wave order (the wave's own W tile
+  // in LDS serves as its slot)
   if (WAVES > 1) {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     float* slot = reinterpret_cast<float*>(w_lds);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) slot[lane * 4 + i] = acc[i];
+    for (int t = 0; t < NW; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) slot[(t * kWave + lane) * 4 + i] = acc[t][i];
     __syncthreads();
     if (wave != 0) return;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float sum = 0.f;
+    for (int t = 0; t < NW; ++t)
 #pragma unroll
-      for (int w2 = 0; w2 < WAVES; ++w2) sum += reinterpret_cast<const float*>(lds + (size_t)w2 * kWaveElems)[lane * 4 + i];
-      acc[i] = sum;
-    }
+      for (int i = 0; i < 4; ++i) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w2 = 0; w2 < WAVES; ++w2)
+          sum += reinterpret_cast<const float*>(lds + (size_t)w2 * kWaveElems)[(t * kWave + lane) * 4 + i];
+        acc[t][i] = sum;
+      }
   }
   if (n16 < M) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int n = n0 + 4 * g4 + i;
-      if (n < N) C[(size_t)n16 * ldc + n] = from_f32<OutT>(acc[i]);
+      if (n >= N) continue;
+      if constexpr (GLU) {
+        const float g = to_f32(from_f32<OutT>(acc[0][i]));
+        const float u = to_f32(from_f32<OutT>(acc[1][i]));
+        const float act = to_f32(from_f32<OutT>(g / (1.0f + expf(-g))));
+        C[(size_t)n16 * ldc + n] = from_f32<OutT>(act * u);
+      } else {
+        C[(size_t)n16 * ldc + n] = from_f32<OutT>(acc[0][i]);
+      }
     }
   }
 }
 
-template <int MR, int WAVES, typename OutT>
+template <int MR, int WAVES, typename OutT, bool GLU>
 int launch_typed(const bf16_t* A, int lda, const bf16_t* W, int ldw, OutT* C, int ldc, int M, int N, int K,
                  hipStream_t stream) {
   const size_t lds = (size_t)WAVES * 2 * kTileElems * sizeof(bf16_t);
   static bool raised = false;  // blocks past 64 KB of LDS have to be allowed once per kernel
   if (lds > 64 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<MR, WAVES, OutT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<MR, WAVES, OutT, GLU>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "gemm_stream: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     raised = true;
   }
   const dim3 grid((N + kStrip - 1) / kStrip);
-  gemm_stream_kernel<MR, WAVES, OutT><<<grid, WAVES * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  gemm_stream_kernel<MR, WAVES, OutT, GLU><<<grid, WAVES * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
   return tl_check_launch("gemm_stream");
 }
 
 template <int MR, int WAVES>
 int launch(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N, int K,
-           int out_dtype, hipStream_t stream) {
-  if (out_dtype == TL_BF16) return launch_typed<MR, WAVES, bf16_t>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, stream);
-  return launch_typed<MR, WAVES, float>(A, lda, W, ldw, (float*)C, ldc, M, N, K, stream);
+           int out_dtype, bool glu, hipStream_t stream) {
+  if (glu) return launch_typed<MR, WAVES, bf16_t, true>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, stream);
+  if (out_dtype == TL_BF16) return launch_typed<MR, WAVES, bf16_t, false>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, stream);
+  return launch_typed<MR, WAVES, float, false>(A, lda, W, ldw, (float*)C, ldc, M, N, K, stream);
 }
 
 template <int MR>
 int launch_waves(int waves, const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N,
-                 int K, int out_dtype, hipStream_t stream) {
+                 int K, int out_dtype, bool glu, hipStream_t stream) {
   switch (waves) {
-    case 1: return launch<MR, 1>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
-    case 2: return launch<MR, 2>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
-    case 4: return launch<MR, 4>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
-    default: return launch<MR, 8>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, stream);
+    case 1: return launch<MR, 1>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
+    case 2: return launch<MR, 2>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
+    case 4: return launch<MR, 4>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
+    default: return launch<MR, 8>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
   }
 }
 
-}  // namespace
-
-// A [M, K] and W [N, K] bfloat16, row-major with leading dimensions lda / ldw (multiples of 8, bases
-// 16-byte aligned); C [M, N] bfloat16 (out_dtype 1) or 32-bit (out_dtype 0).  M <= 16, K a multiple of 8.
-// waves = 0 picks the number of K splits from the sizes.
-TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
-                             int K, int out_dtype, int waves, hipStream_t stream) {
+int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K, int out_dtype,
+        int waves, bool glu, hipStream_t stream) {
   TL_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_stream: bad sizes M=%d N=%d K=%d", M, N, K);
   if (M > 16) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream: M=%d exceeds 16", M);
   if (K % 8) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream: K=%d is not a multiple of 8", K);
@@ -227,7 +252,25 @@ TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, voi
   TL_REQUIRE(waves == 1 || waves == 2 || waves == 4 || waves == 8, "gemm_stream: waves must be 1, 2, 4 or 8");
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  if (M <= 4) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
-  if (M <= 8) return launch_waves<2>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
-  return launch_waves<4>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, stream);
+  if (M <= 4) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
+  if (M <= 8) return launch_waves<2>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
+  return launch_waves<4>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
+}
+
+}  // namespace
+
+// A [M, K] and W [N, K] bfloat16, row-major with leading dimensions lda / ldw (multiples of 8, bases
+// 16-byte aligned); C [M, N] bfloat16 (out_dtype 1) or 32-bit (out_dtype 0).  M <= 16, K a multiple of 8.
+// waves = 0 picks the number of K splits from the sizes.
+TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
+                             int K, int out_dtype, int waves, hipStream_t stream) {
+  return run(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, waves, false, stream);
+}
+
+// The gated pair of products: W [2 N, K] = gate rows | up rows; C [M, N] bfloat16 =
+// silu(A gate^T) * (A up^T), rounded as the two products, the activation and the final product
+// would be if each were stored in bfloat16.
+TL_EXPORT int tl_gemm_stream_glu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
+                                 int K, int waves, hipStream_t stream) {
+  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, true, stream);
 }

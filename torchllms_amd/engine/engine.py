@@ -169,7 +169,7 @@ class Engine:
                 )
         starts = [self.cache.extend(e.rid, len(e.tokens)) for e in entries]
         slots = [self.cache.slot(e.rid) for e in entries]
-        tables = [[self.cache.block_table(e.rid, g) for e in entries] for g in range(len(self.cache.groups))]
+        tables = [[self.cache.block_table_array(e.rid, g) for e in entries] for g in range(len(self.cache.groups))]
         return build_step_layout(entries, starts, slots, tables, self.page_size)
 
     @torch.inference_mode()

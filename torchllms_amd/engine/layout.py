@@ -92,17 +92,23 @@ def build_step_layout(
     token_seq = np.empty(T, dtype=np.int32)
     kv_lens = np.empty(B, dtype=np.int32)
     slot_ids = np.empty(B, dtype=np.int32)
+    bounds = qo_indptr.tolist()
     for row, i in enumerate(order):
-        lo, hi = int(qo_indptr[row]), int(qo_indptr[row + 1])
-        tokens[lo:hi] = np.asarray(entries[i].tokens, dtype=np.int64)
-        positions[lo:hi] = np.arange(starts[i], starts[i] + (hi - lo), dtype=np.int32)
-        token_seq[lo:hi] = row
+        lo, hi = bounds[row], bounds[row + 1]
+        if hi - lo == 1:  # a decoded token: scalars, no small arrays
+            tokens[lo] = entries[i].tokens[0]
+            positions[lo] = starts[i]
+            token_seq[lo] = row
+        else:
+            tokens[lo:hi] = np.asarray(entries[i].tokens, dtype=np.int64)
+            positions[lo:hi] = np.arange(starts[i], starts[i] + (hi - lo), dtype=np.int32)
+            token_seq[lo:hi] = row
         kv_lens[row] = starts[i] + (hi - lo)
         slot_ids[row] = slots[i]
 
     logit_rows: List[int] = []
     for i, e in enumerate(entries):
-        base = int(qo_indptr[row_of_entry[i]])
+        base = bounds[row_of_entry[i]]
         n = len(e.tokens)
         for w in e.want:
             if not 0 <= w < n:
@@ -119,7 +125,13 @@ def build_step_layout(
         for row, i in enumerate(order):
             table = np.asarray(block_tables[g][i], dtype=np.int32)
             bt[row, : len(table)] = table
-            lo, hi = int(qo_indptr[row]), int(qo_indptr[row + 1])
+            lo, hi = bounds[row], bounds[row + 1]
+            if hi - lo == 1:
+                page = int(table[starts[i] // page_size])
+                if page < 0:
+                    raise RuntimeError(f"request {entries[i].rid!r}: a new token has no page (extend first)")
+                sm[lo] = page * page_size + starts[i] % page_size
+                continue
             pos = positions[lo:hi]
             pages = table[pos // page_size]
             if (pages < 0).any():

@@ -29,7 +29,8 @@ def paged_attention(
     n = qkv.shape[0]
     n_dec = ctx.host.n_decode
     fast_decode = n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
-    fast_prefill = n_dec < n and ops.prefill_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
+    # the MFMA prefill kernel takes positive softmax scales only; anything else runs the plain kernel
+    fast_prefill = n_dec < n and scale > 0 and ops.prefill_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
     if not fast_decode and not fast_prefill:
         return ops.attention_generic(
             qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq, ctx.positions,

@@ -237,6 +237,25 @@ def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     return out
 
 
+def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0) -> torch.Tensor:
+    """``silu(x @ gate.T) * (x @ up.T)`` for at most 16 rows of bfloat16 ``x`` and ``w`` [2F, K] =
+    gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``."""
+    _gpu(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("gemm_stream_glu takes bfloat16 tensors")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1 or w.shape[0] % 2:
+        raise KernelError(f"gemm_stream_glu: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
+    m, k = x.shape
+    n = w.shape[0] // 2
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    check(
+        core().tl_gemm_stream_glu(
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k, waves, _stream(),
+        )
+    )
+    return out
+
+
 def stream_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the weight-streaming kernel can take this product at all."""
     return (
@@ -325,6 +344,16 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         return gemm_stream(x, w, out_dtype, waves)
     y = torch.nn.functional.linear(x, w)
     return y if y.dtype == out_dtype else y.to(out_dtype)
+
+
+def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``silu(x @ gate.T) * (x @ up.T)`` for ``w`` [2F, K] = gate rows | up rows: one fused kernel
+    where the weight-streaming kernel serves the shape, else the product followed by the gate."""
+    if x.dtype == torch.bfloat16:
+        waves = stream_choice(x, w)
+        if waves is not None:
+            return gemm_stream_glu(x, w, waves)
+    return silu_mul(linear(x, w))
 
 
 def sample(

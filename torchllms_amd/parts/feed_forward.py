@@ -34,5 +34,4 @@ class SwiGLU(FeedForward):
         return [self.w13, self.w2]
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        gate_up = ops.linear(x, self.w13)
-        return ops.linear(ops.silu_mul(gate_up), self.w2)
+        return ops.linear(ops.linear_glu(x, self.w13), self.w2)

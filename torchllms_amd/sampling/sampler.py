@@ -18,6 +18,12 @@ class Sampler:
     the batch and however often it was preempted.
     """
 
+    def __init__(self):
+        # the tensors of the last batch's parameters: a generation loop asks with the same
+        # requests step after step, and only the counters change
+        self._key = None
+        self._fixed = None
+
     def __call__(self, logits: torch.Tensor, params: Sequence[SamplingParams], steps: Sequence[int]) -> List[int]:
         n = logits.shape[0]
         if n == 0:
@@ -25,12 +31,16 @@ class Sampler:
         if len(params) != n or len(steps) != n:
             raise ValueError("one SamplingParams and one step counter per logits row")
         dev = logits.device
-        temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32, device=dev)
-        seeds = torch.tensor([_as_i64(p.seed) for p in params], dtype=torch.int64, device=dev)
+        key = (dev, tuple((p.temperature, p.seed, p.top_k) for p in params))
+        if key != self._key:
+            temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32, device=dev)
+            seeds = torch.tensor([_as_i64(p.seed) for p in params], dtype=torch.int64, device=dev)
+            top_k = None
+            if any(p.top_k for p in params):
+                top_k = torch.tensor([p.top_k or 0 for p in params], dtype=torch.int32, device=dev)
+            self._key, self._fixed = key, (temperature, seeds, top_k)
+        temperature, seeds, top_k = self._fixed
         counters = torch.tensor([int(s) for s in steps], dtype=torch.int64, device=dev)
-        top_k = None
-        if any(p.top_k for p in params):
-            top_k = torch.tensor([p.top_k or 0 for p in params], dtype=torch.int32, device=dev)
         return ops.sample(logits, temperature, seeds, counters, top_k).tolist()
 
 
