@@ -146,6 +146,62 @@ def test_rope_half_pairing_partial_rotary_and_no_pages(dtype):
     assert torch.equal(dev.cpu(), qkv)
 
 
+def test_rope_table_and_its_use_give_what_the_kernel_computes_itself():
+    torch.manual_seed(0)
+    n, hq, hkv, dh, rot = 9, 4, 2, 32, 24
+    pos = torch.tensor([0, 1, 7, 500, 8191, 131071, 3, 3, 12])
+    inv_freq = plain.rope_inverse_frequencies(rot, 500000.0, None)
+    table = _ops().rope_table(_i32(pos.tolist()), inv_freq.to(DEV))
+    ang = pos.float()[:, None] * inv_freq[None, :]  # 32-bit product, as the reference's table
+    torch.testing.assert_close(table[..., 0].cpu(), torch.cos(ang), rtol=0, atol=2e-7)
+    torch.testing.assert_close(table[..., 1].cpu(), torch.sin(ang), rtol=0, atol=2e-7)
+    for dtype in DTYPES:
+        qkv = torch.randn(n, (hq + 2 * hkv) * dh).to(dtype)
+        a, b = qkv.to(DEV), qkv.to(DEV)
+        _ops().rope_kv_write(a, hq, hkv, dh, _i32(pos.tolist()), inv_freq.to(DEV), rot, 0)
+        _ops().rope_kv_write(b, hq, hkv, dh, _i32(pos.tolist()), None, rot, 0, cos_sin=table)
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("m, hq, hkv, dh, rot, page, k", [(8, 32, 8, 128, 128, 16, 4096), (1, 4, 4, 64, 64, 16, 256),
+                                                           (13, 6, 3, 48, 24, 4, 136), (16, 5, 1, 20, 0, 8, 64), (3, 2, 2, 16, 16, 2, 8)])
+@pytest.mark.parametrize("with_pages", [True, False])
+def test_gemm_stream_qkv_equals_product_then_rotary_kernel(m, hq, hkv, dh, rot, page, k, with_pages):
+    """The fused projection against the two kernels it replaces, on every output: rotated queries
+    in the buffer, rotated keys and raw values in their pages (or in the buffer without pages);
+    a row whose slot is negative stores nothing."""
+    torch.manual_seed(2)
+    width = (hq + 2 * hkv) * dh
+    x = torch.randn(m, k).bfloat16().to(DEV)
+    w = (torch.randn(width, k) * k ** -0.5).bfloat16().to(DEV)
+    pos = torch.randint(0, 9000, (m,))
+    inv_freq = plain.rope_inverse_frequencies(rot, 500000.0, None).to(DEV) if rot else None
+    table = _ops().rope_table(_i32(pos.tolist()), inv_freq) if rot else None
+    n_pages = 40
+    slots = torch.randperm(n_pages * page)[:m].tolist()
+    if m > 2:
+        slots[1] = -1
+    outs = []
+    for fused in (False, True):
+        kp, vp = _pages(n_pages, hkv, page, dh, torch.bfloat16) if with_pages else (None, None)
+        sm = _i32(slots) if with_pages else None
+        if fused:
+            qkv = _ops().gemm_stream_qkv(x, w, hq, hkv, dh, rot, table, kp, vp, sm, page if with_pages else 0)
+        else:
+            qkv = _ops().gemm_stream(x, w)
+            _ops().rope_kv_write(qkv, hq, hkv, dh, _i32(pos.tolist()), inv_freq, rot, 0, kp, vp, sm, page if with_pages else 0, cos_sin=table)
+        outs.append((qkv, kp, vp))
+    (qa, ka, va), (qb, kb, vb) = outs
+    cols = hq * dh if with_pages else width  # with pages only the queries of the buffer are defined
+    tol = dict(rtol=2 ** -7, atol=2 ** -8 * qa.float().abs().max().item())
+    torch.testing.assert_close(qb[:, :cols].float(), qa[:, :cols].float(), **tol)
+    assert (qb[:, :cols] != qa[:, :cols]).float().mean().item() < 0.05  # only last-bit differences of the sums
+    if with_pages:
+        torch.testing.assert_close(kb.float(), ka.float(), **tol)
+        torch.testing.assert_close(vb.float(), va.float(), **tol)
+        assert (kb.float().abs().sum(dim=(1, 3)) > 0).sum().item() == m - (1 if m > 2 else 0)  # one slot per stored row
+
+
 def test_cache_write_round_trip_with_distinct_values():
     # reference: torchllms/models/test_paged_kv.py:440-484 (append then extract, value = position)
     hq, hkv, dh, page = 2, 2, 8, 4

@@ -209,10 +209,33 @@ TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, 
 //   x0' = x0 cos - x1 sin ;  x1' = x1 cos + x0 sin        (32-bit, then one rounding)
 // q is rotated in place.  k is rotated and, with v, stored at slot_mapping[t] = page * P + offset
 // of pages laid out [page][Hkv][P][dh]; slot < 0 skips the store.  Without pages k is rotated in place.
+// The cosines and sines may come from a table [token][rotary_dim/2] of (cos, sin) made by
+// rope_table_kernel from the same positions (one table serves all layers of a step).
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  int n_tokens, int rot_half, float2* __restrict__ table) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_tokens * rot_half) return;
+  const int t = idx / rot_half;
+  const int i = idx % rot_half;
+  const float ang = (float)positions[t] * inv_freq[i];
+  table[idx] = make_float2(cosf(ang), sinf(ang));
+}
+
+TL_EXPORT int tl_rope_table(const int32_t* positions, const float* inv_freq, int n_tokens, int rot_half,
+                            float* table, hipStream_t stream) {
+  TL_REQUIRE(n_tokens >= 0 && rot_half > 0, "rope_table: bad sizes");
+  TL_REQUIRE((long long)n_tokens * rot_half < (1ll << 31), "rope_table: too many entries");
+  if (n_tokens == 0) return TL_OK;
+  const int total = n_tokens * rot_half;
+  rope_table_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, n_tokens, rot_half, (float2*)table);
+  return tl_check_launch("rope_table");
+}
+
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_kv_heads, int head_dim,
                                      const int32_t* __restrict__ positions,
-                                     const float* __restrict__ inv_freq, int rotary_dim, int pairing,
+                                     const float* __restrict__ inv_freq, const float2* __restrict__ cos_sin,
+                                     int rotary_dim, int pairing,
                                      T* __restrict__ k_pages, T* __restrict__ v_pages,
                                      const int32_t* __restrict__ slot_mapping, int page_size) {
   const int t = blockIdx.x;
@@ -246,9 +269,15 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_k
         i0 = i;
         i1 = i + rot_half;
       }
-      const float ang = pos * inv_freq[i];
-      c = cosf(ang);
-      sn = sinf(ang);
+      if (cos_sin) {
+        const float2 cs = cos_sin[(size_t)t * rot_half + i];
+        c = cs.x;
+        sn = cs.y;
+      } else {
+        const float ang = pos * inv_freq[i];
+        c = cosf(ang);
+        sn = sinf(ang);
+      }
     } else {
       // channels beyond rotary_dim pass unchanged
       i0 = rotary_dim + 2 * (i - rot_half);
@@ -286,15 +315,15 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_k
 }
 
 TL_EXPORT int tl_rope_kv_write(void* qkv, int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
-                               const int32_t* positions, const float* inv_freq, int rotary_dim,
-                               int pairing, void* k_pages, void* v_pages, const int32_t* slot_mapping,
-                               int page_size, int dtype, hipStream_t stream) {
+                               const int32_t* positions, const float* inv_freq, const float* cos_sin,
+                               int rotary_dim, int pairing, void* k_pages, void* v_pages,
+                               const int32_t* slot_mapping, int page_size, int dtype, hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q_heads > 0 && n_kv_heads >= 0 && head_dim > 0, "rope: bad sizes");
   TL_REQUIRE(head_dim % 2 == 0, "rope: head_dim=%d must be even", head_dim);
   TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0,
              "rope: rotary_dim=%d must be even and at most head_dim=%d", rotary_dim, head_dim);
   TL_REQUIRE(pairing == 0 || pairing == 1, "rope: pairing must be 0 (interleaved) or 1 (half split)");
-  TL_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope: inv_freq missing");
+  TL_REQUIRE(rotary_dim == 0 || inv_freq != nullptr || cos_sin != nullptr, "rope: neither inv_freq nor a table given");
   TL_REQUIRE(k_pages == nullptr || (slot_mapping != nullptr && page_size > 0),
              "rope: pages given without slot_mapping/page_size");
   if (n_tokens == 0) return TL_OK;
@@ -307,11 +336,11 @@ TL_EXPORT int tl_rope_kv_write(void* qkv, int n_tokens, int n_q_heads, int n_kv_
   const dim3 grid(n_tokens, columns);
   if (dtype == TL_F32)
     rope_kv_write_kernel<float><<<grid, threads, 0, stream>>>(
-        (float*)qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, rotary_dim, pairing,
+        (float*)qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, (const float2*)cos_sin, rotary_dim, pairing,
         (float*)k_pages, (float*)v_pages, slot_mapping, page_size);
   else if (dtype == TL_BF16)
     rope_kv_write_kernel<bf16_t><<<grid, threads, 0, stream>>>(
-        (bf16_t*)qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, rotary_dim, pairing,
+        (bf16_t*)qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, (const float2*)cos_sin, rotary_dim, pairing,
         (bf16_t*)k_pages, (bf16_t*)v_pages, slot_mapping, page_size);
   else
     return tl_fail(TL_ERR_ARG, "rope: unknown dtype %d", dtype);

@@ -17,6 +17,10 @@
 //   * gated variant (GLU): W = gate rows | up rows; a block computes the same 16 columns of both
 //     products from one fetch of A and stores silu(gate) * up, with the roundings of the unfused
 //     sequence (both products rounded to bfloat16, the activation rounded, then the product).
+//   * query/key/value variant (QKV): the columns are query heads | key heads | value heads; query and
+//     key heads are rotated by position (interleaved pairs, cosines and sines from a table), keys
+//     and values go straight into their cache pages, queries into C: the rotary kernel's work, done
+//     on the 32-bit sums after the rounding the unfused product would have applied.
 #include "common.h"
 
 namespace {
@@ -34,12 +38,26 @@ constexpr int kTileElems = 16 * kPitch;
 __device__ __forceinline__ short4_t lo_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[0], v[1]}); }
 __device__ __forceinline__ short4_t hi_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[2], v[3]}); }
 
+enum Epilogue { kPlain = 0, kGated = 1, kQkv = 2 };
+
+// What the query/key/value epilogue needs beside the product.
+struct QkvArgs {
+  int n_q_heads, n_kv_heads, head_dim;
+  int rotary_dim;                 // leading channels of a head that rotate (even; 0: none)
+  const float2* cos_sin;          // [row of A][rotary_dim / 2] = (cos, sin) of the row's position
+  bf16_t* k_pages;                // [page][kv head][page_size][head_dim], or null: keys and values stay in C
+  bf16_t* v_pages;
+  const int32_t* slot_mapping;    // per row of A: page * page_size + offset, < 0: not stored
+  int page_size;
+};
+
 // MR: groups of four rows of A that are fetched (M <= 4 * MR).  WAVES: waves per block = splits of K.
-// GLU: W holds 2 N rows, gate rows then up rows; C[M, N] = silu(A gate^T) * (A up^T).
-template <int MR, int WAVES, typename OutT, bool GLU>
+// EPI kGated: W holds 2 N rows, gate rows then up rows; C[M, N] = silu(A gate^T) * (A up^T).
+template <int MR, int WAVES, typename OutT, int EPI>
 __global__ void __launch_bounds__(WAVES* kWave)
 gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-                   OutT* __restrict__ C, int ldc, int M, int N, int K) {
+                   OutT* __restrict__ C, int ldc, int M, int N, int K, QkvArgs qa) {
+  constexpr bool GLU = EPI == kGated;
   constexpr int NW = GLU ? 2 : 1;  // W tiles per step
   // per wave: a tile of W [16][kPitch], then a tile of A [4 MR][kPitch] (rows past 4 MR are read as
   // whatever the neighbour holds: they only feed output columns that are never stored)
@@ -180,7 +198,44 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
         acc[t][i] = sum;
       }
   }
-  if (n16 < M) {
+  if constexpr (EPI == kQkv) {
+    // the lane's four columns are channels d .. d+3 of one head (the host checks head_dim % 4 == 0
+    // and N % 4 == 0): two rotary pairs
+    const int n = n0 + 4 * g4;
+    if (n16 < M && n < N) {
+      const int head = n / qa.head_dim;
+      const int d = n % qa.head_dim;
+      float x[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] = to_f32(from_f32<bf16_t>(acc[0][i]));  // as the stored product would read
+      if (head < qa.n_q_heads + qa.n_kv_heads) {
+#pragma unroll
+        for (int pi = 0; pi < 2; ++pi) {
+          if (d + 2 * pi < qa.rotary_dim) {
+            const float2 cs = qa.cos_sin[(size_t)n16 * (qa.rotary_dim / 2) + (d / 2 + pi)];
+            const float x0 = x[2 * pi], x1 = x[2 * pi + 1];
+            x[2 * pi] = x0 * cs.x - x1 * cs.y;
+            x[2 * pi + 1] = x1 * cs.x + x0 * cs.y;
+          }
+        }
+      }
+      const u32x2_t packed = {
+          (uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x[0])) | ((uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x[1])) << 16),
+          (uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x[2])) | ((uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x[3])) << 16)};
+      bf16_t* dst = reinterpret_cast<bf16_t*>(C) + (size_t)n16 * ldc + n;
+      bool store = true;
+      if (head >= qa.n_q_heads && qa.k_pages != nullptr) {
+        const int slot = qa.slot_mapping[n16];
+        store = slot >= 0;
+        const int kvh = head < qa.n_q_heads + qa.n_kv_heads ? head - qa.n_q_heads : head - qa.n_q_heads - qa.n_kv_heads;
+        bf16_t* pages = head < qa.n_q_heads + qa.n_kv_heads ? qa.k_pages : qa.v_pages;
+        const int page = store ? slot / qa.page_size : 0;
+        const int off = store ? slot % qa.page_size : 0;
+        dst = pages + (((size_t)page * qa.n_kv_heads + kvh) * qa.page_size + off) * qa.head_dim + d;
+      }
+      if (store) *reinterpret_cast<u32x2_t*>(dst) = packed;
+    }
+  } else if (n16 < M) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int n = n0 + 4 * g4 + i;
@@ -197,43 +252,44 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   }
 }
 
-template <int MR, int WAVES, typename OutT, bool GLU>
+template <int MR, int WAVES, typename OutT, int EPI>
 int launch_typed(const bf16_t* A, int lda, const bf16_t* W, int ldw, OutT* C, int ldc, int M, int N, int K,
-                 hipStream_t stream) {
+                 const QkvArgs& qa, hipStream_t stream) {
   const size_t lds = (size_t)WAVES * 2 * kTileElems * sizeof(bf16_t);
   static bool raised = false;  // blocks past 64 KB of LDS have to be allowed once per kernel
   if (lds > 64 * 1024 && !raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<MR, WAVES, OutT, GLU>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_stream_kernel<MR, WAVES, OutT, EPI>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "gemm_stream: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     raised = true;
   }
   const dim3 grid((N + kStrip - 1) / kStrip);
-  gemm_stream_kernel<MR, WAVES, OutT, GLU><<<grid, WAVES * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  gemm_stream_kernel<MR, WAVES, OutT, EPI><<<grid, WAVES * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, qa);
   return tl_check_launch("gemm_stream");
 }
 
 template <int MR, int WAVES>
 int launch(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N, int K,
-           int out_dtype, bool glu, hipStream_t stream) {
-  if (glu) return launch_typed<MR, WAVES, bf16_t, true>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, stream);
-  if (out_dtype == TL_BF16) return launch_typed<MR, WAVES, bf16_t, false>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, stream);
-  return launch_typed<MR, WAVES, float, false>(A, lda, W, ldw, (float*)C, ldc, M, N, K, stream);
+           int out_dtype, int epi, const QkvArgs& qa, hipStream_t stream) {
+  if (epi == kGated) return launch_typed<MR, WAVES, bf16_t, kGated>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
+  if (epi == kQkv) return launch_typed<MR, WAVES, bf16_t, kQkv>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
+  if (out_dtype == TL_BF16) return launch_typed<MR, WAVES, bf16_t, kPlain>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
+  return launch_typed<MR, WAVES, float, kPlain>(A, lda, W, ldw, (float*)C, ldc, M, N, K, qa, stream);
 }
 
 template <int MR>
 int launch_waves(int waves, const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N,
-                 int K, int out_dtype, bool glu, hipStream_t stream) {
+                 int K, int out_dtype, int epi, const QkvArgs& qa, hipStream_t stream) {
   switch (waves) {
-    case 1: return launch<MR, 1>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
-    case 2: return launch<MR, 2>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
-    case 4: return launch<MR, 4>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
-    default: return launch<MR, 8>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
+    case 1: return launch<MR, 1>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
+    case 2: return launch<MR, 2>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
+    case 4: return launch<MR, 4>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
+    default: return launch<MR, 8>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
   }
 }
 
 int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K, int out_dtype,
-        int waves, bool glu, hipStream_t stream) {
+        int waves, int epi, const QkvArgs& qa, hipStream_t stream) {
   TL_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_stream: bad sizes M=%d N=%d K=%d", M, N, K);
   if (M > 16) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream: M=%d exceeds 16", M);
   if (K % 8) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream: K=%d is not a multiple of 8", K);
@@ -252,9 +308,9 @@ int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M,
   TL_REQUIRE(waves == 1 || waves == 2 || waves == 4 || waves == 8, "gemm_stream: waves must be 1, 2, 4 or 8");
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  if (M <= 4) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
-  if (M <= 8) return launch_waves<2>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
-  return launch_waves<4>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, glu, stream);
+  if (M <= 4) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
+  if (M <= 8) return launch_waves<2>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
+  return launch_waves<4>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
 }
 
 }  // namespace
@@ -264,7 +320,7 @@ int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M,
 // waves = 0 picks the number of K splits from the sizes.
 TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
                              int K, int out_dtype, int waves, hipStream_t stream) {
-  return run(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, waves, false, stream);
+  return run(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, waves, kPlain, QkvArgs{}, stream);
 }
 
 // The gated pair of products: W [2 N, K] = gate rows | up rows; C [M, N] bfloat16 =
@@ -272,5 +328,27 @@ TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, voi
 // would be if each were stored in bfloat16.
 TL_EXPORT int tl_gemm_stream_glu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
                                  int K, int waves, hipStream_t stream) {
-  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, true, stream);
+  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, kGated, QkvArgs{}, stream);
+}
+
+// The query/key/value projection with the rotary kernel's work in its epilogue.  W [(Hq + 2 Hkv) *
+// head_dim, K]; C [M, that width] receives the rotated queries (and keys and values when no pages are
+// given).  cos_sin [M][rotary_dim / 2][2]: cosine and sine of each row's position (interleaved pairs
+// only).  k_pages / v_pages [page][Hkv][page_size][head_dim]; slot_mapping [M].  head_dim % 4 == 0.
+TL_EXPORT int tl_gemm_stream_qkv(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int K,
+                                 int n_q_heads, int n_kv_heads, int head_dim, int rotary_dim,
+                                 const float* cos_sin, void* k_pages, void* v_pages,
+                                 const int32_t* slot_mapping, int page_size, int waves, hipStream_t stream) {
+  TL_REQUIRE(n_q_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && head_dim % 4 == 0, "gemm_stream_qkv: bad head sizes");
+  TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "gemm_stream_qkv: bad rotary_dim=%d", rotary_dim);
+  TL_REQUIRE(rotary_dim == 0 || cos_sin != nullptr, "gemm_stream_qkv: the table of cosines and sines is missing");
+  TL_REQUIRE(k_pages == nullptr || (v_pages != nullptr && slot_mapping != nullptr && page_size > 0),
+             "gemm_stream_qkv: pages given without v_pages/slot_mapping/page_size");
+  TL_REQUIRE(ldc % 4 == 0 && ((uintptr_t)C % 8) == 0, "gemm_stream_qkv: rows of C must start on 8-byte boundaries");
+  QkvArgs qa;
+  qa.n_q_heads = n_q_heads; qa.n_kv_heads = n_kv_heads; qa.head_dim = head_dim; qa.rotary_dim = rotary_dim;
+  qa.cos_sin = (const float2*)cos_sin; qa.k_pages = (bf16_t*)k_pages; qa.v_pages = (bf16_t*)v_pages;
+  qa.slot_mapping = slot_mapping; qa.page_size = page_size;
+  const int N = (n_q_heads + 2 * n_kv_heads) * head_dim;
+  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, kQkv, qa, stream);
 }

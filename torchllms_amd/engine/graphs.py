@@ -69,6 +69,9 @@ class DecodeGraph:
         result = logits.clone()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
+        # what the eager run derived from the step's plan (tables of cosines, ...) belongs to that
+        # run: the recording has to contain the kernels that derive it anew from the fixed buffers
+        ctx.scratch.clear()
         # nothing may be destroyed while the stream is capturing: collect garbage now and keep the
         # collector off until the capture has ended
         gc.collect()

@@ -26,13 +26,15 @@ _U64 = c_uint64
 _CORE_SIGNATURES = {
     "tl_embed": [_P, _P, _P, _I, _I, _I, _P],
     "tl_rmsnorm": [_P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _I, _P],
-    "tl_rope_kv_write": [_P, _I, _I, _I, _I, _P, _P, _I, _I, _P, _P, _P, _I, _I, _P],
+    "tl_rope_table": [_P, _P, _I, _I, _P, _P],
+    "tl_rope_kv_write": [_P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _P],
     "tl_silu_mul": [_P, _P, _I, _I, _I, _P],
     "tl_add_bias": [_P, _P, _I, _I, _I, _I, _P],
     "tl_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "tl_gemm_f32": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+    "tl_gemm_stream_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _P],
     "tl_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P],
     "tl_philox_uniform": [_U64, _U64, _P, _I, _P],
 }

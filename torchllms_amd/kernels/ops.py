@@ -90,6 +90,19 @@ def rmsnorm(
     return (h_out, y) if return_sum else y
 
 
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """float32 [n, len(inv_freq), 2]: cosine and sine of ``float(position) * inv_freq`` (32-bit angle,
+    precise functions).  One table serves every layer of a step that rotates alike."""
+    _gpu(positions, inv_freq)
+    _i32(positions, "positions")
+    if inv_freq.dtype != torch.float32 or inv_freq.dim() != 1 or not inv_freq.is_contiguous() or inv_freq.numel() == 0:
+        raise KernelError("inv_freq must be a contiguous float32 vector")
+    n, half = positions.numel(), inv_freq.numel()
+    out = torch.empty((n, half, 2), dtype=torch.float32, device=positions.device)
+    check(core().tl_rope_table(positions.data_ptr(), inv_freq.data_ptr(), n, half, out.data_ptr(), _stream()))
+    return out
+
+
 def rope_kv_write(
     qkv: torch.Tensor,
     n_q_heads: int,
@@ -103,10 +116,14 @@ def rope_kv_write(
     v_pages: Optional[torch.Tensor] = None,
     slot_mapping: Optional[torch.Tensor] = None,
     page_size: int = 0,
+    cos_sin: Optional[torch.Tensor] = None,
 ) -> None:
     """Rotate the query and key heads of ``qkv`` [n, (Hq + 2 Hkv) * dh] by position and store keys
-    and values into pages [pages, Hkv, page_size, dh] at ``slot_mapping`` (page * page_size + offset)."""
-    _gpu(qkv, positions, inv_freq, k_pages, v_pages, slot_mapping)
+    and values into pages [pages, Hkv, page_size, dh] at ``slot_mapping`` (page * page_size + offset).
+    ``cos_sin``: the step's ``rope_table`` for these positions, instead of forming the angles here."""
+    _gpu(qkv, positions, inv_freq, k_pages, v_pages, slot_mapping, cos_sin)
+    if cos_sin is not None and (cos_sin.dtype != torch.float32 or tuple(cos_sin.shape) != (qkv.shape[0], rotary_dim // 2, 2) or not cos_sin.is_contiguous()):
+        raise KernelError(f"cos_sin must be contiguous float32 [{qkv.shape[0]}, {rotary_dim // 2}, 2]")
     _i32(positions, "positions")
     _i32(slot_mapping, "slot_mapping")
     n = qkv.shape[0]
@@ -115,7 +132,7 @@ def rope_kv_write(
         raise KernelError(f"qkv must be contiguous [n, {width}], got {tuple(qkv.shape)}")
     if positions.numel() != n:
         raise KernelError("positions must have one entry per token")
-    if rotary_dim > 0:
+    if rotary_dim > 0 and cos_sin is None:
         if inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2 or not inv_freq.is_contiguous():
             raise KernelError(f"inv_freq must be float32 with {rotary_dim // 2} entries")
     if k_pages is not None:
@@ -128,7 +145,7 @@ def rope_kv_write(
                 )
     check(
         core().tl_rope_kv_write(
-            qkv.data_ptr(), n, n_q_heads, n_kv_heads, head_dim, positions.data_ptr(), _ptr(inv_freq),
+            qkv.data_ptr(), n, n_q_heads, n_kv_heads, head_dim, positions.data_ptr(), _ptr(inv_freq), _ptr(cos_sin),
             rotary_dim, pairing, _ptr(k_pages), _ptr(v_pages), _ptr(slot_mapping), page_size,
             dtype_code(qkv.dtype), _stream(),
         )
@@ -256,6 +273,51 @@ def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0) -> torch.T
     return out
 
 
+def gemm_stream_qkv(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    rotary_dim: int,
+    cos_sin: Optional[torch.Tensor],
+    k_pages: Optional[torch.Tensor],
+    v_pages: Optional[torch.Tensor],
+    slot_mapping: Optional[torch.Tensor],
+    page_size: int,
+    waves: int = 0,
+) -> torch.Tensor:
+    """The fused projection ``x @ w.T`` of at most 16 rows into query | key | value heads with the
+    rotation (interleaved pairs, from the ``rope_table`` of the rows' positions) and the cache
+    write in the kernel's epilogue.  Returns [n, (Hq + 2 Hkv) * dh] whose query part is rotated;
+    the key and value parts are only filled when no pages are given."""
+    _gpu(x, w, cos_sin, k_pages, v_pages, slot_mapping)
+    _i32(slot_mapping, "slot_mapping")
+    width = (n_q_heads + 2 * n_kv_heads) * head_dim
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("gemm_stream_qkv takes bfloat16 tensors")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1 or w.shape[0] != width:
+        raise KernelError(f"gemm_stream_qkv: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match {width} output columns")
+    m, k = x.shape
+    if rotary_dim > 0 and (cos_sin is None or cos_sin.dtype != torch.float32 or tuple(cos_sin.shape) != (m, rotary_dim // 2, 2) or not cos_sin.is_contiguous()):
+        raise KernelError(f"cos_sin must be contiguous float32 [{m}, {rotary_dim // 2}, 2]")
+    if k_pages is not None:
+        if v_pages is None or slot_mapping is None or slot_mapping.numel() != m:
+            raise KernelError("pages need v_pages and one slot per row")
+        for pg in (k_pages, v_pages):
+            if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != torch.bfloat16 or not pg.is_contiguous():
+                raise KernelError(f"pages must be contiguous bfloat16 [pages, {n_kv_heads}, {page_size}, {head_dim}], got {tuple(pg.shape)} {pg.dtype}")
+    out = torch.empty((m, width), dtype=torch.bfloat16, device=x.device)
+    check(
+        core().tl_gemm_stream_qkv(
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, k,
+            n_q_heads, n_kv_heads, head_dim, rotary_dim, _ptr(cos_sin), _ptr(k_pages), _ptr(v_pages),
+            _ptr(slot_mapping), page_size, waves, _stream(),
+        )
+    )
+    return out
+
+
 def stream_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether the weight-streaming kernel can take this product at all."""
     return (
@@ -354,6 +416,44 @@ def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         if waves is not None:
             return gemm_stream_glu(x, w, waves)
     return silu_mul(linear(x, w))
+
+
+def qkv_rope_store(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    positions: torch.Tensor,
+    inv_freq: Optional[torch.Tensor],
+    rotary_dim: int,
+    pairing: int,
+    cos_sin: Optional[torch.Tensor],
+    k_pages: Optional[torch.Tensor],
+    v_pages: Optional[torch.Tensor],
+    slot_mapping: Optional[torch.Tensor],
+    page_size: int,
+) -> torch.Tensor:
+    """Projection into query | key | value heads, rotation of queries and keys by position, keys
+    and values appended to their pages; returns the row-major [n, (Hq + 2 Hkv) * dh] buffer whose
+    query part the attention kernels read.  One fused kernel where the weight-streaming kernel
+    serves the product (few bfloat16 rows, no bias, interleaved pairs, head size a multiple of 4),
+    else product, bias and rotary kernels in turn."""
+    if x.dtype == torch.bfloat16 and bias is None and (rotary_dim == 0 or pairing == 0) and head_dim % 4 == 0:
+        waves = stream_choice(x, w)
+        if waves is not None and (rotary_dim == 0 or cos_sin is not None):
+            return gemm_stream_qkv(
+                x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size, waves
+            )
+    qkv = linear(x, w)
+    if bias is not None:
+        add_bias_(qkv, bias)
+    rope_kv_write(
+        qkv, n_q_heads, n_kv_heads, head_dim, positions, inv_freq, rotary_dim, pairing, k_pages, v_pages,
+        slot_mapping, page_size, cos_sin=cos_sin,
+    )
+    return qkv
 
 
 def sample(

@@ -86,14 +86,21 @@ class Attention(Mixer):
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         n_kv_in_row = 0 if self.shares_kv else self.num_kv_heads
-        qkv = ops.linear(x, self.wqkv)
-        if self.bqkv is not None:
-            ops.add_bias_(qkv, self.bqkv)
         rot = self.position.rotary_args()
         g = cache.group
         store = cache.writes and not self.shares_kv
-        ops.rope_kv_write(
-            qkv,
+        # cosines and sines of this step's positions: made once per step and shared by every layer
+        # whose position encoding has the same frequencies
+        table = None
+        if rot is not None and rot.rotary_dim > 0:
+            key = ("rope_table", rot.inv_freq.data_ptr())
+            table = ctx.scratch.get(key)
+            if table is None:
+                table = ctx.scratch[key] = ops.rope_table(ctx.positions, rot.inv_freq)
+        qkv = ops.qkv_rope_store(
+            x,
+            self.wqkv,
+            self.bqkv,
             self.num_heads,
             n_kv_in_row,
             self.head_dim,
@@ -101,6 +108,7 @@ class Attention(Mixer):
             rot.inv_freq if rot else None,
             rot.rotary_dim if rot else 0,
             rot.pairing if rot else 0,
+            table,
             cache.k_pages if store else None,
             cache.v_pages if store else None,
             ctx.slot_mappings[g] if store else None,

@@ -50,12 +50,17 @@ def rotary_inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[
     return torch.where(in_band, blended, stretched)
 
 
+#: inverse frequencies on a device, by (device, values)
+_DEVICE_FREQUENCIES: Dict[Any, torch.Tensor] = {}
+
+
 @POSITIONS.register("rope")
 class RotaryEmbedding(PositionEncoding):
     """Rotation of (query, key) channel pairs by ``position * inv_freq`` in 32-bit
     (reference: torchllms/models/networks.py:284-352 builds a cos/sin table and rotates
-    interleaved pairs; here the angle is formed per token inside the kernel from the same
-    32-bit product)."""
+    interleaved pairs over all positions; here the cosines and sines of a step's positions are
+    formed from the same 32-bit product, once per step).  Instances with equal frequencies share
+    one device tensor, so that the layers of a model also share the step's table."""
 
     def __init__(self, head_dim: int, rotary_dim: int, theta: float, scaling: Optional[Dict[str, Any]], pairing: str = "interleaved"):
         if rotary_dim % 2 or rotary_dim > head_dim:
@@ -71,7 +76,11 @@ class RotaryEmbedding(PositionEncoding):
         self._device_args: Optional[RotaryArgs] = None
 
     def to(self, device) -> None:
-        self._device_args = RotaryArgs(self.inv_freq.to(device).contiguous(), self.rotary_dim, PAIRING[self.pairing])
+        key = (str(torch.device(device)), self.inv_freq.numpy().tobytes())
+        freqs = _DEVICE_FREQUENCIES.get(key)
+        if freqs is None:
+            freqs = _DEVICE_FREQUENCIES[key] = self.inv_freq.to(device).contiguous()
+        self._device_args = RotaryArgs(freqs, self.rotary_dim, PAIRING[self.pairing])
 
     def rotary_args(self) -> Optional[RotaryArgs]:
         return self._device_args
