@@ -4,12 +4,15 @@
 //   * a block of 4 waves takes a tile of consecutive queries of one request and one kv head, with
 //     all query heads that share it: its 128 MFMA columns are (query, head) pairs, so a key or value
 //     is fetched once for the whole group.
-//   * keys and values stream through LDS in tiles of 64 keys.  Keys lie there as in the page, values
-//     transposed (channel-major), so that both are MFMA A operands that a lane reads with one
-//     contiguous LDS load.
-//   * scores are computed transposed, S^T[key][column] = K Q^T, by MFMA 16x16x16 bf16; their output
-//     layout is exactly the B-operand layout of P^T in O^T[channel][column] = V^T P^T, so the
-//     probabilities never leave their registers.  Softmax statistics are 32-bit, per column.
+//   * keys and values stream through LDS in tiles of 64 keys, both as they lie in the page.
+//   * scores are computed transposed, S^T[key][column] = K Q^T, by MFMA 16x16x32 bf16 (a lane's 16
+//     bytes of a key row are one operand); their output layout, taken over two blocks of 16 keys, is
+//     exactly the B-operand layout of P^T in O^T[channel][column] = V^T P^T, so the probabilities
+//     never leave their registers.  Softmax statistics are 32-bit, per column.
+//   * the A operand of the second product wants, per lane, one channel of eight keys.  A lane reads
+//     from each of its eight key rows the DH/16 consecutive channels (DH/16) * n16 ...; the operand of
+//     output block b is channel b of the eight rows (four byte permutes).  Row m of output block b is
+//     therefore channel (DH/16) * m + b: a renaming that makes a lane's results contiguous in memory.
 //   * every column has its own causal limit (its query's position) and window start.
 //
 // Compiled once per head size (-DTL_HEAD_DIM=32|64|128|256).
@@ -48,8 +51,7 @@ constexpr int KT = DH <= 128 ? 64 : 32;       // keys per LDS tile
 constexpr int KL = DH / 32;                  // 16-byte pieces of a key row per lane
 constexpr int DT = DH / 16;                  // channel tiles of the output
 constexpr int kKPitch = DH + 8;              // bf16 elements per key row in LDS
-constexpr int kVPitch = KT + 2;              // bf16 elements per channel row in LDS: an odd number of
-                                             // dwords, so the transposed 16-bit writes spread over the banks
+constexpr int kVWords = DT / 2;              // 32-bit words a lane reads from one value row (DT channels)
 constexpr int kChunksPerRow = DH / 8;        // 16-byte chunks in a key/value row
 constexpr int kLoadsPerThread = KT * kChunksPerRow / kThreads;
 static_assert(KT * kChunksPerRow % kThreads == 0, "tile does not divide over the block");
@@ -77,29 +79,48 @@ struct PrefillArgs {
 
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
-// 16 bytes as they come from memory; the two halves are MFMA operands
+// 16 bytes as they come from memory = eight bfloat16 = one operand of the 16x16x32 MFMA
 struct Pack16 {
   u32x4_t u;
-  __device__ __forceinline__ short4_t half(int e) const {
-    return __builtin_bit_cast(short4_t, e == 0 ? u32x2_t{u[0], u[1]} : u32x2_t{u[2], u[3]});
-  }
+  __device__ __forceinline__ bf16x8_t op() const { return __builtin_bit_cast(bf16x8_t, u); }
 };
 
-__device__ __forceinline__ uint32_t bf16_bits(float x) {
-  return (uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x));
+// two floats -> two bfloat16 in one 32-bit word (first in the low half), round to nearest even
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{a, b}, bf16x2_t));
 }
-// two floats -> two bfloat16 in one 32-bit word (first in the low half)
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) { return bf16_bits(a) | (bf16_bits(b) << 16); }
+
+// W consecutive 32-bit words from LDS (W = 1, 2, 4 or 8)
+template <int W>
+__device__ __forceinline__ void lds_words(const bf16_t* src, uint32_t* dst) {
+  if constexpr (W == 1) {
+    dst[0] = *reinterpret_cast<const uint32_t*>(src);
+  } else if constexpr (W == 2) {
+    const u32x2_t v = *reinterpret_cast<const u32x2_t*>(src);
+    dst[0] = v[0];
+    dst[1] = v[1];
+  } else {
+#pragma unroll
+    for (int i = 0; i < W / 4; ++i) {
+      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + 8 * i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dst[4 * i + e] = v[e];
+    }
+  }
+}
 
 template <int RP>
 __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[KT * kKPitch];
-  __shared__ __attribute__((aligned(16))) bf16_t vt_lds[DH * kVPitch];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[KT * kKPitch];
   constexpr int QB = kCols / RP;  // queries per block
 
-  const int tile = gridDim.x - 1 - blockIdx.x;  // late query tiles see the most keys: start them first
-  const int kvh = blockIdx.y;
+  const int tile = blockIdx.y;  // the host lists the tiles in the order that balances the launch
+  const int kvh = blockIdx.x;
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   const int n16 = lane % 16;
@@ -191,9 +212,7 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
       const int key = id / kChunksPerRow;
       const int dc = id % kChunksPerRow;
       *reinterpret_cast<u32x4_t*>(&k_lds[key * kKPitch + 8 * dc]) = kst[j].u;
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        reinterpret_cast<uint16_t*>(vt_lds)[(8 * dc + e) * kVPitch + key] = (uint16_t)(vst[j].u[e / 2] >> (16 * (e & 1)));
+      *reinterpret_cast<u32x4_t*>(&v_lds[key * kKPitch + 8 * dc]) = vst[j].u;
     }
   };
 
@@ -230,15 +249,13 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
 #pragma unroll
       for (int u = 0; u < KL; ++u)
 #pragma unroll
-        for (int i = 0; i < NC; ++i) {
-          c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[u].half(0), qreg[i][u].half(0), c[i][sub], 0, 0, 0);
-          c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[u].half(1), qreg[i][u].half(1), c[i][sub], 0, 0, 0);
-        }
+        for (int i = 0; i < NC; ++i)
+          c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[u].op(), qreg[i][u].op(), c[i][sub], 0, 0, 0);
     }
     // softmax bookkeeping once per chunk and column: mask, maximum, rescale, probabilities.
     // Scores stay unscaled; the scale enters through one fused multiply-add per element:
     // exp2(s * scale - m), with m the running maximum of s * scale.
-    short4_t pb[NC][NS];
+    bf16x8_t pb[NC];  // slot e < 4: key 4 g4 + e of the first 16 keys; e >= 4: the same of the second 16
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
       // keys of the chunk that every lane of this column sees need no test at all
@@ -263,6 +280,7 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
       const float alpha = none ? 1.f : __builtin_amdgcn_exp2f(m_run[i] - m_new);
       const float neg_m = none ? 0.f : -m_new;
       float psum = 0.f;
+      uint32_t pw[2 * NS];
 #pragma unroll
       for (int sub = 0; sub < NS; ++sub) {
         float pr[4];
@@ -271,25 +289,40 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
           pr[r] = __builtin_amdgcn_exp2f(fmaf(c[i][sub][r], a.scale_log2e, neg_m));  // exp2(-inf) = 0
           psum += pr[r];
         }
-        pb[i][sub] = __builtin_bit_cast(short4_t, u32x2_t{pack_bf16x2(pr[0], pr[1]), pack_bf16x2(pr[2], pr[3])});
+        pw[2 * sub] = pack_bf16x2(pr[0], pr[1]);
+        pw[2 * sub + 1] = pack_bf16x2(pr[2], pr[3]);
       }
+      pb[i] = __builtin_bit_cast(bf16x8_t, u32x4_t{pw[0], pw[1], pw[2], pw[3]});
       l_part[i] = l_part[i] * alpha + psum;
       m_run[i] = m_new;
+      // the sums so far are rescaled only when some column's maximum has moved
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
-      for (int t = 0; t < DT; ++t)
+        for (int t = 0; t < DT; ++t)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha;
+          for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha;
+      }
     }
-    // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column]
+    // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column] over the chunk's 32 keys.
+    // A block of 16 keys that no column of the wave sees has zero probabilities: its rows are read
+    // all the same (they lie in the tile) and add nothing.
+    {
+      uint32_t vrow[8][kVWords];
 #pragma unroll
-    for (int sub = 0; sub < NS; ++sub) {
-      if (!live[sub]) continue;
+      for (int e = 0; e < 8; ++e) {
+        const int key = 16 * NS * chunk + 16 * (e / 4) + 4 * g4 + (e % 4);  // within the tile
+        lds_words<kVWords>(&v_lds[key * kKPitch + DT * n16], vrow[e]);
+      }
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
-        const uint32_t* vp = reinterpret_cast<const uint32_t*>(&vt_lds[(16 * t + n16) * kVPitch + 16 * (NS * chunk + sub) + 4 * g4]);
-        const short4_t va = __builtin_bit_cast(short4_t, u32x2_t{vp[0], vp[1]});
+        const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;  // the odd or the even halves of two words
+        const u32x4_t vw = {__builtin_amdgcn_perm(vrow[1][t / 2], vrow[0][t / 2], sel),
+                            __builtin_amdgcn_perm(vrow[3][t / 2], vrow[2][t / 2], sel),
+                            __builtin_amdgcn_perm(vrow[5][t / 2], vrow[4][t / 2], sel),
+                            __builtin_amdgcn_perm(vrow[7][t / 2], vrow[6][t / 2], sel)};
+        const bf16x8_t va = __builtin_bit_cast(bf16x8_t, vw);
 #pragma unroll
-        for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(va, pb[i][sub], acc[i][t], 0, 0, 0);
+        for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[i], acc[i][t], 0, 0, 0);
       }
     }
     }  // chunk
@@ -303,11 +336,22 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
     if (!col_ok[i]) continue;
     const float inv = 1.0f / l;
     bf16_t* orow = a.out + (size_t)col_tok[i] * a.out_stride + (size_t)col_head[i] * DH;
+    // acc[i][t][r] is channel DT * (4 g4 + r) + t: for each r the DT output blocks are contiguous
 #pragma unroll
-    for (int t = 0; t < DT; ++t) {
-      const uint2 o = make_uint2(pack_bf16x2(acc[i][t][0] * inv, acc[i][t][1] * inv),
-                                 pack_bf16x2(acc[i][t][2] * inv, acc[i][t][3] * inv));
-      *reinterpret_cast<uint2*>(orow + 16 * t + 4 * g4) = o;
+    for (int r = 0; r < 4; ++r) {
+      uint32_t w[kVWords];
+#pragma unroll
+      for (int t = 0; t < DT; t += 2) w[t / 2] = pack_bf16x2(acc[i][t][r] * inv, acc[i][t + 1][r] * inv);
+      bf16_t* dst = orow + DT * (4 * g4 + r);
+      if constexpr (kVWords == 1) {
+        *reinterpret_cast<uint32_t*>(dst) = w[0];
+      } else if constexpr (kVWords == 2) {
+        *reinterpret_cast<u32x2_t*>(dst) = u32x2_t{w[0], w[1]};
+      } else {
+#pragma unroll
+        for (int j = 0; j < kVWords / 4; ++j)
+          *reinterpret_cast<u32x4_t*>(dst + 8 * j) = u32x4_t{w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
+      }
     }
   }
 }
@@ -334,11 +378,11 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   if (n_q_heads % n_kv_heads) return variant_fail(TL_ERR_ARG, "attn_prefill: %d query heads are not a multiple of %d kv heads", n_q_heads, n_kv_heads);
   const int R = n_q_heads / n_kv_heads;
   if (R > 16) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: %d query heads per kv head exceed 16", R);
-  if (n_kv_heads > 65535) return variant_fail(TL_ERR_ARG, "attn_prefill: grid out of range");
+  if (n_tiles > 65535) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: %d query tiles exceed a launch's 65535", n_tiles);
   // the running maximum is taken over raw scores and scaled afterwards
   if (!(scale > 0.f)) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: softmax scale %g must be positive", (double)scale);
-  if (q_stride % 8 || ((uintptr_t)q % 16) || out_stride % 4 || ((uintptr_t)out % 8))
-    return variant_fail(TL_ERR_ARG, "attn_prefill: queries need 16-byte aligned rows, outputs 8-byte aligned rows");
+  if (q_stride % 8 || ((uintptr_t)q % 16) || out_stride % 8 || ((uintptr_t)out % 16))
+    return variant_fail(TL_ERR_ARG, "attn_prefill: queries and outputs need 16-byte aligned rows");
   if (n_tiles == 0) return TL_OK;
   PrefillArgs a;
   a.q = (const bf16_t*)q; a.q_stride = q_stride; a.out = (bf16_t*)out; a.out_stride = out_stride;
@@ -350,7 +394,7 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   for (int sh = 0; sh < 31; ++sh)
     if ((1 << sh) == page_size) a.page_shift = sh;
   a.scale_log2e = scale * 1.4426950408889634f;
-  dim3 grid(n_tiles, n_kv_heads);
+  dim3 grid(n_kv_heads, n_tiles);  // consecutive blocks share a query tile: their loads of q overlap
   if (R == 1) attn_prefill_kernel<1><<<grid, kThreads, 0, stream>>>(a);
   else if (R == 2) attn_prefill_kernel<2><<<grid, kThreads, 0, stream>>>(a);
   else if (R <= 4) attn_prefill_kernel<4><<<grid, kThreads, 0, stream>>>(a);

@@ -59,12 +59,13 @@ def paged_attention(
     if n_dec < n:
         if fast_prefill:
             qpt = ops.prefill_queries_per_tile(n_q_heads, n_kv_heads, head_dim)
-            tiles = ctx.scratch.get(("prefill_tiles", qpt))
+            key = ("prefill_tiles", qpt, window, n_kv_heads)
+            tiles = ctx.scratch.get(key)
             if tiles is None:
-                rows, q0s = ops.prefill_tiles(ctx.host.qo_indptr, n_dec, ctx.host.n_seqs, qpt)
+                rows, q0s = ops.prefill_tiles(ctx.host.qo_indptr, n_dec, ctx.host.n_seqs, qpt, ctx.host.kv_lens, window, n_kv_heads)
                 both = torch.tensor([rows, q0s], dtype=torch.int32).to(qkv.device)
                 tiles = (both[0], both[1])
-                ctx.scratch[("prefill_tiles", qpt)] = tiles
+                ctx.scratch[key] = tiles
             ops.attention_prefill(
                 qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.qo_indptr, ctx.kv_lens,
                 ctx.block_tables[group], tiles[0], tiles[1], window, scale, out,

@@ -605,15 +605,37 @@ def prefill_queries_per_tile(n_q_heads: int, n_kv_heads: int, head_dim: int) -> 
     return (128 if head_dim <= 128 else 64) // rp
 
 
-def prefill_tiles(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int):
-    """Host lists ``(tile_row, tile_q0)`` that cut rows ``first_row .. n_rows-1`` into query tiles."""
-    rows, q0s = [], []
+#: blocks of the prefill kernel that the GPU holds at once: 256 CUs, two blocks each
+PREFILL_RESIDENT_BLOCKS = 512
+
+
+def prefill_tiles(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int, kv_lens=None, window: int = 0,
+                  n_kv_heads: int = 1):
+    """Host lists ``(tile_row, tile_q0)`` that cut rows ``first_row .. n_rows-1`` into query tiles.
+
+    With ``kv_lens`` the tiles are put in the order that balances the launch: a tile's cost is the
+    number of keys it sees, and late tiles of a causal prompt see many times more than early ones.
+    Blocks are handed to the CUs in launch order.  When there are far more blocks than fit at once,
+    longest first lets short ones fill the gaps at the end; when about all fit at once, the first
+    half of the launch takes the long tiles in descending order and the second half the short ones in
+    ascending order, so that the blocks that meet on a CU have complementary lengths."""
+    rows, q0s, costs = [], [], []
     for r in range(first_row, n_rows):
         q_len = int(qo_indptr[r + 1]) - int(qo_indptr[r])
+        pos0 = (int(kv_lens[r]) - q_len) if kv_lens is not None else 0
         for q0 in range(0, q_len, queries_per_tile):
             rows.append(r)
             q0s.append(q0)
-    return rows, q0s
+            hi = pos0 + min(q0 + queries_per_tile, q_len) - 1
+            lo = max(pos0 + q0 - window + 1, 0) if window > 0 else 0
+            costs.append(hi - lo + 1)
+    if kv_lens is None or len(rows) < 2:
+        return rows, q0s
+    order = sorted(range(len(rows)), key=lambda i: -costs[i])
+    if len(rows) * n_kv_heads <= 2 * PREFILL_RESIDENT_BLOCKS:
+        half = (len(order) + 1) // 2
+        order = order[:half] + order[half:][::-1]
+    return [rows[i] for i in order], [q0s[i] for i in order]
 
 
 def attention_prefill(
