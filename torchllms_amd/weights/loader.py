@@ -132,7 +132,6 @@ def load_weights(
                     t = rule.load(t)
                 t = t.to(dtype=_final_dtype(spec, t.dtype, dtype)).contiguous()
                 out[internal] = t.to(device) if str(device) != "cpu" else t
-    missing_internal = [n for n in expected if n not in out and n not in {w[0] for w in wrong}]
     # report missing tensors under the names a checkpoint would use
     wrong_internal = set()
     for ext_name, _, _ in wrong:
