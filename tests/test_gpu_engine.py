@@ -201,3 +201,60 @@ def test_step_refuses_what_it_cannot_run(cases):
     eng.free("x")
     eng.free("y")
     eng.cache.check_invariants()
+
+
+def test_decode_steps_planned_from_the_last_plan_equal_the_general_plan(cases):
+    """A decode step that follows a decode step of the same requests is planned from that step's
+    plan.  Both planners are run side by side on two engines through starts of pages, a request
+    that ends, one that joins, a step with a prompt portion in between and a changed `want`."""
+    import numpy as np
+
+    from torchllms_amd.engine import Engine, StepEntry
+
+    case = cases["B"]
+    page = 4
+    engines = [Engine.from_folder(case.folder, dtype="float32", page_size=page, num_pages=64, max_seqs=4, use_graphs=False) for _ in range(2)]
+    fast, general = engines
+    rng = torch.Generator().manual_seed(5)
+
+    def both(entries):
+        general._last_decode = None  # this engine always plans from scratch
+        la, lb = fast.plan(entries), general.plan(entries)
+        for name in ("tokens", "positions", "token_seq", "qo_indptr", "kv_lens", "slot_ids", "logit_rows"):
+            assert np.array_equal(getattr(la, name), getattr(lb, name)), name
+        assert (la.n_tokens, la.n_seqs, la.n_decode, la.max_q_len, la.max_kv_len) == (lb.n_tokens, lb.n_seqs, lb.n_decode, lb.max_q_len, lb.max_kv_len)
+        for g in range(len(la.block_tables)):
+            assert np.array_equal(la.slot_mappings[g], lb.slot_mappings[g])
+            wa, wb = la.block_tables[g].shape[1], lb.block_tables[g].shape[1]
+            w = min(wa, wb)
+            assert np.array_equal(la.block_tables[g][:, :w], lb.block_tables[g][:, :w])
+            assert (la.block_tables[g][:, w:] == -1).all() and (lb.block_tables[g][:, w:] == -1).all()
+        for eng in engines:
+            for e in entries:
+                eng.cache.advance(e.rid, len(e.tokens))
+        return la
+
+    def tok():
+        return int(torch.randint(0, case.cfg["vocab_size"], (1,), generator=rng))
+
+    for eng in engines:
+        for rid in ("a", "b", "c"):
+            eng.admit(rid)
+    both([StepEntry("a", [tok() for _ in range(5)], [4]), StepEntry("b", [tok() for _ in range(3)], [2]), StepEntry("c", [tok()], [0])])
+    used_fast = 0
+    for step in range(30):
+        live = ["a", "b", "c"] if step < 12 else (["a", "c"] if step < 20 else ["a", "c", "d"])
+        if step == 12:
+            for eng in engines:
+                eng.free("b")
+        if step == 20:
+            for eng in engines:
+                eng.admit("d")
+            both([StepEntry("d", [tok(), tok()], [1])])
+        want = [] if step == 7 else [0]
+        before = fast._last_decode
+        layout = both([StepEntry(r, [tok()], want) for r in live])
+        used_fast += before is not None and fast._last_decode is not None and fast._last_decode[2] is layout and before[0] == tuple(live)
+    assert used_fast >= 15  # the shortcut did plan most of these steps
+    for eng in engines:
+        eng.cache.check_invariants()

@@ -446,6 +446,22 @@ def test_sample_greedy_and_ties():
     assert got.tolist() == logits.argmax(-1).tolist() and got[2] == 77
 
 
+@pytest.mark.parametrize("vocab", [128256, 40000, 16388, 4099])
+def test_sample_greedy_over_a_large_vocabulary(vocab):
+    """Wide loads, their unrolled part, their tail and the unaligned rows of an odd vocabulary; the
+    maximum is planted at the far end, at the start and twice (the lower index wins)."""
+    torch.manual_seed(1)
+    logits = torch.randn(6, vocab)
+    logits[0, vocab - 1] = 50.0
+    logits[1, 0] = 50.0
+    logits[2, vocab - 3] = logits[2, 5] = 50.0
+    mid = min(4 * 1024 * 3 + 2, vocab - 7)
+    logits[3, mid] = logits[3, vocab - 2] = 50.0
+    logits[4, vocab // 2 + 1] = 50.0
+    got = _sample(logits, [0.0] * 6, [1] * 6, [0] * 6)
+    assert got.tolist() == [vocab - 1, 0, 5, mid, vocab // 2 + 1, int(logits[5].argmax())]
+
+
 @pytest.mark.parametrize("vocab", [8, 301, 5000])
 def test_sample_temperature_matches_the_plain_rule(vocab):
     torch.manual_seed(0)

@@ -179,6 +179,9 @@ class CacheManager:
             n = num_pages[g.name] if isinstance(num_pages, dict) else num_pages
             self.pools.append(PagePool(int(n)))
         self._requests: Dict[Hashable, RequestEntry] = {}
+        #: counts admissions, releases and truncations: a plan made at one epoch describes the same
+        #: requests, slots and pages at the same epoch only
+        self.epoch = 0
         self._free_slots: List[int] = list(range(max_seqs - 1, -1, -1))
         # run id -> (group index, layer index inside the group) / (state index, layer index)
         self._run_to_kv: Dict[int, Tuple[int, int]] = {}
@@ -233,6 +236,7 @@ class CacheManager:
         if not self._free_slots:
             raise OutOfSlots(f"all {self.max_seqs} request slots are taken")
         slot = self._free_slots.pop()
+        self.epoch += 1
         self._requests[rid] = RequestEntry(
             slot=slot,
             block_tables=[[] for _ in self.groups],
@@ -355,12 +359,14 @@ class CacheManager:
             e.table_arrays[gi] = None
         e.num_tokens = num_tokens
         e.reserved_tokens = num_tokens
+        self.epoch += 1
 
     def free(self, rid: Hashable) -> None:
         """The request ends: all its pages and its slot go back."""
         e = self._requests.pop(rid, None)
         if e is None:
             raise KeyError(f"request {rid!r} is not live (freed twice?)")
+        self.epoch += 1
         for gi, pool in enumerate(self.pools):
             pool.give_back([p for p in e.block_tables[gi] if p >= 0])
         self._free_slots.append(e.slot)

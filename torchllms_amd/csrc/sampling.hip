@@ -93,7 +93,36 @@ sample_kernel(const float* __restrict__ logits, int row_stride, int vocab,
 
   if (temp == 0.f) {
     Best b = {-INFINITY, kNone};
-    for (int i = tid; i < vocab; i += kThreads) b = better(b, Best{x[i], i});
+    // 16-byte loads, four of them in flight per thread, where the row allows it; `better` keeps the
+    // lowest index among equal maxima whatever the order of the visits
+    int done = 0;
+    if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+      const int n4 = vocab / 4;
+      const float4* x4 = reinterpret_cast<const float4*>(x);
+      int i = tid;
+      for (; i + 3 * kThreads < n4; i += 4 * kThreads) {
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = x4[i + u * kThreads];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int at = 4 * (i + u * kThreads);
+          b = better(b, Best{v[u].x, at});
+          b = better(b, Best{v[u].y, at + 1});
+          b = better(b, Best{v[u].z, at + 2});
+          b = better(b, Best{v[u].w, at + 3});
+        }
+      }
+      for (; i < n4; i += kThreads) {
+        const float4 v = x4[i];
+        b = better(b, Best{v.x, 4 * i});
+        b = better(b, Best{v.y, 4 * i + 1});
+        b = better(b, Best{v.z, 4 * i + 2});
+        b = better(b, Best{v.w, 4 * i + 3});
+      }
+      done = 4 * n4;
+    }
+    for (int i = done + tid; i < vocab; i += kThreads) b = better(b, Best{x[i], i});
     b = block_best(b, best_scratch);
     if (tid == 0) out[row] = b.idx;
     return;

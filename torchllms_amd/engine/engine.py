@@ -13,6 +13,7 @@ from __future__ import annotations
 from pathlib import Path
 from typing import Dict, Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, OutOfPages, group_layers
@@ -84,8 +85,12 @@ class Engine:
             else:
                 num_pages = max_seqs * (-(-self.max_model_len // page_size))
         self.cache = CacheManager(groups, states, page_size, num_pages, max_seqs, dtype=dtype, device=self.device)
+        self._windowed = any(g.window > 0 for g in groups)
         self.steps_run = 0
         self.tokens_run = 0
+        # the last step's plan when every row of it brought one token: (request ids, wanted places,
+        # layout); a decode step that follows it with the same requests is planned from it
+        self._last_decode = None
         if dtype == torch.bfloat16 and tune_kernels:
             # which matrix-product kernel serves decode steps best is measured, not guessed
             from ..kernels import ops
@@ -141,8 +146,80 @@ class Engine:
         return self.cache.num_tokens(rid)
 
     # ------------------------------------------------------------------ the step
+    def _plan_next_decode(self, entries: Sequence[StepEntry]) -> Optional[StepLayout]:
+        """The plan of a decode step that follows a decode step of the same requests, made from
+        that step's plan: positions move on by one, a block table gains an entry where a page
+        begins.  None when the step is anything else (the general planner then checks and says
+        what is wrong with it)."""
+        last = self._last_decode
+        if last is None or len(entries) != len(last[0]):
+            return None
+        rids, wants, prev, epoch = last
+        cache = self.cache
+        if epoch != cache.epoch:
+            return None
+        n = len(entries)
+        tokens = np.empty(n, dtype=np.int32)
+        need = 0
+        for i, e in enumerate(entries):
+            if e.rid != rids[i] or len(e.tokens) != 1 or tuple(e.want) != wants[i]:
+                return None
+            tok = e.tokens[0]
+            if not 0 <= tok < self.vocab_size:
+                return None
+            if not cache.has(e.rid) or cache.num_tokens(e.rid) != int(prev.kv_lens[i]) or int(prev.kv_lens[i]) + 1 > self.max_model_len:
+                return None
+            tokens[i] = tok
+            need += cache.new_pages_needed(e.rid, 1)
+        if any(need > pool.free_count for pool in cache.pools):
+            return None
+        page = self.page_size
+        positions = prev.kv_lens.copy()  # the new token's position = tokens held so far
+        for e in entries:
+            cache.extend(e.rid, 1)
+        tables, slots = [], []
+        fresh = (positions % page) == 0  # rows whose new token opens a page
+        for g in range(len(cache.groups)):
+            bt = prev.block_tables[g]
+            sm = prev.slot_mappings[g] + 1
+            if fresh.any():
+                width = max(bt.shape[1], int(positions.max()) // page + 1)
+                wider = np.full((n, width), -1, dtype=np.int32)
+                wider[:, : bt.shape[1]] = bt
+                bt = wider
+                for i in np.nonzero(fresh)[0]:
+                    blk = int(positions[i]) // page
+                    bt[i, blk] = cache.block_table(entries[i].rid, g)[blk]
+                    sm[i] = bt[i, blk] * page
+            tables.append(bt)
+            slots.append(sm)
+        return StepLayout(
+            n_tokens=n, n_seqs=n, n_decode=n, row_of_entry=prev.row_of_entry, tokens=tokens, positions=positions,
+            token_seq=prev.token_seq, qo_indptr=prev.qo_indptr, kv_lens=positions + 1, slot_ids=prev.slot_ids,
+            logit_rows=prev.logit_rows, block_tables=tables, slot_mappings=slots, page_size=page, max_q_len=1,
+            max_kv_len=int(positions.max()) + 1,
+        )
+
     def plan(self, entries: Sequence[StepEntry]) -> StepLayout:
         """Reserve pages for the step's tokens (all or nothing) and lay the step out."""
+        # decode steps follow one another with the same requests: such a step is planned from the
+        # last one's plan.  Pages that a window releases change block tables behind the planner's
+        # back, so models with windows always take the general path.
+        if self._last_decode is not None:
+            last = self._last_decode
+            layout = self._plan_next_decode(entries) if not self._windowed else None
+            self._last_decode = None
+            if layout is not None:
+                self._last_decode = (last[0], last[1], layout, self.cache.epoch)
+                return layout
+        layout = self._plan_general(entries)
+        if layout.n_decode == layout.n_seqs:
+            self._last_decode = (
+                tuple(e.rid for e in entries), tuple(tuple(e.want) for e in entries), layout, self.cache.epoch
+            )
+        return layout
+
+    def _plan_general(self, entries: Sequence[StepEntry]) -> StepLayout:
         seen = set()
         for e in entries:
             if e.rid in seen:
@@ -153,16 +230,18 @@ class Engine:
             n = len(e.tokens)
             if n == 0:
                 raise ValueError(f"request {e.rid!r}: an entry needs at least one token")
-            for tok in e.tokens:
-                if not 0 <= int(tok) < self.vocab_size:
-                    raise ValueError(f"request {e.rid!r}: token id {tok} outside the vocabulary of {self.vocab_size}")
+            lo, hi = min(e.tokens), max(e.tokens)
+            if lo < 0 or hi >= self.vocab_size:
+                raise ValueError(
+                    f"request {e.rid!r}: token id {lo if lo < 0 else hi} outside the vocabulary of {self.vocab_size}"
+                )
             if self.cache.num_tokens(e.rid) + n > self.max_model_len:
                 raise ValueError(
                     f"request {e.rid!r}: {self.cache.num_tokens(e.rid)} + {n} tokens exceed max_model_len={self.max_model_len}"
                 )
         # all-or-nothing over the whole batch: count the pages the step takes from every pool
+        need = sum(self.cache.new_pages_needed(e.rid, len(e.tokens)) for e in entries)
         for gi, pool in enumerate(self.cache.pools):
-            need = sum(self.cache.new_pages_needed(e.rid, len(e.tokens)) for e in entries)
             if need > pool.free_count:
                 raise OutOfPages(
                     f"step needs {need} new pages in group {self.cache.groups[gi].name}, {pool.free_count} are free"

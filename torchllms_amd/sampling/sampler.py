@@ -23,6 +23,11 @@ class Sampler:
         # requests step after step, and only the counters change
         self._key = None
         self._fixed = None
+        # the counters travel through a pinned buffer with an asynchronous copy, so that the sampling
+        # kernel is queued behind the step's kernels without the host waiting in between; the buffer
+        # is free again once the previous call's result has been read (its .tolist() waits)
+        self._pinned = None
+        self._counters = None
 
     def __call__(self, logits: torch.Tensor, params: Sequence[SamplingParams], steps: Sequence[int]) -> List[int]:
         n = logits.shape[0]
@@ -40,7 +45,12 @@ class Sampler:
                 top_k = torch.tensor([p.top_k or 0 for p in params], dtype=torch.int32, device=dev)
             self._key, self._fixed = key, (temperature, seeds, top_k)
         temperature, seeds, top_k = self._fixed
-        counters = torch.tensor([int(s) for s in steps], dtype=torch.int64, device=dev)
+        if self._pinned is None or self._pinned.numel() < n or self._counters.device != dev:
+            self._pinned = torch.empty((max(n, 64),), dtype=torch.int64, pin_memory=True)
+            self._counters = torch.empty((max(n, 64),), dtype=torch.int64, device=dev)
+        self._pinned[:n] = torch.as_tensor([int(s) for s in steps], dtype=torch.int64)
+        counters = self._counters[:n]
+        counters.copy_(self._pinned[:n], non_blocking=True)
         return ops.sample(logits, temperature, seeds, counters, top_k).tolist()
 
 
