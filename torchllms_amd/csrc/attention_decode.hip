@@ -200,7 +200,7 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int key = base + 4 * g4 + i;
-      const bool valid = key >= lo && key <= p;
+      const bool valid = (key >= lo) & (key <= p);  // bit operation: no branch behind the MFMAs
       s[i] = valid ? c[i] * a.scale_log2e : -INFINITY;
       tmax = fmaxf(tmax, s[i]);
     }

@@ -232,52 +232,53 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
     for (int chunk = 0; chunk < KT / (16 * NS); ++chunk) {
     const int cbase = base + 16 * NS * chunk;
     if (cbase > wave_hi || cbase + 16 * NS - 1 < wave_lo) continue;
-    // phase 1: scores S^T[key][column], one MFMA chain per (16 keys, column block)
+    // phase 1: scores S^T[key][column], one MFMA chain per (16 keys, column block).  No branch from
+    // here to the end of the chunk but one, so that the compiler can interleave the chains and the
+    // two column blocks' softmax arithmetic; a block of 16 keys that the wave does not see at all is
+    // computed and masked like any other.
     float4_t c[NC][NS];
-    bool live[NS];
 #pragma unroll
-    for (int sub = 0; sub < NS; ++sub) {
-      const int kb = cbase + 16 * sub;
-      live[sub] = !(kb > wave_hi || kb + 15 < wave_lo);
+    for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
       for (int i = 0; i < NC; ++i) c[i][sub] = float4_t{0.f, 0.f, 0.f, 0.f};
-      if (!live[sub]) continue;
-      Pack16 ka[KL];
 #pragma unroll
-      for (int u = 0; u < KL; ++u)
-        ka[u].u = *reinterpret_cast<const u32x4_t*>(&k_lds[(16 * (NS * chunk + sub) + n16) * kKPitch + 32 * u + 8 * g4]);
+    for (int u = 0; u < KL; ++u) {
+      Pack16 ka[NS];
 #pragma unroll
-      for (int u = 0; u < KL; ++u)
+      for (int sub = 0; sub < NS; ++sub)
+        ka[sub].u = *reinterpret_cast<const u32x4_t*>(&k_lds[(16 * (NS * chunk + sub) + n16) * kKPitch + 32 * u + 8 * g4]);
+#pragma unroll
+      for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
         for (int i = 0; i < NC; ++i)
-          c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[u].op(), qreg[i][u].op(), c[i][sub], 0, 0, 0);
+          c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[sub].op(), qreg[i][u].op(), c[i][sub], 0, 0, 0);
     }
     // softmax bookkeeping once per chunk and column: mask, maximum, rescale, probabilities.
     // Scores stay unscaled; the scale enters through one fused multiply-add per element:
     // exp2(s * scale - m), with m the running maximum of s * scale.
     bf16x8_t pb[NC];  // slot e < 4: key 4 g4 + e of the first 16 keys; e >= 4: the same of the second 16
+    float alpha[NC];
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
-      // keys of the chunk that every lane of this column sees need no test at all
-      const bool all_seen = live[0] && live[NS - 1] && cbase >= col_lo[i] && cbase + 16 * NS - 1 <= col_pos[i];
       float tmax = -INFINITY;
 #pragma unroll
       for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          if (!all_seen) {
-            const int key = cbase + 16 * sub + 4 * g4 + r;
-            const bool valid = live[sub] && key >= col_lo[i] && key <= col_pos[i];
-            if (!valid) c[i][sub][r] = -INFINITY;
-          }
-          tmax = fmaxf(tmax, c[i][sub][r]);
+          // plain bit operations, no short-circuit: a branch here, right behind the MFMAs, is what
+          // this compiler has been seen to get wrong (the masked value overwrote live scores)
+          const int key = cbase + 16 * sub + 4 * g4 + r;
+          const bool valid = (key >= col_lo[i]) & (key <= col_pos[i]);
+          const float sc = valid ? c[i][sub][r] : -INFINITY;
+          c[i][sub][r] = sc;
+          tmax = fmaxf(tmax, sc);
         }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
       const float m_new = fmaxf(m_run[i], tmax * a.scale_log2e);  // the scale is positive
       // a column may not have met a visible key yet: then nothing is rescaled and nothing added
       const bool none = m_new == -INFINITY;
-      const float alpha = none ? 1.f : __builtin_amdgcn_exp2f(m_run[i] - m_new);
+      alpha[i] = none ? 1.f : __builtin_amdgcn_exp2f(m_run[i] - m_new);
       const float neg_m = none ? 0.f : -m_new;
       float psum = 0.f;
       uint32_t pw[2 * NS];
@@ -293,15 +294,20 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
         pw[2 * sub + 1] = pack_bf16x2(pr[2], pr[3]);
       }
       pb[i] = __builtin_bit_cast(bf16x8_t, u32x4_t{pw[0], pw[1], pw[2], pw[3]});
-      l_part[i] = l_part[i] * alpha + psum;
+      l_part[i] = l_part[i] * alpha[i] + psum;
       m_run[i] = m_new;
-      // the sums so far are rescaled only when some column's maximum has moved
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+    }
+    // the sums so far are rescaled only when some column's maximum has moved
+    bool moved = false;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) moved = moved || alpha[i] != 1.f;
+    if (__builtin_amdgcn_ballot_w64(moved)) {
+#pragma unroll
+      for (int i = 0; i < NC; ++i)
 #pragma unroll
         for (int t = 0; t < DT; ++t)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha;
-      }
+          for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha[i];
     }
     // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column] over the chunk's 32 keys.
     // A block of 16 keys that no column of the wave sees has zero probabilities: its rows are read
