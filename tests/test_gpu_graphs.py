@@ -58,7 +58,7 @@ def test_graph_replays_match_eager_steps(tmp_path, name, dtype):
         a, b = both([take(r, 1) for r in rows])
         check(a, b, f"decode step {step} with {len(rows)} rows")
         held.append((a, b))
-    assert sum(g.replays for g in graphed.graphs.graphs.values()) >= 30
+    assert sum(g.replays for g in graphed.graphs.graphs.values()) >= 25  # a shape runs eagerly until it has come back
     assert len(graphed.graphs.graphs) >= 3  # batch sizes 2, 3, 4
     # results handed out earlier were not overwritten by later replays
     for a, b in held:

@@ -38,10 +38,11 @@ class DecodeGraph:
     owns it: a reference cycle would leave the graph to the cyclic garbage collector, which may
     run, and destroy the graph, in the middle of somebody else's stream capture."""
 
-    def __init__(self, model, cache, device, page_size: int, layout: StepLayout, cap: int):
+    def __init__(self, model, cache, device, page_size: int, layout: StepLayout, cap: int, pool=None):
         self.model = model
         self.cache = cache
         self.cap = cap
+        self.pool = pool
         width = -(-cap // page_size)
         n_groups = len(layout.block_tables)
         self.shapes = section_shapes(layout.n_tokens, layout.n_seqs, layout.logit_rows.size, [width] * n_groups)
@@ -72,13 +73,12 @@ class DecodeGraph:
         # what the eager run derived from the step's plan (tables of cosines, ...) belongs to that
         # run: the recording has to contain the kernels that derive it anew from the fixed buffers
         ctx.scratch.clear()
-        # nothing may be destroyed while the stream is capturing: collect garbage now and keep the
-        # collector off until the capture has ended
-        gc.collect()
+        # nothing may be destroyed while the stream is capturing (a graph of an engine that is
+        # garbage, say): the collector stays off until the capture has ended
         gc_was_on = gc.isenabled()
         gc.disable()
         try:
-            with torch.cuda.graph(graph):
+            with torch.cuda.graph(graph, pool=self.pool):
                 self.logits = self.model.forward(ctx, self.cache)
         finally:
             if gc_was_on:
@@ -95,24 +95,40 @@ class DecodeGraph:
 
 
 class DecodeGraphs:
-    """The engine's recorded decode steps, by (requests, wanted rows, context cap)."""
+    """The engine's recorded decode steps, by (requests, wanted rows, context cap).
 
-    def __init__(self, model, cache, device, page_size: int, max_graphs: int = 32):
+    Recording costs many times a step, so a shape is recorded only when it comes back: the first
+    ``record_after`` steps of a shape run eagerly (while requests join one by one every step has a
+    new shape that never returns).  All recordings share one memory pool: they are replayed one at
+    a time and a step's logits are copied out before the next replay."""
+
+    def __init__(self, model, cache, device, page_size: int, max_graphs: int = 128, record_after: int = 2):
         self.model = model
         self.cache = cache
         self.device = device
         self.page_size = page_size
         self.max_graphs = max_graphs
+        self.record_after = record_after
         self.graphs: Dict[Tuple[int, int, int], DecodeGraph] = {}
+        self.seen: Dict[Tuple[int, int, int], int] = {}
+        self.pool = None
 
     def run(self, layout: StepLayout) -> torch.Tensor:
         cap = context_cap(layout.max_kv_len)
         key = (layout.n_seqs, int(layout.logit_rows.size), cap)
         g = self.graphs.get(key)
-        if g is None:
-            if len(self.graphs) >= self.max_graphs:
-                self.graphs.pop(next(iter(self.graphs)))
-            g = DecodeGraph(self.model, self.cache, self.device, self.page_size, layout, cap)
-            self.graphs[key] = g
-            return g.first_run(layout)
-        return g.replay(layout)
+        if g is not None:
+            return g.replay(layout)
+        count = self.seen.get(key, 0) + 1
+        self.seen[key] = count
+        if count <= self.record_after:
+            from .context import upload
+
+            return self.model.forward(upload(layout, self.device), self.cache)
+        if len(self.graphs) >= self.max_graphs:
+            self.graphs.pop(next(iter(self.graphs)))
+        if self.pool is None:
+            self.pool = torch.cuda.graph_pool_handle()
+        g = DecodeGraph(self.model, self.cache, self.device, self.page_size, layout, cap, self.pool)
+        self.graphs[key] = g
+        return g.first_run(layout)

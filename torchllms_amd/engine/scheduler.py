@@ -33,7 +33,7 @@ from .layout import StepEntry
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
 
 
-@dataclass
+@dataclass(eq=False)  # a request is itself, not its field values: membership tests stay cheap
 class Request:
     rid: Hashable
     prompt: List[int]
@@ -60,7 +60,7 @@ class Request:
         return self.state == FINISHED
 
 
-@dataclass
+@dataclass(eq=False)
 class ScheduledEntry:
     request: Request
     tokens: List[int]
