@@ -22,7 +22,7 @@ import time
 HBM_GBS = 8000.0  # MI355X HBM3E, published
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # dense MFMA, published
 
-# BASELINE.json configs[2]: Llama-3.1-8B shape
+# the model of the headline benchmark: Llama-3.1-8B layer sizes, random weights
 LLAMA_8B = dict(
     architectures=["LlamaForCausalLM"], hidden_size=4096, num_hidden_layers=32, num_attention_heads=32,
     num_key_value_heads=8, head_dim=128, intermediate_size=14336, vocab_size=128256, rms_norm_eps=1e-5,
