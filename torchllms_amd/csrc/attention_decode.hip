@@ -154,10 +154,25 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
   for (int e = 0; e < kE; ++e) acc[e] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   auto clamp_key = [&](int key) { return key < lo ? lo : (key > p ? p : key); };
-  auto row_ptr = [&](const bf16_t* pages, int key) {
-    const int blk = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
-    const int off = a.page_shift >= 0 ? key & (a.page_size - 1) : key % a.page_size;
-    return pages + ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH;
+  auto block_of = [&](int key) { return a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size; };
+  auto offset_of = [&](int key) { return a.page_shift >= 0 ? key & (a.page_size - 1) : key % a.page_size; };
+  auto row_ptr = [&](const bf16_t* pages, int page, int key) {
+    return pages + ((size_t)page * a.n_kv_heads + kvh) * head_elems + (size_t)offset_of(key) * DH;
+  };
+
+  // The page ids of a tile's rows: one for the lane's key row, four for its value rows.  They are
+  // fetched from the block table a tile before the rows themselves, so that a row's load waits for
+  // one trip to memory, not for two in a row (at small batches a tile is worked off faster than that).
+  struct TilePages {
+    int32_t k;
+    int32_t v[4];
+  };
+  auto fetch_pages = [&](int base) {
+    TilePages tp;
+    tp.k = bt[block_of(clamp_key(base + n16))];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) tp.v[j] = bt[block_of(clamp_key(base + 4 * g4 + j))];
+    return tp;
   };
 
   // Rolling prefetch: the keys of tile t+1 are requested as soon as the MFMAs of tile t have read
@@ -168,21 +183,23 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
   // that nobody uses.
   Pack16 kreg[kKLoads];
   uint32_t vreg[4][kVDwords];
-  auto load_k = [&](int base) {
-    const bf16_t* kr = row_ptr(a.k_pages, clamp_key(base + n16));
+  auto load_k = [&](int base, const TilePages& tp) {
+    const bf16_t* kr = row_ptr(a.k_pages, tp.k, clamp_key(base + n16));
 #pragma unroll
     for (int u = 0; u < kKLoads; ++u) kreg[u].u = *reinterpret_cast<const u32x4_t*>(kr + 32 * u + 8 * g4);
   };
-  auto load_v = [&](int base) {
+  auto load_v = [&](int base, const TilePages& tp) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      load_value_words(row_ptr(a.v_pages, clamp_key(base + 4 * g4 + j)) + kE * n16, vreg[j]);
+      load_value_words(row_ptr(a.v_pages, tp.v[j], clamp_key(base + 4 * g4 + j)) + kE * n16, vreg[j]);
   };
 
   int base = split_begin + wave * kTile;
+  TilePages pages_next = fetch_pages(base + kWaves * kTile);
   if (base <= split_end) {
-    load_k(base);
-    load_v(base);
+    const TilePages pages_now = fetch_pages(base);
+    load_k(base, pages_now);
+    load_v(base, pages_now);
   }
   for (; base <= split_end; base += kWaves * kTile) {
     const int next = base + kWaves * kTile;
@@ -194,7 +211,7 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
       c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].half(0), qreg[u].half(0), c, 0, 0, 0);
       c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].half(1), qreg[u].half(1), c, 0, 0, 0);
     }
-    load_k(next);  // unconditional: past the split's end the keys are clamped and unused
+    load_k(next, pages_next);  // unconditional: past the split's end the keys are clamped and unused
     float s[4];
     float tmax = -INFINITY;
 #pragma unroll
@@ -227,7 +244,8 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
       acc[e] = acc[e] * alpha;
       acc[e] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop, pop, acc[e], 0, 0, 0);
     }
-    load_v(next);
+    load_v(next, pages_next);
+    pages_next = fetch_pages(next + kWaves * kTile);  // for the tile after the next
   }
 
   // the lane's own sums join over the four row groups
