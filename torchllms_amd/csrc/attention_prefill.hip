@@ -297,18 +297,14 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
       l_part[i] = l_part[i] * alpha[i] + psum;
       m_run[i] = m_new;
     }
-    // the sums so far are rescaled only when some column's maximum has moved
-    bool moved = false;
+    // the sums so far follow the maxima (no test whether any moved: a branch here keeps the compiler
+    // from overlapping this arithmetic with the MFMAs around it, which costs more than it saves)
 #pragma unroll
-    for (int i = 0; i < NC; ++i) moved = moved || alpha[i] != 1.f;
-    if (__builtin_amdgcn_ballot_w64(moved)) {
+    for (int i = 0; i < NC; ++i)
 #pragma unroll
-      for (int i = 0; i < NC; ++i)
+      for (int t = 0; t < DT; ++t)
 #pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha[i];
-    }
+        for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha[i];
     // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column] over the chunk's 32 keys.
     // A block of 16 keys that no column of the wave sees has zero probabilities: its rows are read
     // all the same (they lie in the tile) and add nothing.
