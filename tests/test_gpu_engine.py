@@ -258,3 +258,24 @@ def test_decode_steps_planned_from_the_last_plan_equal_the_general_plan(cases):
     assert used_fast >= 15  # the shortcut did plan most of these steps
     for eng in engines:
         eng.cache.check_invariants()
+
+
+def test_pool_sizes(cases):
+    """The pool is as large as asked: pages, gigabytes, a fraction of free memory, or room for
+    ``max_seqs`` requests of ``max_model_len`` tokens."""
+    from torchllms_amd.cache import CacheManager
+    from torchllms_amd.engine import Engine
+
+    folder = cases["A"].folder
+    per_page = None
+    for kw, check in [
+        (dict(num_pages=7), lambda n, pp: n == 7),
+        (dict(kv_memory_gb=1 / 1024), lambda n, pp: n == (1 << 20) // pp),
+        (dict(kv_memory_fraction=1e-4), lambda n, pp: 1 <= n <= torch.cuda.mem_get_info()[1] * 1e-4 // pp),
+        (dict(max_seqs=3, max_model_len=50), lambda n, pp: n == 3 * 7),
+    ]:
+        eng = Engine.from_folder(folder, dtype="float32", page_size=8, **kw)
+        per_page = CacheManager.bytes_per_page(eng.cache.groups, 8, torch.float32)
+        assert check(eng.cache.pools[0].num_pages, per_page), kw
+    with pytest.raises(ValueError, match="kv_memory_fraction"):
+        Engine.from_folder(folder, dtype="float32", kv_memory_fraction=1.5)

@@ -58,6 +58,7 @@ class Engine:
         page_size: int = 16,
         num_pages: Optional[int] = None,
         kv_memory_gb: Optional[float] = None,
+        kv_memory_fraction: Optional[float] = None,
         max_seqs: int = 8,
         max_model_len: Optional[int] = None,
         device="cuda:0",
@@ -65,8 +66,9 @@ class Engine:
         tune_kernels: bool = True,
     ):
         """``tensors``: the model's tensors under the parts' own names, on ``device``.
-        Pool size: ``num_pages`` pages per group, else what ``kv_memory_gb`` holds, else room for
-        ``max_seqs`` requests of ``max_model_len`` tokens (reference: networks.py:872-884)."""
+        Pool size: ``num_pages`` pages per group, else what ``kv_memory_gb`` holds, else
+        ``kv_memory_fraction`` of the device memory that is free once the weights are loaded, else
+        room for ``max_seqs`` requests of ``max_model_len`` tokens (reference: networks.py:872-884)."""
         self.device = require_gpu(device)
         self.arch = arch
         self.config = config
@@ -82,6 +84,11 @@ class Engine:
             per_page = CacheManager.bytes_per_page(groups, page_size, dtype)
             if kv_memory_gb is not None and per_page > 0:
                 num_pages = max(int(kv_memory_gb * (1 << 30)) // per_page, 1)
+            elif kv_memory_fraction is not None and per_page > 0:
+                if not 0.0 < kv_memory_fraction <= 1.0:
+                    raise ValueError(f"kv_memory_fraction must lie in (0, 1], got {kv_memory_fraction}")
+                free_bytes, _ = torch.cuda.mem_get_info(self.device)
+                num_pages = max(int(free_bytes * kv_memory_fraction) // per_page, 1)
             else:
                 num_pages = max_seqs * (-(-self.max_model_len // page_size))
         self.cache = CacheManager(groups, states, page_size, num_pages, max_seqs, dtype=dtype, device=self.device)

@@ -78,6 +78,7 @@ class LLM:
         page_size: int = 16,
         kv_memory_gb: Optional[float] = None,
         num_pages: Optional[int] = None,
+        kv_memory_fraction: Optional[float] = None,
         max_num_batched_tokens: int = 2048,
         tokenizer=None,
         seed: int = 0,
@@ -109,7 +110,7 @@ class LLM:
             raise ValueError(f"unknown model_kwargs {sorted(model_kwargs)}")
         self.engine = Engine.from_folder(
             folder, dtype=precision, device=device, page_size=page_size, num_pages=num_pages,
-            kv_memory_gb=kv_memory_gb, max_seqs=max_bsz, max_model_len=max_len,
+            kv_memory_gb=kv_memory_gb, kv_memory_fraction=kv_memory_fraction, max_seqs=max_bsz, max_model_len=max_len,
         )
         self.max_len = self.engine.max_model_len
         self.max_bsz = max_bsz
