@@ -160,6 +160,15 @@ def test_rope_table_and_its_use_give_what_the_kernel_computes_itself():
         a, b = qkv.to(DEV), qkv.to(DEV)
         _ops().rope_kv_write(a, hq, hkv, dh, _i32(pos.tolist()), inv_freq.to(DEV), rot, 0)
         _ops().rope_kv_write(b, hq, hkv, dh, _i32(pos.tolist()), None, rot, 0, cos_sin=table)
+        # the table takes the wide-access kernel: the same cosines and sines, products possibly
+        # fused differently, so equal but for the last bit
+        tol = dict(rtol=2e-7, atol=1e-6) if dtype == torch.float32 else dict(rtol=2 ** -8, atol=1e-6)
+        torch.testing.assert_close(a.float(), b.float(), **tol)
+        assert (a != b).float().mean().item() < 0.02
+        # half-split pairing keeps the narrow kernel, table or not: bit-equal
+        a, b = qkv.to(DEV), qkv.to(DEV)
+        _ops().rope_kv_write(a, hq, hkv, dh, _i32(pos.tolist()), inv_freq.to(DEV), rot, 1)
+        _ops().rope_kv_write(b, hq, hkv, dh, _i32(pos.tolist()), None, rot, 1, cos_sin=table)
         assert torch.equal(a, b)
 
 
@@ -200,6 +209,39 @@ def test_gemm_stream_qkv_equals_product_then_rotary_kernel(m, hq, hkv, dh, rot, 
         torch.testing.assert_close(kb.float(), ka.float(), **tol)
         torch.testing.assert_close(vb.float(), va.float(), **tol)
         assert (kb.float().abs().sum(dim=(1, 3)) > 0).sum().item() == m - (1 if m > 2 else 0)  # one slot per stored row
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq, hkv, dh, rot, page", [(32, 8, 128, 128, 16), (6, 3, 48, 20, 4), (5, 5, 16, 16, 16), (3, 1, 24, 0, 8)])
+def test_rope_wide_kernel_with_table_and_pages(dtype, hq, hkv, dh, rot, page):
+    """The kernel the engine's prefill takes (table of cosines, 16-byte accesses): queries in place,
+    rotated keys and raw values in their pages, partial rotary cut inside a 16-byte piece, a
+    token without a slot stores nothing."""
+    torch.manual_seed(0)
+    n = 37
+    qkv = torch.randn(n, (hq + 2 * hkv) * dh).to(dtype)
+    pos = torch.randint(0, 9000, (n,))
+    inv_freq = plain.rope_inverse_frequencies(rot, 500000.0, None) if rot else None
+    table = _ops().rope_table(_i32(pos.tolist()), inv_freq.to(DEV)) if rot else None
+    n_pages = 12
+    slots = torch.randperm(n_pages * page)[:n].tolist()
+    slots[5] = -1
+    k_pages, v_pages = _pages(n_pages, hkv, page, dh, dtype)
+    dev = qkv.to(DEV)
+    _ops().rope_kv_write(dev, hq, hkv, dh, _i32(pos.tolist()), None, rot, 0, k_pages, v_pages, _i32(slots), page, cos_sin=table)
+    heads = qkv.view(n, hq + 2 * hkv, dh)
+    want = heads.clone().float()
+    if rot:
+        want[:, : hq + hkv, :rot] = plain.rope_rotate_interleaved(heads[:, : hq + hkv, :rot], pos, inv_freq)
+    tol = dict(rtol=1e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=1e-3)
+    torch.testing.assert_close(dev.cpu().view(n, hq + 2 * hkv, dh)[:, :hq].float(), want[:, :hq], **tol)
+    for i, s in enumerate(slots):
+        if s < 0:
+            continue
+        torch.testing.assert_close(k_pages[s // page, :, s % page].cpu().float(), want[i, hq : hq + hkv], **tol)
+        assert torch.equal(v_pages[s // page, :, s % page].cpu(), heads[i, hq + hkv :])
+    stored = (k_pages.float().abs().sum(dim=(1, 3)) > 0).sum().item()
+    assert stored == n - 1
 
 
 def test_cache_write_round_trip_with_distinct_values():

@@ -314,6 +314,68 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int n_q_heads, int n_k
   }
 }
 
+// The same work with 16-byte accesses, for the common case: interleaved pairs, the step's table of
+// cosines and sines, head and rotary sizes that are multiples of the V elements a thread takes.
+// One thread = V consecutive channels of one head of one token.
+template <typename T, int V>
+__global__ void rope_kv_write_vec_kernel(T* __restrict__ qkv, int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
+                                         const float2* __restrict__ cos_sin, int rotary_dim,
+                                         T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                         const int32_t* __restrict__ slot_mapping, int page_size) {
+  struct alignas(sizeof(T) * V) Vec { T e[V]; };
+  const int chunks_per_head = head_dim / V;
+  const int heads = n_q_heads + (k_pages ? 2 : 1) * n_kv_heads;  // values only move when there are pages
+  const int per_token = heads * chunks_per_head;
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long long)n_tokens * per_token) return;
+  const int t = (int)(idx / per_token);
+  const int c = (int)(idx % per_token);
+  const int head = c / chunks_per_head;
+  const int d0 = (c % chunks_per_head) * V;
+  const int row = (n_q_heads + 2 * n_kv_heads) * head_dim;
+  T* src = qkv + (size_t)t * row + (size_t)head * head_dim + d0;
+  Vec v = *reinterpret_cast<const Vec*>(src);
+  const bool rotates = head < n_q_heads + n_kv_heads;
+  if (rotates && d0 < rotary_dim) {
+    const float2* cs = cos_sin + (size_t)t * (rotary_dim / 2) + d0 / 2;
+#pragma unroll
+    for (int j = 0; j < V / 2; ++j) {
+      if (d0 + 2 * j < rotary_dim) {
+        const float2 f = cs[j];
+        const float a0 = to_f32(v.e[2 * j]), a1 = to_f32(v.e[2 * j + 1]);
+        v.e[2 * j] = from_f32<T>(a0 * f.x - a1 * f.y);
+        v.e[2 * j + 1] = from_f32<T>(a1 * f.x + a0 * f.y);
+      }
+    }
+  }
+  if (head < n_q_heads || k_pages == nullptr) {
+    if (rotates) *reinterpret_cast<Vec*>(src) = v;
+    return;
+  }
+  const int slot = slot_mapping[t];
+  if (slot < 0) return;
+  const int page = slot / page_size, off = slot % page_size;
+  const bool is_key = head < n_q_heads + n_kv_heads;
+  const int kh = is_key ? head - n_q_heads : head - n_q_heads - n_kv_heads;
+  T* dst = (is_key ? k_pages : v_pages) + (((size_t)page * n_kv_heads + kh) * page_size + off) * head_dim + d0;
+  *reinterpret_cast<Vec*>(dst) = v;
+}
+
+template <typename T>
+bool rope_vec_launch(T* qkv, int n_tokens, int n_q_heads, int n_kv_heads, int head_dim, const float2* cos_sin,
+                     int rotary_dim, int pairing, T* k_pages, T* v_pages, const int32_t* slot_mapping, int page_size,
+                     hipStream_t stream) {
+  constexpr int V = 16 / sizeof(T);
+  if (pairing != 0 || (rotary_dim > 0 && cos_sin == nullptr) || head_dim % V || rotary_dim % 2) return false;
+  if (((uintptr_t)qkv % 16) || (k_pages && (((uintptr_t)k_pages % 16) || ((uintptr_t)v_pages % 16)))) return false;
+  const long long threads_needed = (long long)n_tokens * (n_q_heads + (k_pages ? 2 : 1) * n_kv_heads) * (head_dim / V);
+  const long long blocks = (threads_needed + 255) / 256;
+  if (blocks > 0x7fffffffLL) return false;
+  rope_kv_write_vec_kernel<T, V><<<(unsigned)blocks, 256, 0, stream>>>(
+      qkv, n_tokens, n_q_heads, n_kv_heads, head_dim, cos_sin, rotary_dim, k_pages, v_pages, slot_mapping, page_size);
+  return true;
+}
+
 TL_EXPORT int tl_rope_kv_write(void* qkv, int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
                                const int32_t* positions, const float* inv_freq, const float* cos_sin,
                                int rotary_dim, int pairing, void* k_pages, void* v_pages,
@@ -327,6 +389,13 @@ TL_EXPORT int tl_rope_kv_write(void* qkv, int n_tokens, int n_q_heads, int n_kv_
   TL_REQUIRE(k_pages == nullptr || (slot_mapping != nullptr && page_size > 0),
              "rope: pages given without slot_mapping/page_size");
   if (n_tokens == 0) return TL_OK;
+  if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "rope: unknown dtype %d", dtype);
+  if (dtype == TL_F32
+          ? rope_vec_launch((float*)qkv, n_tokens, n_q_heads, n_kv_heads, head_dim, (const float2*)cos_sin, rotary_dim,
+                            pairing, (float*)k_pages, (float*)v_pages, slot_mapping, page_size, stream)
+          : rope_vec_launch((bf16_t*)qkv, n_tokens, n_q_heads, n_kv_heads, head_dim, (const float2*)cos_sin, rotary_dim,
+                            pairing, (bf16_t*)k_pages, (bf16_t*)v_pages, slot_mapping, page_size, stream))
+    return tl_check_launch("rope_kv_write");
   const int threads = 256;
   // heads per block column: all of them when the tokens alone fill the GPU, one pass otherwise
   const int head_groups = threads / (head_dim / 2) > 0 ? threads / (head_dim / 2) : 1;
