@@ -77,6 +77,42 @@ __device__ __forceinline__ Best block_best(Best v, Best* scratch) {
   return total;
 }
 
+// The thread's share of argmax(x): 16-byte loads, four of them in flight, where the row allows it.
+// `better` keeps the lowest index among equal maxima whatever the order of the visits.
+__device__ __forceinline__ Best row_best(const float* __restrict__ x, int vocab, int tid) {
+  constexpr int kNone = 0x7fffffff;
+  Best b = {-INFINITY, kNone};
+  int done = 0;
+  if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const int n4 = vocab / 4;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    int i = tid;
+    for (; i + 3 * kThreads < n4; i += 4 * kThreads) {
+      float4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = x4[i + u * kThreads];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int at = 4 * (i + u * kThreads);
+        b = better(b, Best{v[u].x, at});
+        b = better(b, Best{v[u].y, at + 1});
+        b = better(b, Best{v[u].z, at + 2});
+        b = better(b, Best{v[u].w, at + 3});
+      }
+    }
+    for (; i < n4; i += kThreads) {
+      const float4 v = x4[i];
+      b = better(b, Best{v.x, 4 * i});
+      b = better(b, Best{v.y, 4 * i + 1});
+      b = better(b, Best{v.z, 4 * i + 2});
+      b = better(b, Best{v.w, 4 * i + 3});
+    }
+    done = 4 * n4;
+  }
+  for (int i = done + tid; i < vocab; i += kThreads) b = better(b, Best{x[i], i});
+  return b;
+}
+
 __global__ void __launch_bounds__(kThreads)
 sample_kernel(const float* __restrict__ logits, int row_stride, int vocab,
               const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
@@ -92,38 +128,7 @@ sample_kernel(const float* __restrict__ logits, int row_stride, int vocab,
   constexpr int kNone = 0x7fffffff;
 
   if (temp == 0.f) {
-    Best b = {-INFINITY, kNone};
-    // 16-byte loads, four of them in flight per thread, where the row allows it; `better` keeps the
-    // lowest index among equal maxima whatever the order of the visits
-    int done = 0;
-    if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
-      const int n4 = vocab / 4;
-      const float4* x4 = reinterpret_cast<const float4*>(x);
-      int i = tid;
-      for (; i + 3 * kThreads < n4; i += 4 * kThreads) {
-        float4 v[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) v[u] = x4[i + u * kThreads];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int at = 4 * (i + u * kThreads);
-          b = better(b, Best{v[u].x, at});
-          b = better(b, Best{v[u].y, at + 1});
-          b = better(b, Best{v[u].z, at + 2});
-          b = better(b, Best{v[u].w, at + 3});
-        }
-      }
-      for (; i < n4; i += kThreads) {
-        const float4 v = x4[i];
-        b = better(b, Best{v.x, 4 * i});
-        b = better(b, Best{v.y, 4 * i + 1});
-        b = better(b, Best{v.z, 4 * i + 2});
-        b = better(b, Best{v.w, 4 * i + 3});
-      }
-      done = 4 * n4;
-    }
-    for (int i = done + tid; i < vocab; i += kThreads) b = better(b, Best{x[i], i});
-    b = block_best(b, best_scratch);
+    const Best b = block_best(row_best(x, vocab, tid), best_scratch);
     if (tid == 0) out[row] = b.idx;
     return;
   }
@@ -164,23 +169,32 @@ sample_kernel(const float* __restrict__ logits, int row_stride, int vocab,
     pivot = __uint_as_float(u);
   }
 
-  Best mx = {-INFINITY, kNone};
-  for (int i = tid; i < vocab; i += kThreads) mx = better(mx, Best{x[i] / tdiv, i});
-  mx = block_best(mx, best_scratch);
-  const float m = mx.val;
+  // the largest scaled logit: dividing by a positive number keeps the order, so the maximum of the
+  // raw row is found with wide loads and scaled once
+  const float m = block_best(row_best(x, vocab, tid), best_scratch).val / tdiv;
 
   const uint64_t seed = seeds[row];
   const uint64_t step = steps[row];
   Best b = {-INFINITY, kNone};
-  // each thread handles whole groups of four indices, so one generator call serves four draws
+  // each thread handles whole groups of four indices, so one generator call serves four draws; an
+  // aligned row gives the four logits in one 16-byte load
+  const bool wide = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
   for (int i4 = tid * 4; i4 < vocab; i4 += kThreads * 4) {
     uint32_t r[4];
     philox4(seed, (uint32_t)i4 >> 2, step, r);
+    float xs[4];
+    if (wide && i4 + 3 < vocab) {
+      const float4 v = *reinterpret_cast<const float4*>(x + i4);
+      xs[0] = v.x; xs[1] = v.y; xs[2] = v.z; xs[3] = v.w;
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) xs[u] = i4 + u < vocab ? x[i4 + u] : -INFINITY;
+    }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int i = i4 + u;
       if (i >= vocab) break;
-      const float xi = x[i] / tdiv;
+      const float xi = xs[u] / tdiv;
       if (xi < pivot) continue;
       const float q = -logf(uniform_open(r[u]));
       b = better(b, Best{expf(xi - m) / q, i});
