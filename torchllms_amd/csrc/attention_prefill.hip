@@ -4,7 +4,12 @@
 //   * a block of 4 waves takes a tile of consecutive queries of one request and one kv head, with
 //     all query heads that share it: its 128 MFMA columns are (query, head) pairs, so a key or value
 //     is fetched once for the whole group.
-//   * keys and values stream through LDS in tiles of 64 keys, both as they lie in the page.
+//   * keys and values stream through LDS in tiles of 64 keys, both as they lie in the page, and get
+//     there without passing through registers: `global_load_lds_dwordx4` puts a wave's 64 x 16 bytes
+//     at consecutive LDS addresses.  Rows are therefore not padded; instead the 16-byte pieces of a
+//     row are stored in an order that depends on the row (piece ^ f(row)), so that the 16 lanes that
+//     read the same piece of 16 rows still meet 16 different banks.  Two buffers: the next tile lands
+//     while the current one is worked off, with one barrier a tile.
 //   * scores are computed transposed, S^T[key][column] = K Q^T, by MFMA 16x16x32 bf16 (a lane's 16
 //     bytes of a key row are one operand); their output layout, taken over two blocks of 16 keys, is
 //     exactly the B-operand layout of P^T in O^T[channel][column] = V^T P^T, so the probabilities
@@ -50,11 +55,19 @@ constexpr int kCols = kWaves * NC * 16;      // columns per block
 constexpr int KT = DH <= 128 ? 64 : 32;       // keys per LDS tile
 constexpr int KL = DH / 32;                  // 16-byte pieces of a key row per lane
 constexpr int DT = DH / 16;                  // channel tiles of the output
-constexpr int kKPitch = DH + 8;              // bf16 elements per key row in LDS
 constexpr int kVWords = DT / 2;              // 32-bit words a lane reads from one value row (DT channels)
-constexpr int kChunksPerRow = DH / 8;        // 16-byte chunks in a key/value row
-constexpr int kLoadsPerThread = KT * kChunksPerRow / kThreads;
-static_assert(KT * kChunksPerRow % kThreads == 0, "tile does not divide over the block");
+constexpr int kPieces = DH / 8;              // 16-byte pieces in a key/value row
+constexpr int kRowsPerLoad = kWave / kPieces;  // rows that one wave load (64 lanes x 16 bytes) covers
+constexpr int kLoadsPerWave = KT / kRowsPerLoad / kWaves;  // wave loads per tile and operand
+static_assert(kRowsPerLoad >= 1 && KT % (kRowsPerLoad * kWaves) == 0, "tile does not divide over the block");
+constexpr int kTileElems = KT * DH;          // one operand's tile in LDS, rows unpadded
+// The piece s of row r lies at slot s ^ swizzle(r).  Banks repeat every 256 bytes, that is every
+// kRowsPerSweep rows; rows that start on the same bank get different slots for the same piece.
+constexpr int kRowsPerSweep = DH >= 128 ? 1 : 128 / DH;
+constexpr int kSwizzle = kPieces < 16 ? kPieces : 16;
+__device__ __forceinline__ int swizzle(int row) { return (row / kRowsPerSweep) % kSwizzle; }
+// element offset of piece `piece` of row `row` within a tile
+__device__ __forceinline__ int tile_at(int row, int piece) { return row * DH + 8 * (piece ^ swizzle(row)); }
 
 struct PrefillArgs {
   const bf16_t* q;
@@ -115,8 +128,7 @@ __device__ __forceinline__ void lds_words(const bf16_t* src, uint32_t* dst) {
 
 template <int RP>
 __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a) {
-  __shared__ __attribute__((aligned(16))) bf16_t k_lds[KT * kKPitch];
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds[KT * kKPitch];
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[2][2][kTileElems];  // [buffer][keys | values]
   constexpr int QB = kCols / RP;  // queries per block
 
   const int tile = blockIdx.y;  // the host lists the tiles in the order that balances the launch
@@ -189,40 +201,36 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
     for (int t = 0; t < DT; ++t) acc[i][t] = float4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // global -> registers for one tile of keys and values; keys outside the visible range are
-  // clamped into it (their scores are masked), so no load touches a page the request does not hold
-  Pack16 kst[kLoadsPerThread], vst[kLoadsPerThread];
-  auto fetch = [&](int base) {
+  // global -> LDS for one tile of keys and values, asynchronously.  Wave load j of wave w covers rows
+  // (j * kWaves + w) * kRowsPerLoad ... of the tile: lane -> (row, slot), and fetches the piece that
+  // belongs in that slot.  Keys outside the visible range are clamped into it (their scores are
+  // masked), so no load touches a page the request does not hold.
+  auto dma = [&](int base, int buffer) {
 #pragma unroll
-    for (int j = 0; j < kLoadsPerThread; ++j) {
-      const int id = threadIdx.x + j * kThreads;
-      int key = base + id / kChunksPerRow;
+    for (int j = 0; j < kLoadsPerWave; ++j) {
+      const int first = (j * kWaves + wave) * kRowsPerLoad;
+      const int r = first + lane / kPieces;
+      const int piece = (lane % kPieces) ^ swizzle(r);
+      int key = base + r;
       key = key < key_lo ? key_lo : (key > key_hi ? key_hi : key);
       const int blk = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
       const int off = a.page_shift >= 0 ? key & (a.page_size - 1) : key % a.page_size;
-      const size_t at = ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH + 8 * (id % kChunksPerRow);
-      kst[j].u = *reinterpret_cast<const u32x4_t*>(a.k_pages + at);
-      vst[j].u = *reinterpret_cast<const u32x4_t*>(a.v_pages + at);
-    }
-  };
-  auto stash = [&]() {
-#pragma unroll
-    for (int j = 0; j < kLoadsPerThread; ++j) {
-      const int id = threadIdx.x + j * kThreads;
-      const int key = id / kChunksPerRow;
-      const int dc = id % kChunksPerRow;
-      *reinterpret_cast<u32x4_t*>(&k_lds[key * kKPitch + 8 * dc]) = kst[j].u;
-      *reinterpret_cast<u32x4_t*>(&v_lds[key * kKPitch + 8 * dc]) = vst[j].u;
+      const size_t at = ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH + 8 * piece;
+      __builtin_amdgcn_global_load_lds(a.k_pages + at, &tiles[buffer][0][first * DH], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(a.v_pages + at, &tiles[buffer][1][first * DH], 16, 0, 0);
     }
   };
 
-  fetch(tile_begin);
-  for (int base = tile_begin; base <= key_hi; base += KT) {
-    __syncthreads();  // the previous tile has been read by every wave
-    stash();
+  dma(tile_begin, 0);
+  int buffer = 0;
+  for (int base = tile_begin; base <= key_hi; base += KT, buffer ^= 1) {
+    // this wave's loads of the tile have landed; after the barrier everybody's have, and everybody
+    // has finished with the tile before, whose buffer the next tile's loads may now overwrite
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    fetch(base + KT);  // in flight while this tile is computed; unconditional (keys are clamped), so
-                       // that no wait has to cover a path without it
+    dma(base + KT, buffer ^ 1);  // unconditional (keys are clamped): no wait has to cover a path without it
+    const bf16_t* k_lds = tiles[buffer][0];
+    const bf16_t* v_lds = tiles[buffer][1];
 
     if (base > wave_hi || base + KT - 1 < wave_lo) continue;  // nothing here for this wave's columns
 
@@ -246,7 +254,7 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
       Pack16 ka[NS];
 #pragma unroll
       for (int sub = 0; sub < NS; ++sub)
-        ka[sub].u = *reinterpret_cast<const u32x4_t*>(&k_lds[(16 * (NS * chunk + sub) + n16) * kKPitch + 32 * u + 8 * g4]);
+        ka[sub].u = *reinterpret_cast<const u32x4_t*>(&k_lds[tile_at(16 * (NS * chunk + sub) + n16, g4 + 4 * u)]);
 #pragma unroll
       for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
@@ -313,7 +321,13 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int key = 16 * NS * chunk + 16 * (e / 4) + 4 * g4 + (e % 4);  // within the tile
-        lds_words<kVWords>(&v_lds[key * kKPitch + DT * n16], vrow[e]);
+        // the lane's DT channels start at channel DT * n16: part of one piece, or two whole pieces
+        if constexpr (kVWords <= 4) {
+          lds_words<kVWords>(&v_lds[tile_at(key, DT * n16 / 8) + DT * n16 % 8], vrow[e]);
+        } else {
+          lds_words<4>(&v_lds[tile_at(key, 2 * n16)], vrow[e]);
+          lds_words<4>(&v_lds[tile_at(key, 2 * n16 + 1)], vrow[e] + 4);
+        }
       }
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
