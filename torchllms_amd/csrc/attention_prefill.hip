@@ -234,16 +234,14 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
 
     if (base > wave_hi || base + KT - 1 < wave_lo) continue;  // nothing here for this wave's columns
 
-    // the tile is worked off in chunks of 32 keys: scores, softmax bookkeeping, then P.V
-    constexpr int NS = 2;
-#pragma unroll
-    for (int chunk = 0; chunk < KT / (16 * NS); ++chunk) {
-    const int cbase = base + 16 * NS * chunk;
-    if (cbase > wave_hi || cbase + 16 * NS - 1 < wave_lo) continue;
+    // the whole tile at once: scores, softmax bookkeeping (one running maximum and one rescaling of
+    // the sums per tile), then P.V in groups of 32 keys
+    constexpr int NS = KT / 16;  // blocks of 16 keys
+    {
     // phase 1: scores S^T[key][column], one MFMA chain per (16 keys, column block).  No branch from
-    // here to the end of the chunk but one, so that the compiler can interleave the chains and the
-    // two column blocks' softmax arithmetic; a block of 16 keys that the wave does not see at all is
-    // computed and masked like any other.
+    // here to the end of the tile, so that the compiler can interleave the chains and the column
+    // blocks' softmax arithmetic; a block of 16 keys that the wave does not see at all is computed
+    // and masked like any other.
     float4_t c[NC][NS];
 #pragma unroll
     for (int sub = 0; sub < NS; ++sub)
@@ -254,17 +252,17 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
       Pack16 ka[NS];
 #pragma unroll
       for (int sub = 0; sub < NS; ++sub)
-        ka[sub].u = *reinterpret_cast<const u32x4_t*>(&k_lds[tile_at(16 * (NS * chunk + sub) + n16, g4 + 4 * u)]);
+        ka[sub].u = *reinterpret_cast<const u32x4_t*>(&k_lds[tile_at(16 * sub + n16, g4 + 4 * u)]);
 #pragma unroll
       for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
         for (int i = 0; i < NC; ++i)
           c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[sub].op(), qreg[i][u].op(), c[i][sub], 0, 0, 0);
     }
-    // softmax bookkeeping once per chunk and column: mask, maximum, rescale, probabilities.
+    // softmax bookkeeping once per tile and column: mask, maximum, rescale, probabilities.
     // Scores stay unscaled; the scale enters through one fused multiply-add per element:
     // exp2(s * scale - m), with m the running maximum of s * scale.
-    bf16x8_t pb[NC];  // slot e < 4: key 4 g4 + e of the first 16 keys; e >= 4: the same of the second 16
+    bf16x8_t pb[NC][NS / 2];  // per 32 keys; slot e < 4: key 4 g4 + e of the first 16 keys; e >= 4: of the second 16
     float alpha[NC];
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
@@ -275,7 +273,7 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
         for (int r = 0; r < 4; ++r) {
           // plain bit operations, no short-circuit: a branch here, right behind the MFMAs, is what
           // this compiler has been seen to get wrong (the masked value overwrote live scores)
-          const int key = cbase + 16 * sub + 4 * g4 + r;
+          const int key = base + 16 * sub + 4 * g4 + r;
           const bool valid = (key >= col_lo[i]) & (key <= col_pos[i]);
           const float sc = valid ? c[i][sub][r] : -INFINITY;
           c[i][sub][r] = sc;
@@ -301,7 +299,9 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
         pw[2 * sub] = pack_bf16x2(pr[0], pr[1]);
         pw[2 * sub + 1] = pack_bf16x2(pr[2], pr[3]);
       }
-      pb[i] = __builtin_bit_cast(bf16x8_t, u32x4_t{pw[0], pw[1], pw[2], pw[3]});
+#pragma unroll
+      for (int g = 0; g < NS / 2; ++g)
+        pb[i][g] = __builtin_bit_cast(bf16x8_t, u32x4_t{pw[4 * g], pw[4 * g + 1], pw[4 * g + 2], pw[4 * g + 3]});
       l_part[i] = l_part[i] * alpha[i] + psum;
       m_run[i] = m_new;
     }
@@ -313,14 +313,15 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
       for (int t = 0; t < DT; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha[i];
-    // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column] over the chunk's 32 keys.
+    // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column], 32 keys at a time.
     // A block of 16 keys that no column of the wave sees has zero probabilities: its rows are read
     // all the same (they lie in the tile) and add nothing.
-    {
+#pragma unroll
+    for (int g = 0; g < NS / 2; ++g) {
       uint32_t vrow[8][kVWords];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const int key = 16 * NS * chunk + 16 * (e / 4) + 4 * g4 + (e % 4);  // within the tile
+        const int key = 32 * g + 16 * (e / 4) + 4 * g4 + (e % 4);  // within the tile
         // the lane's DT channels start at channel DT * n16: part of one piece, or two whole pieces
         if constexpr (kVWords <= 4) {
           lds_words<kVWords>(&v_lds[tile_at(key, DT * n16 / 8) + DT * n16 % 8], vrow[e]);
@@ -338,10 +339,10 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
                             __builtin_amdgcn_perm(vrow[7][t / 2], vrow[6][t / 2], sel)};
         const bf16x8_t va = __builtin_bit_cast(bf16x8_t, vw);
 #pragma unroll
-        for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[i], acc[i][t], 0, 0, 0);
+        for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[i][g], acc[i][t], 0, 0, 0);
       }
     }
-    }  // chunk
+    }
   }
 
 #pragma unroll
