@@ -126,7 +126,9 @@ __device__ __forceinline__ void lds_words(const bf16_t* src, uint32_t* dst) {
   }
 }
 
-template <int RP>
+// RP: query heads per kv head, rounded up to a power of two.  WINDOWED: whether queries have a lower
+// bound on the keys they see; without one the test against it is compiled out.
+template <int RP, bool WINDOWED>
 __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a) {
   __shared__ __attribute__((aligned(16))) bf16_t tiles[2][2][kTileElems];  // [buffer][keys | values]
   constexpr int QB = kCols / RP;  // queries per block
@@ -274,7 +276,7 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
           // plain bit operations, no short-circuit: a branch here, right behind the MFMAs, is what
           // this compiler has been seen to get wrong (the masked value overwrote live scores)
           const int key = base + 16 * sub + 4 * g4 + r;
-          const bool valid = (key >= col_lo[i]) & (key <= col_pos[i]);
+          const bool valid = WINDOWED ? (key >= col_lo[i]) & (key <= col_pos[i]) : key <= col_pos[i];
           const float sc = valid ? c[i][sub][r] : -INFINITY;
           c[i][sub][r] = sc;
           tmax = fmaxf(tmax, sc);
@@ -412,11 +414,18 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
     if ((1 << sh) == page_size) a.page_shift = sh;
   a.scale_log2e = scale * 1.4426950408889634f;
   dim3 grid(n_kv_heads, n_tiles);  // consecutive blocks share a query tile: their loads of q overlap
-  if (R == 1) attn_prefill_kernel<1><<<grid, kThreads, 0, stream>>>(a);
-  else if (R == 2) attn_prefill_kernel<2><<<grid, kThreads, 0, stream>>>(a);
-  else if (R <= 4) attn_prefill_kernel<4><<<grid, kThreads, 0, stream>>>(a);
-  else if (R <= 8) attn_prefill_kernel<8><<<grid, kThreads, 0, stream>>>(a);
-  else attn_prefill_kernel<16><<<grid, kThreads, 0, stream>>>(a);
+  const bool windowed = window > 0;
+#define TL_PREFILL_LAUNCH(rp)                                                      \
+  do {                                                                             \
+    if (windowed) attn_prefill_kernel<rp, true><<<grid, kThreads, 0, stream>>>(a);  \
+    else attn_prefill_kernel<rp, false><<<grid, kThreads, 0, stream>>>(a);          \
+  } while (0)
+  if (R == 1) TL_PREFILL_LAUNCH(1);
+  else if (R == 2) TL_PREFILL_LAUNCH(2);
+  else if (R <= 4) TL_PREFILL_LAUNCH(4);
+  else if (R <= 8) TL_PREFILL_LAUNCH(8);
+  else TL_PREFILL_LAUNCH(16);
+#undef TL_PREFILL_LAUNCH
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return variant_fail(TL_ERR_HIP, "attn_prefill: %s", hipGetErrorString(e));
   return TL_OK;
