@@ -24,6 +24,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 #ifndef TL_HEAD_DIM
@@ -225,7 +227,10 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
 
   dma(tile_begin, 0);
   int buffer = 0;
-  for (int base = tile_begin; base <= key_hi; base += KT, buffer ^= 1) {
+  // One tile of keys: wait for it, start the next one's loads, work it off.  `masked`: whether some
+  // column may not see some key of the tile; where every column sees every key the tests are
+  // compiled out.
+  auto work_tile = [&](int base, auto masked) {
     // this wave's loads of the tile have landed; after the barrier everybody's have, and everybody
     // has finished with the tile before, whose buffer the next tile's loads may now overwrite
     __builtin_amdgcn_s_waitcnt(0);
@@ -234,7 +239,7 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
     const bf16_t* k_lds = tiles[buffer][0];
     const bf16_t* v_lds = tiles[buffer][1];
 
-    if (base > wave_hi || base + KT - 1 < wave_lo) continue;  // nothing here for this wave's columns
+    if (base > wave_hi || base + KT - 1 < wave_lo) return;  // nothing here for this wave's columns
 
     // the whole tile at once: scores, softmax bookkeeping (one running maximum and one rescaling of
     // the sums per tile), then P.V in groups of 32 keys
@@ -275,10 +280,13 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
         for (int r = 0; r < 4; ++r) {
           // plain bit operations, no short-circuit: a branch here, right behind the MFMAs, is what
           // this compiler has been seen to get wrong (the masked value overwrote live scores)
-          const int key = base + 16 * sub + 4 * g4 + r;
-          const bool valid = WINDOWED ? (key >= col_lo[i]) & (key <= col_pos[i]) : key <= col_pos[i];
-          const float sc = valid ? c[i][sub][r] : -INFINITY;
-          c[i][sub][r] = sc;
+          float sc = c[i][sub][r];
+          if constexpr (decltype(masked)::value) {
+            const int key = base + 16 * sub + 4 * g4 + r;
+            const bool valid = WINDOWED ? (key >= col_lo[i]) & (key <= col_pos[i]) : key <= col_pos[i];
+            sc = valid ? sc : -INFINITY;
+            c[i][sub][r] = sc;
+          }
           tmax = fmaxf(tmax, sc);
         }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
@@ -345,7 +353,16 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
       }
     }
     }
+  };
+  // Tiles that lie wholly before the tile's first query (and after no window's edge) are seen by all
+  // columns of the block: they run in a loop of their own, without masks.  The two loops are code
+  // one after the other, not two arms of a branch inside one loop, which is what keeps the register
+  // count where it was.
+  int base = tile_begin;
+  if (!WINDOWED) {
+    for (; base + KT - 1 <= pos0 + q0; base += KT, buffer ^= 1) work_tile(base, std::false_type{});
   }
+  for (; base <= key_hi; base += KT, buffer ^= 1) work_tile(base, std::true_type{});
 
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
