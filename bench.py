@@ -157,7 +157,6 @@ def main(argv=None) -> int:
         return 2
     import torch
 
-    from torchllms_amd.cache.manager import CacheManager
     from torchllms_amd.config import LlamaConfig
     from torchllms_amd.engine import Engine
     from torchllms_amd.sampling import Sampler

@@ -10,8 +10,7 @@ claim order (networks.py:985-990); here any subset of the live requests may run,
 
 from __future__ import annotations
 
-from pathlib import Path
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, Optional, Sequence
 
 import numpy as np
 import torch
@@ -21,7 +20,7 @@ from ..config.registry import ArchSpec, get_architecture, load_config
 from ..parts.model import Model
 from ..weights.loader import load_weights
 from ..weights.random_init import random_tensors
-from .context import StepContext, upload
+from .context import upload
 from .layout import StepEntry, StepLayout, build_step_layout
 
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "fp32": torch.float32, "bf16": torch.bfloat16}

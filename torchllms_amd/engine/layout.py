@@ -11,7 +11,7 @@ matrix per group and the page/offset of each new token is precomputed as ``slot_
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Hashable, List, Sequence
 
 import numpy as np
 

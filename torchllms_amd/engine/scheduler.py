@@ -24,7 +24,7 @@ from __future__ import annotations
 
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional, Sequence
+from typing import Deque, Hashable, List, Optional, Sequence
 
 from ..cache.manager import CacheManager
 from ..sampling.params import SamplingParams
