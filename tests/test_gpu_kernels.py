@@ -622,7 +622,7 @@ def test_attention_decode_window(window):
 def test_attention_decode_batch_with_different_lengths():
     torch.manual_seed(0)
     hq, hkv, dh, page = 32, 8, 128, 16
-    lens = [1, 700, 64, 33, 1024, 250]
+    lens = [1, 700, 64, 33, 2500, 250]
     n_pages = sum(-(-n // page) for n in lens) + 5
     k_pages = torch.full((n_pages, hkv, page, dh), 30.0, dtype=torch.bfloat16)
     v_pages = torch.full((n_pages, hkv, page, dh), -30.0, dtype=torch.bfloat16)
@@ -634,15 +634,16 @@ def test_attention_decode_batch_with_different_lengths():
         for pos in range(S):
             k_pages[table[pos // page], :, pos % page] = k[pos]
             v_pages[table[pos // page], :, pos % page] = v[pos]
-        tables.append(table + [-1] * (64 - len(table)))
+        tables.append(table + [-1] * (160 - len(table)))
         wants.append(plain.attention(q.float(), k.float(), v.float()))
         qs.append(q.reshape(1, hq * dh))
     # queries sit in a wider row, as in the fused q|k|v buffer
     wide = torch.cat([torch.cat(qs), torch.randn(len(lens), 2 * hkv * dh).bfloat16()], dim=1).to(DEV)
-    for split in (None, 64, 512):
+    # the launch's splits: planned for equal lengths, planned for unequal ones, and given
+    for split, uneven in ((None, False), (None, True), (64, False), (512, False)):
         out = _ops().attention_decode(
             wide, hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32(list(range(len(lens)))), _i32([n - 1 for n in lens]),
-            _i32(tables), 0, dh ** -0.5, max(lens), split_size=split,
+            _i32(tables), 0, dh ** -0.5, max(lens), split_size=split, uneven=uneven,
         )
         torch.testing.assert_close(out.float().cpu(), torch.cat(wants), rtol=2 ** -7, atol=2 ** -7)
 
@@ -653,7 +654,10 @@ def test_attention_decode_says_what_it_takes():
     assert not ops.decode_attention_supported(torch.float32, 32, 8, 128)
     assert not ops.decode_attention_supported(torch.bfloat16, 6, 3, 48)
     assert not ops.decode_attention_supported(torch.bfloat16, 16, 1, 256)
-    assert ops.plan_decode_splits(8, 8, 8192) == (512, 16)
+    assert ops.plan_decode_splits(8, 8, 8192) == (1024, 8)
+    assert ops.plan_decode_splits(64, 8, 8192) == (8192, 1)
+    assert ops.plan_decode_splits(64, 8, 8192, uneven=True) == (1024, 8)
+    assert ops.plan_decode_splits(2, 8, 8192, uneven=True) == (256, 32)
     assert ops.plan_decode_splits(64, 8, 40) == (256, 1)
     assert ops.plan_decode_splits(1, 8, 8192) == (256, 32)
 

@@ -79,3 +79,18 @@ def test_bad_entries():
         build_step_layout([StepEntry("r1", [1, 2], want=[2])], [0], [0], [[c.block_table("r1")]], 4)
     with pytest.raises(IndexError):
         build_step_layout([StepEntry("r1", [1] * 9)], [0], [0], [[c.block_table("r1")]], 4)
+
+
+def test_decode_rows_of_unequal_length_are_told_apart():
+    c = CacheManager([CacheGroupSpec("kv0", (0,), 2, 8)], [], page_size=4, num_pages=64, max_seqs=4)
+    for rid, n in (("a", 40), ("b", 44), ("c", 36)):
+        c.admit(rid)
+        c.extend(rid, n)
+        c.advance(rid, n)
+    lay = _plan(c, [StepEntry(r, [1], want=[0]) for r in "abc"], decode_first=True)
+    assert lay.kv_lens.tolist() == [41, 45, 37] and not lay.decode_uneven
+    c.extend("b", 100)
+    c.advance("b", 100)
+    lay = _plan(c, [StepEntry(r, [1], want=[0]) for r in "abc"], decode_first=True)
+    assert lay.kv_lens.tolist() == [42, 146, 38] and lay.decode_uneven  # 146 > 1.5 * mean(75.3)
+    assert not _plan(c, [StepEntry("b", [1], want=[0])], decode_first=True).decode_uneven  # one row

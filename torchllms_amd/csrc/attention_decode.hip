@@ -117,9 +117,14 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
   extern __shared__ float red_o[];  // [kWaves][group][DH]: per-wave partial outputs for the block merge
   __shared__ float red_m[kWaves][16], red_l[kWaves][16];
 
-  const int split = blockIdx.x;
   const int kvh = blockIdx.y;
   const int t = blockIdx.z;
+  // Blocks go to the eight XCDs in turn by their linear index, and a request's later splits are
+  // short or empty when requests differ in length.  Taken as blockIdx.x alone, split s of every
+  // (token, head) would land on the same XCDs (all of them, when the number of splits divides 8):
+  // some XCDs would get the full splits and others the empty ones.  Rotating by head and token
+  // spreads each split index over all XCDs.
+  const int split = (blockIdx.x + blockIdx.y + blockIdx.z) % a.n_splits;
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   const int n16 = lane % 16;  // MFMA column: head within the group; also the key row this lane loads

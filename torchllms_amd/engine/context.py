@@ -19,7 +19,8 @@ class StepContext:
 
     ``decode_longest``: when set, an upper bound of the key range any single-token row sees; kernels
     then size their launches from it instead of from the host plan (a step recorded in a HIP graph
-    must not depend on values that change from replay to replay).
+    must not depend on values that change from replay to replay).  ``decode_uneven`` likewise fixes
+    what the host plan's property of that name would say.
     """
 
     host: StepLayout
@@ -33,6 +34,7 @@ class StepContext:
     block_tables: List[torch.Tensor] = field(default_factory=list)
     slot_mappings: List[torch.Tensor] = field(default_factory=list)
     decode_longest: Optional[int] = None
+    decode_uneven: Optional[bool] = None
     #: what kernels derive from the plan once per step and share between layers
     scratch: dict = field(default_factory=dict)
 
@@ -82,7 +84,8 @@ def pack_into(buf: np.ndarray, layout: StepLayout, shapes, offsets) -> None:
         buf[off : off + sm.size] = sm
 
 
-def make_context(layout: StepLayout, dev: torch.Tensor, shapes, offsets, decode_longest: Optional[int] = None) -> StepContext:
+def make_context(layout: StepLayout, dev: torch.Tensor, shapes, offsets, decode_longest: Optional[int] = None,
+                 decode_uneven: Optional[bool] = None) -> StepContext:
     views = [dev[off : off + int(np.prod(shape))].view(shape) for shape, off in zip(shapes, offsets)]
     n_groups = (len(shapes) - 7) // 2
     return StepContext(
@@ -97,6 +100,7 @@ def make_context(layout: StepLayout, dev: torch.Tensor, shapes, offsets, decode_
         block_tables=[views[7 + 2 * g] for g in range(n_groups)],
         slot_mappings=[views[8 + 2 * g] for g in range(n_groups)],
         decode_longest=decode_longest,
+        decode_uneven=decode_uneven,
     )
 
 

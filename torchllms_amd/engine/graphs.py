@@ -8,8 +8,9 @@ reference reaches for ``torch.compile(mode="reduce-overhead")`` here:
 torchllms/inference/llm.py:202-283.)
 
 A graph is keyed by what fixes its launches: the number of requests, the number of wanted logit
-rows, and a power-of-two cap on the context length, which bounds the block tables' width and the
-number of key splits of the decode attention.  No memset node is recorded: buffers are written by
+rows, a power-of-two cap on the context length, which bounds the block tables' width and the
+number of key splits of the decode attention, and whether the requests differ much in length,
+which makes those splits shorter.  No memset node is recorded: buffers are written by
 kernels only.
 """
 
@@ -38,10 +39,11 @@ class DecodeGraph:
     owns it: a reference cycle would leave the graph to the cyclic garbage collector, which may
     run, and destroy the graph, in the middle of somebody else's stream capture."""
 
-    def __init__(self, model, cache, device, page_size: int, layout: StepLayout, cap: int, pool=None):
+    def __init__(self, model, cache, device, page_size: int, layout: StepLayout, cap: int, pool=None, uneven: bool = False):
         self.model = model
         self.cache = cache
         self.cap = cap
+        self.uneven = uneven
         self.pool = pool
         width = -(-cap // page_size)
         n_groups = len(layout.block_tables)
@@ -65,7 +67,7 @@ class DecodeGraph:
     def first_run(self, layout: StepLayout) -> torch.Tensor:
         """Run the step eagerly (this is the step's real execution), then record the same launches."""
         self._load(layout)
-        ctx = make_context(layout, self.dev, self.shapes, self.offsets, decode_longest=self.cap)
+        ctx = make_context(layout, self.dev, self.shapes, self.offsets, decode_longest=self.cap, decode_uneven=self.uneven)
         logits = self.model.forward(ctx, self.cache)
         result = logits.clone()
         torch.cuda.synchronize()
@@ -95,7 +97,7 @@ class DecodeGraph:
 
 
 class DecodeGraphs:
-    """The engine's recorded decode steps, by (requests, wanted rows, context cap).
+    """The engine's recorded decode steps, by (requests, wanted rows, context cap, uneven lengths).
 
     Recording costs many times a step, so a shape is recorded only when it comes back: the first
     ``record_after`` steps of a shape run eagerly (while requests join one by one every step has a
@@ -109,13 +111,14 @@ class DecodeGraphs:
         self.page_size = page_size
         self.max_graphs = max_graphs
         self.record_after = record_after
-        self.graphs: Dict[Tuple[int, int, int], DecodeGraph] = {}
-        self.seen: Dict[Tuple[int, int, int], int] = {}
+        self.graphs: Dict[Tuple[int, int, int, bool], DecodeGraph] = {}
+        self.seen: Dict[Tuple[int, int, int, bool], int] = {}
         self.pool = None
 
     def run(self, layout: StepLayout) -> torch.Tensor:
         cap = context_cap(layout.max_kv_len)
-        key = (layout.n_seqs, int(layout.logit_rows.size), cap)
+        uneven = layout.decode_uneven
+        key = (layout.n_seqs, int(layout.logit_rows.size), cap, uneven)
         g = self.graphs.get(key)
         if g is not None:
             return g.replay(layout)
@@ -129,6 +132,6 @@ class DecodeGraphs:
             self.graphs.pop(next(iter(self.graphs)))
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
-        g = DecodeGraph(self.model, self.cache, self.device, self.page_size, layout, cap, self.pool)
+        g = DecodeGraph(self.model, self.cache, self.device, self.page_size, layout, cap, self.pool, uneven)
         self.graphs[key] = g
         return g.first_run(layout)

@@ -48,6 +48,18 @@ class StepLayout:
     max_q_len: int = 0
     max_kv_len: int = 0
 
+    @property
+    def decode_uneven(self) -> bool:
+        """Whether the single-token rows differ much in context length: the longest holds more
+        than one and a half times the mean.  The decode attention kernel then cuts the keys into
+        shorter splits, so that the blocks of long requests spread over the CUs that short
+        requests leave early."""
+        n = self.n_decode
+        if n < 2:
+            return False
+        lens = self.kv_lens[:n]
+        return 2 * n * int(lens.max()) > 3 * int(lens.sum())
+
     # the reference's names for the same facts, for comparison with its test vectors
     @property
     def kv_indptr(self) -> List[int]:

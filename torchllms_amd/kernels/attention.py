@@ -46,9 +46,11 @@ def paged_attention(
                 longest = int(ctx.host.positions[:n_dec].max()) + 1
             if window > 0:
                 longest = min(longest, window + 15)
+            uneven = ctx.decode_uneven if ctx.decode_uneven is not None else ctx.host.decode_uneven
             ops.attention_decode(
                 qkv[:n_dec], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[:n_dec],
                 ctx.positions[:n_dec], ctx.block_tables[group], window, scale, longest, out=out[:n_dec],
+                uneven=uneven,
             )
         else:
             ops.attention_generic(
