@@ -735,10 +735,125 @@ def test_tune_linear_remembers_a_choice_for_every_row_bucket():
         del ops._LINEAR_CHOICE[key]
     ops.tune_linear(weights)
     for bucket in ops.ROW_BUCKETS:
-        assert ops._LINEAR_CHOICE[(48, 64, bucket)] in (None,) + tuple(ops.STREAM_WAVE_CHOICES)
+        if bucket <= ops.STREAM_MAX_ROWS:
+            assert ops._LINEAR_CHOICE[(48, 64, bucket, "plain")] in (None,) + tuple(("stream", w) for w in ops.STREAM_WAVE_CHOICES)
+        else:
+            assert ops._LINEAR_CHOICE[(48, 64, bucket, "plain")] is None  # K = 64 is no multiple of 128: the library
     x = torch.randn(5, 64, device=DEV).bfloat16()
     got = ops.linear(x, weights[0]).float().cpu()
     torch.testing.assert_close(got, (x.float() @ weights[0].float().T).cpu(), rtol=2 ** -7, atol=0.1)
+
+
+# ----------------------------------------------------------------------------- shared-activation matrix product (17 to 64 rows)
+@pytest.mark.parametrize(
+    "m, n, k",
+    [(64, 4096, 4096), (32, 6144, 4096), (17, 200, 128), (64, 4100, 384), (33, 72, 2048), (48, 1000, 1024), (5, 64, 256),
+     (64, 128, 14336), (49, 130, 640)],
+)
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_wide(m, n, k, out_dtype):
+    """Both row tiles (32 and 64), N that is no multiple of a block's columns, one step of K and
+    many, every block shape, splits of K that divide the steps and that do not, both buffer counts."""
+    torch.manual_seed(0)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) * 0.05).bfloat16()
+    want = x.double() @ w.double().T
+    tol = (1e-4 if out_dtype == torch.float32 else 2 ** -8) * want.abs().max().item() + 1e-5
+    for strips in (1, 2):
+        for splits in (1, 2, 3, 8):
+            for stages in (2, 3):
+                got = _ops().gemm_wide(x.to(DEV), w.to(DEV), out_dtype, strips, splits, stages).float().cpu()
+                assert (got.double() - want).abs().max().item() <= tol, f"strips={strips} splits={splits} stages={stages}"
+
+
+@pytest.mark.parametrize("m, f, k", [(64, 14336, 4096), (32, 1000, 256), (17, 40, 128), (50, 72, 1152)])
+def test_gemm_wide_glu_equals_the_product_followed_by_the_gate(m, f, k):
+    """The same roundings as the two kernels it replaces (see the streaming kernel's test)."""
+    torch.manual_seed(1)
+    x = torch.randn(m, k).bfloat16().to(DEV)
+    w = (torch.randn(2 * f, k) * 0.1).bfloat16().to(DEV)
+    ref = torch.nn.functional.silu(x.float() @ w[:f].float().T) * (x.float() @ w[f:].float().T)
+    for strips in (1, 2):
+        for stages in (2, 3):
+            want = _ops().silu_mul(_ops().gemm_wide(x, w, torch.bfloat16, strips, 1, stages))
+            got = _ops().gemm_wide_glu(x, w, strips, stages)
+            torch.testing.assert_close(got.float(), want.float(), rtol=2 ** -6, atol=2 ** -8 * want.float().abs().max().item(), msg=f"strips={strips}")
+            assert (got != want).float().mean().item() < 0.05, f"strips={strips} stages={stages}"
+            torch.testing.assert_close(got.float(), ref, rtol=2 ** -6, atol=2 ** -6 * ref.abs().max().item())
+
+
+@pytest.mark.parametrize("m, hq, hkv, dh, rot, page, k", [(64, 32, 8, 128, 128, 16, 4096), (32, 4, 4, 64, 64, 16, 256),
+                                                           (23, 6, 3, 48, 24, 4, 384), (40, 5, 1, 20, 0, 8, 128)])
+@pytest.mark.parametrize("with_pages", [True, False])
+def test_gemm_wide_qkv_equals_product_then_rotary_kernel(m, hq, hkv, dh, rot, page, k, with_pages):
+    """The split product whose second kernel rotates and scatters, against product and rotary
+    kernel in turn, on every output; a row whose slot is negative stores nothing."""
+    torch.manual_seed(2)
+    width = (hq + 2 * hkv) * dh
+    x = torch.randn(m, k).bfloat16().to(DEV)
+    w = (torch.randn(width, k) * k ** -0.5).bfloat16().to(DEV)
+    pos = torch.randint(0, 9000, (m,))
+    inv_freq = plain.rope_inverse_frequencies(rot, 500000.0, None).to(DEV) if rot else None
+    table = _ops().rope_table(_i32(pos.tolist()), inv_freq) if rot else None
+    n_pages = 80
+    slots = torch.randperm(n_pages * page)[:m].tolist()
+    slots[1] = -1
+    sm = _i32(slots) if with_pages else None
+    ka, va = _pages(n_pages, hkv, page, dh, torch.bfloat16) if with_pages else (None, None)
+    qa = _ops().gemm_wide(x, w, torch.bfloat16, 1, 1, 2)
+    _ops().rope_kv_write(qa, hq, hkv, dh, _i32(pos.tolist()), inv_freq, rot, 0, ka, va, sm, page if with_pages else 0, cos_sin=table)
+    cols = hq * dh if with_pages else width  # with pages only the queries of the buffer are defined
+    tol = dict(rtol=2 ** -7, atol=2 ** -8 * qa.float().abs().max().item())
+    for strips, splits, stages in ((1, 1, 3), (1, 2, 3), (2, 4, 2), (1, 8, 3)):
+        kb, vb = _pages(n_pages, hkv, page, dh, torch.bfloat16) if with_pages else (None, None)
+        qb = _ops().gemm_wide_qkv(x, w, hq, hkv, dh, rot, table, kb, vb, sm, page if with_pages else 0, strips, splits, stages)
+        torch.testing.assert_close(qb[:, :cols].float(), qa[:, :cols].float(), **tol)
+        assert (qb[:, :cols] != qa[:, :cols]).float().mean().item() < 0.05  # only last-bit differences of the sums
+        if with_pages:
+            torch.testing.assert_close(kb.float(), ka.float(), **tol)
+            torch.testing.assert_close(vb.float(), va.float(), **tol)
+            assert (kb.float().abs().sum(dim=(1, 3)) > 0).sum().item() == m - 1  # one slot per stored row
+
+
+def test_gemm_wide_takes_strided_rows_and_says_its_limits():
+    from torchllms_amd.kernels.lib import KernelError
+
+    torch.manual_seed(0)
+    buf = torch.randn(40, 512).bfloat16().to(DEV)
+    x = buf[:, :256]  # row stride 512
+    w = torch.randn(70, 256).bfloat16().to(DEV)
+    got = _ops().gemm_wide(x, w, torch.float32, 2, 2).cpu()
+    torch.testing.assert_close(got, (x.float() @ w.float().T).cpu(), rtol=1e-4, atol=1e-3)
+    with pytest.raises(KernelError, match="exceeds 64"):
+        _ops().gemm_wide(torch.zeros(65, 256, dtype=torch.bfloat16, device=DEV), w)
+    with pytest.raises(KernelError, match="multiple of 128"):
+        _ops().gemm_wide(torch.zeros(20, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
+    with pytest.raises(KernelError, match="stages"):
+        _ops().gemm_wide(x, w, torch.float32, 1, 1, 4)
+
+
+def test_tune_linear_measures_the_wide_kernel_from_17_rows_on():
+    ops = _ops()
+    torch.manual_seed(0)
+    weights = [(torch.randn(96, 256, device=DEV) * 0.1).bfloat16() for _ in range(2)]
+    for key in [k for k in ops._LINEAR_CHOICE if k[:2] == (96, 256)]:
+        del ops._LINEAR_CHOICE[key]
+    for use in ops.LINEAR_USES:
+        ops.tune_linear(weights, use=use)
+    allowed = {None} | {("wide",) + c for c in ops.WIDE_CHOICES if c[1] <= 2}
+    for use in ops.LINEAR_USES:
+        assert ops._LINEAR_CHOICE[(96, 256, 32, use)] in allowed and ops._LINEAR_CHOICE[(96, 256, 64, use)] in allowed
+    # whatever was chosen, and each of the kernel's launches when it is forced, gives the product
+    x = torch.randn(40, 256, device=DEV).bfloat16()
+    want = (x.float() @ weights[0].float().T).cpu()
+    torch.testing.assert_close(ops.linear(x, weights[0]).float().cpu(), want, rtol=2 ** -7, atol=0.05)
+    glu_ref = (torch.nn.functional.silu(x.float() @ weights[0][:48].float().T) * (x.float() @ weights[0][48:].float().T)).cpu()
+    for choice in sorted(allowed - {None}) + [("wide", 1, 2, 2)]:
+        ops._LINEAR_CHOICE[(96, 256, 64, "plain")] = ops._LINEAR_CHOICE[(96, 256, 64, "glu")] = choice
+        torch.testing.assert_close(ops.linear(x, weights[0]).float().cpu(), want, rtol=2 ** -7, atol=0.05)
+        torch.testing.assert_close(ops.linear_glu(x, weights[0]).float().cpu(), glu_ref, rtol=2 ** -6, atol=0.05)
+    for use in ops.LINEAR_USES:
+        del ops._LINEAR_CHOICE[(96, 256, 64, use)]
 
 
 # ----------------------------------------------------------------------------- prefill attention (MFMA)

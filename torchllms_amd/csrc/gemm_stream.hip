@@ -22,6 +22,7 @@
 //     and values go straight into their cache pages, queries into C: the rotary kernel's work, done
 //     on the 32-bit sums after the rounding the unfused product would have applied.
 #include "common.h"
+#include "qkv_epilogue.h"
 
 namespace {
 
@@ -39,17 +40,6 @@ __device__ __forceinline__ short4_t lo_half(u32x4_t v) { return __builtin_bit_ca
 __device__ __forceinline__ short4_t hi_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[2], v[3]}); }
 
 enum Epilogue { kPlain = 0, kGated = 1, kQkv = 2 };
-
-// What the query/key/value epilogue needs beside the product.
-struct QkvArgs {
-  int n_q_heads, n_kv_heads, head_dim;
-  int rotary_dim;                 // leading channels of a head that rotate (even; 0: none)
-  const float2* cos_sin;          // [row of A][rotary_dim / 2] = (cos, sin) of the row's position
-  bf16_t* k_pages;                // [page][kv head][page_size][head_dim], or null: keys and values stay in C
-  bf16_t* v_pages;
-  const int32_t* slot_mapping;    // per row of A: page * page_size + offset, < 0: not stored
-  int page_size;
-};
 
 // MR: groups of four rows of A that are fetched (M <= 4 * MR).  WAVES: waves per block = splits of K.
 // EPI kGated: W holds 2 N rows, gate rows then up rows; C[M, N] = silu(A gate^T) * (A up^T).
@@ -199,41 +189,11 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
       }
   }
   if constexpr (EPI == kQkv) {
-    // the lane's four columns are channels d .. d+3 of one head (the host checks head_dim % 4 == 0
-    // and N % 4 == 0): two rotary pairs
+    // the lane's four columns are channels of one head (N % 4 == 0)
     const int n = n0 + 4 * g4;
     if (n16 < M && n < N) {
-      const int head = n / qa.head_dim;
-      const int d = n % qa.head_dim;
-      float x[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) x[i] = to_f32(from_f32<bf16_t>(acc[0][i]));  // as the stored product would read
-      if (head < qa.n_q_heads + qa.n_kv_heads) {
-#pragma unroll
-        for (int pi = 0; pi < 2; ++pi) {
-          if (d + 2 * pi < qa.rotary_dim) {
-            const float2 cs = qa.cos_sin[(size_t)n16 * (qa.rotary_dim / 2) + (d / 2 + pi)];
-            const float x0 = x[2 * pi], x1 = x[2 * pi + 1];
-            x[2 * pi] = x0 * cs.x - x1 * cs.y;
-            x[2 * pi + 1] = x1 * cs.x + x0 * cs.y;
-          }
-        }
-      }
-      const u32x2_t packed = {
-          (uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x[0])) | ((uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x[1])) << 16),
-          (uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x[2])) | ((uint32_t)__builtin_bit_cast(uint16_t, from_f32<bf16_t>(x[3])) << 16)};
-      bf16_t* dst = reinterpret_cast<bf16_t*>(C) + (size_t)n16 * ldc + n;
-      bool store = true;
-      if (head >= qa.n_q_heads && qa.k_pages != nullptr) {
-        const int slot = qa.slot_mapping[n16];
-        store = slot >= 0;
-        const int kvh = head < qa.n_q_heads + qa.n_kv_heads ? head - qa.n_q_heads : head - qa.n_q_heads - qa.n_kv_heads;
-        bf16_t* pages = head < qa.n_q_heads + qa.n_kv_heads ? qa.k_pages : qa.v_pages;
-        const int page = store ? slot / qa.page_size : 0;
-        const int off = store ? slot % qa.page_size : 0;
-        dst = pages + (((size_t)page * qa.n_kv_heads + kvh) * qa.page_size + off) * qa.head_dim + d;
-      }
-      if (store) *reinterpret_cast<u32x2_t*>(dst) = packed;
+      const float sums[4] = {acc[0][0], acc[0][1], acc[0][2], acc[0][3]};
+      qkv_finish(sums, n16, n, qa, reinterpret_cast<bf16_t*>(C), ldc);
     }
   } else if (n16 < M) {
 #pragma unroll
@@ -339,16 +299,10 @@ TL_EXPORT int tl_gemm_stream_qkv(const void* A, int lda, const void* W, int ldw,
                                  int n_q_heads, int n_kv_heads, int head_dim, int rotary_dim,
                                  const float* cos_sin, void* k_pages, void* v_pages,
                                  const int32_t* slot_mapping, int page_size, int waves, hipStream_t stream) {
-  TL_REQUIRE(n_q_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && head_dim % 4 == 0, "gemm_stream_qkv: bad head sizes");
-  TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "gemm_stream_qkv: bad rotary_dim=%d", rotary_dim);
-  TL_REQUIRE(rotary_dim == 0 || cos_sin != nullptr, "gemm_stream_qkv: the table of cosines and sines is missing");
-  TL_REQUIRE(k_pages == nullptr || (v_pages != nullptr && slot_mapping != nullptr && page_size > 0),
-             "gemm_stream_qkv: pages given without v_pages/slot_mapping/page_size");
-  TL_REQUIRE(ldc % 4 == 0 && ((uintptr_t)C % 8) == 0, "gemm_stream_qkv: rows of C must start on 8-byte boundaries");
   QkvArgs qa;
-  qa.n_q_heads = n_q_heads; qa.n_kv_heads = n_kv_heads; qa.head_dim = head_dim; qa.rotary_dim = rotary_dim;
-  qa.cos_sin = (const float2*)cos_sin; qa.k_pages = (bf16_t*)k_pages; qa.v_pages = (bf16_t*)v_pages;
-  qa.slot_mapping = slot_mapping; qa.page_size = page_size;
+  const int rc = qkv_args("gemm_stream_qkv", n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages,
+                          slot_mapping, page_size, C, ldc, &qa);
+  if (rc != TL_OK) return rc;
   const int N = (n_q_heads + 2 * n_kv_heads) * head_dim;
   return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, kQkv, qa, stream);
 }

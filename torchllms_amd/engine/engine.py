@@ -101,8 +101,8 @@ class Engine:
             # which matrix-product kernel serves decode steps best is measured, not guessed
             from ..kernels import ops
 
-            for shape, group in self.model.linear_weights().items():
-                ops.tune_linear(group, torch.float32 if group[0] is self.model.head.weight else torch.bfloat16)
+            for (shape, use), group in self.model.linear_weights().items():
+                ops.tune_linear(group, torch.float32 if group[0] is self.model.head.weight else torch.bfloat16, use)
         # decode steps are replayed from HIP graphs when every mixer's launches are fixed by the
         # step's shape alone
         from .graphs import DecodeGraphs

@@ -33,9 +33,10 @@ CORE_SOURCES = [
     "attention_generic.hip",
     "gemm_f32.hip",
     "gemm_stream.hip",
+    "gemm_wide.hip",
     "sampling.hip",
 ]
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "qkv_epilogue.h"]
 
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}",

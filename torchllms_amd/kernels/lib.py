@@ -35,6 +35,9 @@ _CORE_SIGNATURES = {
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "tl_gemm_stream_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _P],
+    "tl_gemm_wide": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P],
+    "tl_gemm_wide_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "tl_gemm_wide_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P],
     "tl_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P],
     "tl_philox_uniform": [_U64, _U64, _P, _I, _P],
 }

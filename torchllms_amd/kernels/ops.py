@@ -254,6 +254,107 @@ def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     return out
 
 
+WIDE_MAX_ROWS = 64
+
+
+def _wide_shapes(x: torch.Tensor, w: torch.Tensor, what: str) -> None:
+    _gpu(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"{what} takes bfloat16 tensors")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelError(f"{what}: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
+
+
+def gemm_wide(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, strips_per_wave: int = 1,
+              k_splits: int = 1, stages: int = 3) -> torch.Tensor:
+    """``x @ w.T`` for at most 64 rows of bfloat16 ``x`` (K a multiple of 128) with the kernel whose
+    blocks share their slice of ``x`` through LDS; ``k_splits`` > 1 cuts K over several blocks whose
+    32-bit partial sums a second kernel adds."""
+    _wide_shapes(x, w, "gemm_wide")
+    m, k = x.shape
+    n = w.shape[0]
+    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    partial = torch.empty((k_splits, m, n), dtype=torch.float32, device=x.device) if k_splits > 1 else None
+    check(
+        core().tl_gemm_wide(
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k,
+            dtype_code(out_dtype), strips_per_wave, k_splits, stages, _ptr(partial), _stream(),
+        )
+    )
+    return out
+
+
+def gemm_wide_glu(x: torch.Tensor, w: torch.Tensor, strips_per_wave: int = 1, stages: int = 3) -> torch.Tensor:
+    """``silu(x @ gate.T) * (x @ up.T)`` for at most 64 rows of bfloat16 ``x`` and ``w`` [2F, K] =
+    gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``."""
+    _wide_shapes(x, w, "gemm_wide_glu")
+    if w.shape[0] % 2:
+        raise KernelError("gemm_wide_glu: w must hold gate rows and as many up rows")
+    m, k = x.shape
+    n = w.shape[0] // 2
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    check(
+        core().tl_gemm_wide_glu(
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k,
+            strips_per_wave, stages, _stream(),
+        )
+    )
+    return out
+
+
+def _qkv_shapes(what, x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size) -> int:
+    """Checks the arguments that the fused query|key|value products share; returns the output width."""
+    _gpu(x, w, cos_sin, k_pages, v_pages, slot_mapping)
+    _i32(slot_mapping, "slot_mapping")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"{what} takes bfloat16 tensors")
+    width = (n_q_heads + 2 * n_kv_heads) * head_dim
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1 or w.shape[0] != width:
+        raise KernelError(f"{what}: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match {width} output columns")
+    m = x.shape[0]
+    if rotary_dim > 0 and (cos_sin is None or cos_sin.dtype != torch.float32 or tuple(cos_sin.shape) != (m, rotary_dim // 2, 2) or not cos_sin.is_contiguous()):
+        raise KernelError(f"cos_sin must be contiguous float32 [{m}, {rotary_dim // 2}, 2]")
+    if k_pages is not None:
+        if v_pages is None or slot_mapping is None or slot_mapping.numel() != m:
+            raise KernelError("pages need v_pages and one slot per row")
+        for pg in (k_pages, v_pages):
+            if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != torch.bfloat16 or not pg.is_contiguous():
+                raise KernelError(f"pages must be contiguous bfloat16 [pages, {n_kv_heads}, {page_size}, {head_dim}], got {tuple(pg.shape)} {pg.dtype}")
+    return width
+
+
+def gemm_wide_qkv(
+    x: torch.Tensor,
+    w: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    rotary_dim: int,
+    cos_sin: Optional[torch.Tensor],
+    k_pages: Optional[torch.Tensor],
+    v_pages: Optional[torch.Tensor],
+    slot_mapping: Optional[torch.Tensor],
+    page_size: int,
+    strips_per_wave: int = 1,
+    k_splits: int = 4,
+    stages: int = 3,
+) -> torch.Tensor:
+    """As ``gemm_stream_qkv`` for at most 64 rows: the product split along K, and the kernel that
+    adds the splits rotates the heads and writes keys and values into their pages."""
+    width = _qkv_shapes("gemm_wide_qkv", x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size)
+    m, k = x.shape
+    out = torch.empty((m, width), dtype=torch.bfloat16, device=x.device)
+    partial = torch.empty((k_splits, m, width), dtype=torch.float32, device=x.device)
+    check(
+        core().tl_gemm_wide_qkv(
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, k,
+            n_q_heads, n_kv_heads, head_dim, rotary_dim, _ptr(cos_sin), _ptr(k_pages), _ptr(v_pages),
+            _ptr(slot_mapping), page_size, strips_per_wave, k_splits, stages, partial.data_ptr(), _stream(),
+        )
+    )
+    return out
+
+
 def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0) -> torch.Tensor:
     """``silu(x @ gate.T) * (x @ up.T)`` for at most 16 rows of bfloat16 ``x`` and ``w`` [2F, K] =
     gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``."""
@@ -291,22 +392,8 @@ def gemm_stream_qkv(
     rotation (interleaved pairs, from the ``rope_table`` of the rows' positions) and the cache
     write in the kernel's epilogue.  Returns [n, (Hq + 2 Hkv) * dh] whose query part is rotated;
     the key and value parts are only filled when no pages are given."""
-    _gpu(x, w, cos_sin, k_pages, v_pages, slot_mapping)
-    _i32(slot_mapping, "slot_mapping")
-    width = (n_q_heads + 2 * n_kv_heads) * head_dim
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise KernelError("gemm_stream_qkv takes bfloat16 tensors")
-    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1 or w.shape[0] != width:
-        raise KernelError(f"gemm_stream_qkv: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match {width} output columns")
+    width = _qkv_shapes("gemm_stream_qkv", x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size)
     m, k = x.shape
-    if rotary_dim > 0 and (cos_sin is None or cos_sin.dtype != torch.float32 or tuple(cos_sin.shape) != (m, rotary_dim // 2, 2) or not cos_sin.is_contiguous()):
-        raise KernelError(f"cos_sin must be contiguous float32 [{m}, {rotary_dim // 2}, 2]")
-    if k_pages is not None:
-        if v_pages is None or slot_mapping is None or slot_mapping.numel() != m:
-            raise KernelError("pages need v_pages and one slot per row")
-        for pg in (k_pages, v_pages):
-            if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != torch.bfloat16 or not pg.is_contiguous():
-                raise KernelError(f"pages must be contiguous bfloat16 [pages, {n_kv_heads}, {page_size}, {head_dim}], got {tuple(pg.shape)} {pg.dtype}")
     out = torch.empty((m, width), dtype=torch.bfloat16, device=x.device)
     check(
         core().tl_gemm_stream_qkv(
@@ -326,12 +413,33 @@ def stream_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
     )
 
 
-#: measured choice of bfloat16 kernel: (n, k, row bucket) -> number of waves (splits of K) for the
-#: weight-streaming kernel (0 = its own rule), or None for the library.  Filled by ``tune_linear``;
-#: shapes never measured follow the size rule.
+def wide_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the kernel for 17 to 64 rows can take this product at all."""
+    return (
+        x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and STREAM_MAX_ROWS < x.shape[0] <= WIDE_MAX_ROWS
+        and x.shape[1] % 128 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+        and w.data_ptr() % 16 == 0
+    )
+
+
+#: measured choice of bfloat16 kernel by (n, k, row bucket, use); filled by ``tune_linear``:
+#:   ("stream", waves)                             the weight-streaming kernel (waves 0 = its own rule)
+#:   ("wide", strips_per_wave, k_splits, stages)   the kernel whose blocks share the activations
+#:   None                                          the library
+#: Shapes never measured follow the size rule below.
 _LINEAR_CHOICE: dict = {}
-ROW_BUCKETS = (1, 2, 4, 8, 16)
+ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64)
 STREAM_WAVE_CHOICES = (0, 4)
+#: (strips per wave, splits of K, buffers) that ``tune_linear`` tries from 17 rows on: whole-K
+#: launches for matrices with many rows, splits of K for those with few
+WIDE_CHOICES = ((1, 1, 3), (2, 1, 3), (1, 4, 3), (1, 8, 3), (2, 8, 3))
+#: how a product is used: alone, or as the first half of ``linear_glu`` / ``qkv_rope_store``, whose
+#: second half (gate, rotation and cache write) some kernels take into themselves
+LINEAR_USES = ("plain", "glu", "qkv")
+#: microseconds that a small kernel between large ones costs in a replayed decode step (measured);
+#: ``tune_linear`` charges it to a candidate that leaves the second half of a fused use to a kernel
+#: of its own
+_TAIL_KERNEL_US = 4.5
 
 
 def _row_bucket(m: int) -> int:
@@ -341,84 +449,146 @@ def _row_bucket(m: int) -> int:
     return ROW_BUCKETS[-1]
 
 
-def stream_choice(x: torch.Tensor, w: torch.Tensor):
-    """The number of waves when the weight-streaming kernel should run this product, else None."""
-    if not stream_supported(x, w):
+def _fuses_tail(choice, use: str) -> bool:
+    """Whether the kernel of ``choice`` does the second half of ``use`` itself."""
+    if use == "plain" or choice is None:
+        return use == "plain"
+    if choice[0] == "stream":
+        return True
+    return choice[2] == 1 if use == "glu" else choice[2] > 1  # the gate ends a whole product, the rotation a split one
+
+
+def linear_choice(x: torch.Tensor, w: torch.Tensor, use: str = "plain"):
+    """Which bfloat16 kernel runs ``x @ w.T``: a tuple as in the table above, or None for the library."""
+    m = x.shape[0]
+    if m <= STREAM_MAX_ROWS:
+        if not stream_supported(x, w):
+            return None
+        key = (w.shape[0], w.shape[1], _row_bucket(m), use)
+        if key in _LINEAR_CHOICE:
+            return _LINEAR_CHOICE[key]
+        return ("stream", 0) if w.shape[0] * w.shape[1] <= STREAM_MAX_ELEMENTS else None
+    if not wide_supported(x, w):
         return None
-    key = (w.shape[0], w.shape[1], _row_bucket(x.shape[0]))
-    if key in _LINEAR_CHOICE:
-        return _LINEAR_CHOICE[key]
-    return 0 if w.shape[0] * w.shape[1] <= STREAM_MAX_ELEMENTS else None
+    return _LINEAR_CHOICE.get((w.shape[0], w.shape[1], _row_bucket(m), use))
 
 
-def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, iters: int = 4) -> None:
+_TUNE_FLUSH_BYTES = 512 << 20  # twice the 256 MB of last-level cache
+
+
+def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "plain", iters: int = 8) -> None:
     """Measure, for matrices of one shape and every row bucket, which bfloat16 kernel and launch is
-    fastest on this GPU, and remember it.  ``weights``: the model's tensors of that shape; timing
-    rotates over them, as a decode step does, so that no run is served from cache.  Shapes already
+    fastest on this GPU, and remember it.  ``weights``: the model's tensors of that shape; ``use``:
+    one of ``LINEAR_USES``.  The plain product is what is timed; a candidate that cannot take the
+    second half of a fused use into itself is charged the kernel that has to follow it.
+
+    Timing is made like a decode step: the launches are recorded into a HIP graph and replayed (a
+    product that needs two kernels is then charged what a second graph node costs, not what a
+    second launch from Python costs), they rotate over the tensors, and the caches are flushed
+    before every replay, so that the matrices come from HBM as they do in a step.  Shapes already
     measured are left alone, so every engine of a process makes the same choice."""
+    import gc
+
     weights = [w for w in weights if w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2]
     if not weights:
         return
     n, k = weights[0].shape
     if k % 8 or weights[0].stride(0) % 8:
         return
+    if use not in LINEAR_USES:
+        raise ValueError(f"use must be one of {LINEAR_USES}, got {use!r}")
+    if all((n, k, bucket, use) in _LINEAR_CHOICE for bucket in ROW_BUCKETS):
+        return
+    device = weights[0].device
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    flush = torch.empty(_TUNE_FLUSH_BYTES, dtype=torch.uint8, device=device)
 
     def clock(fn) -> float:
-        for i in range(2):
+        for i in range(2):  # loads the kernel's code and lets it ask for its LDS before the recording
             fn(weights[i % len(weights)])
+        torch.cuda.synchronize(device)
+        graph = torch.cuda.CUDAGraph()
+        # nothing may be destroyed while the stream is recording: the collector stays off meanwhile
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                for i in range(iters):
+                    fn(weights[(i + 2) % len(weights)])
+        finally:
+            if collecting:
+                gc.enable()
         best = float("inf")
-        for rep in range(3):  # the least of three rounds: a stall of the machine does not decide
+        for _ in range(3):  # the least of three replays: a stall of the machine does not decide
+            flush.zero_()
             start.record()
-            for i in range(iters):
-                fn(weights[(i + 2 + rep) % len(weights)])
+            graph.replay()
             stop.record()
             stop.synchronize()
             best = min(best, start.elapsed_time(stop))
         return best
 
+    def cost(choice, fn) -> float:
+        tail = 0.0 if _fuses_tail(choice, use) else _TAIL_KERNEL_US * 1e-3 * iters
+        return clock(fn) + tail
+
     for bucket in ROW_BUCKETS:
-        if (n, k, bucket) in _LINEAR_CHOICE:
+        if (n, k, bucket, use) in _LINEAR_CHOICE:
             continue
-        x = torch.randn((bucket, k), device=weights[0].device, dtype=torch.float32).to(torch.bfloat16)
+        x = torch.randn((bucket, k), device=device, dtype=torch.float32).to(torch.bfloat16)
 
         def library(w):
             y = torch.nn.functional.linear(x, w)
             return y if y.dtype == out_dtype else y.to(out_dtype)
 
-        best, best_time = None, clock(library)
-        for waves in STREAM_WAVE_CHOICES:
-            t = clock(lambda w: gemm_stream(x, w, out_dtype, waves))
+        best, best_time = None, cost(None, library)
+        if bucket <= STREAM_MAX_ROWS:
+            candidates = [("stream", waves) for waves in STREAM_WAVE_CHOICES]
+        elif wide_supported(x, weights[0]):
+            candidates = [("wide",) + c for c in WIDE_CHOICES if c[1] <= k // 128]
+        else:
+            candidates = []
+        for choice in candidates:
+            t = cost(choice, lambda w: _run_choice(choice, x, w, out_dtype))
             if t < best_time:
-                best, best_time = waves, t
-        _LINEAR_CHOICE[(n, k, bucket)] = best
+                best, best_time = choice, t
+        _LINEAR_CHOICE[(n, k, bucket, use)] = best
+
+
+def _run_choice(choice, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    if choice is None:
+        y = torch.nn.functional.linear(x, w)
+        return y if y.dtype == out_dtype else y.to(out_dtype)
+    if choice[0] == "stream":
+        return gemm_stream(x, w, out_dtype, choice[1])
+    return gemm_wide(x, w, out_dtype, choice[1], choice[2], choice[3])
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16: for up to 16 rows (decode steps)
-    the weight-streaming MFMA kernel or the BLAS library's matrix product, whichever was measured
-    faster for the shape (``tune_linear``); for more rows the library, as the reference uses its
-    library's (torchllms/models/networks.py:474-493).  ``out_dtype`` float32 asks for 32-bit
-    results from bfloat16 inputs (logits)."""
+    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16: for up to 64 rows (decode steps)
+    one of the two MFMA kernels that are built around reading ``w`` once, or the BLAS library's
+    matrix product, whichever was measured faster for the shape (``tune_linear``); for more rows the
+    library, as the reference uses its library's (torchllms/models/networks.py:474-493).
+    ``out_dtype`` float32 asks for 32-bit results from bfloat16 inputs (logits)."""
     if x.dtype == torch.float32:
         return gemm_f32(x, w)
     _gpu(x, w)
     out_dtype = out_dtype or x.dtype
-    waves = stream_choice(x, w)
-    if waves is not None:
-        return gemm_stream(x, w, out_dtype, waves)
-    y = torch.nn.functional.linear(x, w)
-    return y if y.dtype == out_dtype else y.to(out_dtype)
+    return _run_choice(linear_choice(x, w), x, w, out_dtype)
 
 
 def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """``silu(x @ gate.T) * (x @ up.T)`` for ``w`` [2F, K] = gate rows | up rows: one fused kernel
-    where the weight-streaming kernel serves the shape, else the product followed by the gate."""
-    if x.dtype == torch.bfloat16:
-        waves = stream_choice(x, w)
-        if waves is not None:
-            return gemm_stream_glu(x, w, waves)
-    return silu_mul(linear(x, w))
+    where one of the decode kernels serves the shape, else the product followed by the gate."""
+    if x.dtype != torch.bfloat16:
+        return silu_mul(linear(x, w))
+    _gpu(x, w)
+    choice = linear_choice(x, w, "glu")
+    if choice is not None and choice[0] == "stream":
+        return gemm_stream_glu(x, w, choice[1])
+    if choice is not None and choice[0] == "wide" and choice[2] == 1:
+        return gemm_wide_glu(x, w, choice[1], choice[3])
+    return silu_mul(_run_choice(choice, x, w, x.dtype))
 
 
 def qkv_rope_store(
@@ -440,16 +610,26 @@ def qkv_rope_store(
 ) -> torch.Tensor:
     """Projection into query | key | value heads, rotation of queries and keys by position, keys
     and values appended to their pages; returns the row-major [n, (Hq + 2 Hkv) * dh] buffer whose
-    query part the attention kernels read.  One fused kernel where the weight-streaming kernel
-    serves the product (few bfloat16 rows, no bias, interleaved pairs, head size a multiple of 4),
-    else product, bias and rotary kernels in turn."""
-    if x.dtype == torch.bfloat16 and bias is None and (rotary_dim == 0 or pairing == 0) and head_dim % 4 == 0:
-        waves = stream_choice(x, w)
-        if waves is not None and (rotary_dim == 0 or cos_sin is not None):
+    query part the attention kernels read.  Fused into the product's own kernels where one of the
+    decode kernels serves it (at most 64 bfloat16 rows, no bias, interleaved pairs, head size a
+    multiple of 4), else product, bias and rotary kernels in turn."""
+    if x.dtype == torch.bfloat16:
+        _gpu(x, w)
+        choice = linear_choice(x, w, "qkv")
+        fusable = bias is None and head_dim % 4 == 0 and (rotary_dim == 0 or (pairing == 0 and cos_sin is not None))
+        if fusable and choice is not None and choice[0] == "stream":
             return gemm_stream_qkv(
-                x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size, waves
+                x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size, choice[1]
             )
-    qkv = linear(x, w)
+        # (a product that is not split ends without a second kernel, so the rotary kernel follows it)
+        if fusable and choice is not None and choice[0] == "wide" and choice[2] > 1:
+            return gemm_wide_qkv(
+                x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size,
+                choice[1], choice[2], choice[3],
+            )
+        qkv = _run_choice(choice, x, w, x.dtype)
+    else:
+        qkv = linear(x, w)
     if bias is not None:
         add_bias_(qkv, bias)
     rope_kv_write(

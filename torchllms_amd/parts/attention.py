@@ -82,7 +82,7 @@ class Attention(Mixer):
         self.position.to(self.wo.device)
 
     def linear_weights(self):
-        return [self.wqkv, self.wo]
+        return [(self.wqkv, "qkv"), self.wo]
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         n_kv_in_row = 0 if self.shares_kv else self.num_kv_heads

@@ -74,7 +74,9 @@ class Part:
             raise ValueError(f"{type(self).__name__} takes no tensors, got {sorted(tensors)}")
 
     def linear_weights(self):
-        """The matrices this part multiplies activations with (for kernel selection by measurement)."""
+        """The matrices this part multiplies activations with (for kernel selection by measurement):
+        tensors, or pairs ``(tensor, use)`` where ``use`` names the fused form of the product that
+        the part calls ("glu": ``ops.linear_glu``, "qkv": ``ops.qkv_rope_store``)."""
         return []
 
 

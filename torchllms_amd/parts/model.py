@@ -80,15 +80,16 @@ class Model:
         self.device = emb.device
 
     def linear_weights(self):
-        """All matrices of the model, grouped by shape."""
+        """All matrices of the model, grouped by (shape, use): see ``Part.linear_weights``."""
         groups = {}
         parts = [self.head]
         for b in self.blocks:
             parts += [b.mixer, b.feed_forward]
         for part in parts:
-            for w in part.linear_weights():
+            for item in part.linear_weights():
+                w, use = item if isinstance(item, tuple) else (item, "plain")
                 if w is not None:
-                    groups.setdefault(tuple(w.shape), []).append(w)
+                    groups.setdefault((tuple(w.shape), use), []).append(w)
         return groups
 
     # ------------------------------------------------------------------ cache
