@@ -476,7 +476,7 @@ def linear_choice(x: torch.Tensor, w: torch.Tensor, use: str = "plain"):
 _TUNE_FLUSH_BYTES = 512 << 20  # twice the 256 MB of last-level cache
 
 
-def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "plain", iters: int = 8) -> None:
+def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "plain", iters: int = 8, report=None) -> None:
     """Measure, for matrices of one shape and every row bucket, which bfloat16 kernel and launch is
     fastest on this GPU, and remember it.  ``weights``: the model's tensors of that shape; ``use``:
     one of ``LINEAR_USES``.  The plain product is what is timed; a candidate that cannot take the
@@ -486,7 +486,8 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
     product that needs two kernels is then charged what a second graph node costs, not what a
     second launch from Python costs), they rotate over the tensors, and the caches are flushed
     before every replay, so that the matrices come from HBM as they do in a step.  Shapes already
-    measured are left alone, so every engine of a process makes the same choice."""
+    measured are left alone, so every engine of a process makes the same choice.  ``report``, if
+    given, is called with (row bucket, candidate, microseconds per product) for everything timed."""
     import gc
 
     weights = [w for w in weights if w.is_cuda and w.dtype == torch.bfloat16 and w.dim() == 2]
@@ -501,7 +502,9 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         return
     device = weights[0].device
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    flush = torch.empty(_TUNE_FLUSH_BYTES, dtype=torch.uint8, device=device)
+    # read, not written, before every replay: written lines would still be on their way to HBM
+    # while the products are timed
+    flush = torch.zeros(_TUNE_FLUSH_BYTES // 4, dtype=torch.int32, device=device)
 
     def clock(fn) -> float:
         for i in range(2):  # loads the kernel's code and lets it ask for its LDS before the recording
@@ -520,7 +523,7 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
                 gc.enable()
         best = float("inf")
         for _ in range(3):  # the least of three replays: a stall of the machine does not decide
-            flush.zero_()
+            flush.sum()
             start.record()
             graph.replay()
             stop.record()
@@ -528,9 +531,12 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
             best = min(best, start.elapsed_time(stop))
         return best
 
-    def cost(choice, fn) -> float:
+    def cost(bucket, choice, fn) -> float:
         tail = 0.0 if _fuses_tail(choice, use) else _TAIL_KERNEL_US * 1e-3 * iters
-        return clock(fn) + tail
+        t = clock(fn) + tail
+        if report is not None:
+            report(bucket, choice, t / iters * 1e3)
+        return t
 
     for bucket in ROW_BUCKETS:
         if (n, k, bucket, use) in _LINEAR_CHOICE:
@@ -541,7 +547,7 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
             y = torch.nn.functional.linear(x, w)
             return y if y.dtype == out_dtype else y.to(out_dtype)
 
-        best, best_time = None, cost(None, library)
+        best, best_time = None, cost(bucket, None, library)
         if bucket <= STREAM_MAX_ROWS:
             candidates = [("stream", waves) for waves in STREAM_WAVE_CHOICES]
         elif wide_supported(x, weights[0]):
@@ -549,7 +555,7 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         else:
             candidates = []
         for choice in candidates:
-            t = cost(choice, lambda w: _run_choice(choice, x, w, out_dtype))
+            t = cost(bucket, choice, lambda w: _run_choice(choice, x, w, out_dtype))
             if t < best_time:
                 best, best_time = choice, t
         _LINEAR_CHOICE[(n, k, bucket, use)] = best
