@@ -206,3 +206,34 @@ def test_sampling_counter_survives_preemption():
     for seed in (11, 22):
         steps = [s for sd, s in asked if sd == seed]
         assert steps == list(range(10))  # each draw asked for exactly once, in order
+
+
+def test_the_short_cut_for_decode_steps_plans_what_the_rules_plan():
+    """A step in which everybody decodes and nobody can join is planned without walking the rules;
+    whenever that happens the rules are asked too (they change nothing in that case) and must say
+    the same."""
+    rng = random.Random(3)
+    prompts = [[1] * rng.randint(1, 12) for _ in range(7)]
+    eng = FakeEngine(num_pages=40, page_size=4, max_seqs=3)
+    loop = GenerationLoop(eng, greedy, 3, 64, 256)
+    sched = loop.scheduler
+    rules, schedule = sched._schedule, sched.schedule
+    state = {"by_rules": 0, "short_cuts": 0}
+
+    def counted_rules():
+        state["by_rules"] += 1
+        return rules()
+
+    def checked_schedule():
+        before = state["by_rules"]
+        plan = schedule()
+        if state["by_rules"] == before:  # the short cut answered
+            state["short_cuts"] += 1
+            again = rules()
+            assert [(e.request.rid, e.tokens, e.samples) for e in again.entries] == [(e.request.rid, e.tokens, e.samples) for e in plan.entries]
+            assert not again.preempted
+        return plan
+
+    sched._schedule, sched.schedule = counted_rules, checked_schedule
+    reqs = loop.run(prompts, [SamplingParams(max_new_tokens=rng.randint(2, 15)) for _ in prompts])
+    assert all(r.finished for r in reqs) and state["short_cuts"] > 10 and state["by_rules"] >= 3

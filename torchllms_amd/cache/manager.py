@@ -179,6 +179,8 @@ class CacheManager:
             n = num_pages[g.name] if isinstance(num_pages, dict) else num_pages
             self.pools.append(PagePool(int(n)))
         self._requests: Dict[Hashable, RequestEntry] = {}
+        #: without a window no page is given back before its request ends
+        self._windowed = any(g.window > 0 for g in self.groups)
         #: counts admissions, releases and truncations: a plan made at one epoch describes the same
         #: requests, slots and pages at the same epoch only
         self.epoch = 0
@@ -248,6 +250,10 @@ class CacheManager:
                 t[:, slot].zero_()
         return slot
 
+    def get(self, rid: Hashable) -> Optional[RequestEntry]:
+        """The live request's entry, or None."""
+        return self._requests.get(rid)
+
     def entry(self, rid: Hashable) -> RequestEntry:
         try:
             return self._requests[rid]
@@ -309,6 +315,11 @@ class CacheManager:
         if n_new < 0:
             raise ValueError("n_new must be >= 0")
         e = self.entry(rid)
+        total = e.num_tokens + n_new
+        if all(total <= len(bt) * self.page_size for bt in e.block_tables):
+            # the pages it holds have room (most decode steps): nothing to take
+            e.reserved_tokens = max(e.reserved_tokens, total)
+            return e.num_tokens
         short = self.pages_short(rid, n_new)
         if any(short.values()):
             raise OutOfPages(
@@ -331,6 +342,8 @@ class CacheManager:
             if e.num_tokens + n_new > len(bt) * self.page_size:
                 raise RuntimeError(f"request {rid!r}: advancing past the pages it holds (extend first)")
         e.num_tokens += n_new
+        if not self._windowed:
+            return
         for gi, pool in enumerate(self.pools):
             first = min(self._first_needed_block(gi, e.num_tokens), len(e.block_tables[gi]))
             bt = e.block_tables[gi]

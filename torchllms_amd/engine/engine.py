@@ -165,26 +165,30 @@ class Engine:
         if epoch != cache.epoch:
             return None
         n = len(entries)
-        tokens = np.empty(n, dtype=np.int32)
+        held = prev.kv_lens.tolist()
+        page = self.page_size
+        get = cache.get
+        toks = []
         need = 0
-        for i, e in enumerate(entries):
-            if e.rid != rids[i] or len(e.tokens) != 1 or tuple(e.want) != wants[i]:
+        for e, rid, want, have in zip(entries, rids, wants, held):
+            if e.rid != rid or len(e.tokens) != 1 or list(e.want) != want:
                 return None
-            tok = e.tokens[0]
-            if not 0 <= tok < self.vocab_size:
+            live = get(rid)
+            if live is None or live.num_tokens != have:
                 return None
-            if not cache.has(e.rid) or cache.num_tokens(e.rid) != int(prev.kv_lens[i]) or int(prev.kv_lens[i]) + 1 > self.max_model_len:
-                return None
-            tokens[i] = tok
-            need += cache.new_pages_needed(e.rid, 1)
+            toks.append(e.tokens[0])
+            if have % page == 0:  # the new token opens a page
+                need += cache.new_pages_needed(rid, 1)
+        if min(toks) < 0 or max(toks) >= self.vocab_size or max(held) + 1 > self.max_model_len:
+            return None
         if any(need > pool.free_count for pool in cache.pools):
             return None
-        page = self.page_size
+        tokens = np.asarray(toks, dtype=np.int32)
         positions = prev.kv_lens.copy()  # the new token's position = tokens held so far
-        for e in entries:
-            cache.extend(e.rid, 1)
+        fresh = (positions % page) == 0  # rows whose new token opens a page; the others have room
+        for i in np.nonzero(fresh)[0]:
+            cache.extend(rids[i], 1)
         tables, slots = [], []
-        fresh = (positions % page) == 0  # rows whose new token opens a page
         for g in range(len(cache.groups)):
             bt = prev.block_tables[g]
             sm = prev.slot_mappings[g] + 1
@@ -221,7 +225,7 @@ class Engine:
         layout = self._plan_general(entries)
         if layout.n_decode == layout.n_seqs:
             self._last_decode = (
-                tuple(e.rid for e in entries), tuple(tuple(e.want) for e in entries), layout, self.cache.epoch
+                tuple(e.rid for e in entries), tuple(list(e.want) for e in entries), layout, self.cache.epoch
             )
         return layout
 

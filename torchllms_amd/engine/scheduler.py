@@ -51,6 +51,19 @@ class Request:
         return self.prompt + self.output
 
     @property
+    def last_token(self) -> int:
+        return self.output[-1] if self.output else self.prompt[-1]
+
+    def token_slice(self, lo: int, hi: int) -> List[int]:
+        """``tokens[lo:hi]`` without putting prompt and output together first."""
+        n = len(self.prompt)
+        if hi <= n:
+            return self.prompt[lo:hi]
+        if lo >= n:
+            return self.output[lo - n : hi - n]
+        return self.prompt[lo:] + self.output[: hi - n]
+
+    @property
     def remaining(self) -> int:
         """Tokens not yet in the cache (the last generated token included)."""
         return len(self.prompt) + len(self.output) - self.num_computed
@@ -149,6 +162,20 @@ class Scheduler:
 
     def schedule(self) -> StepPlan:
         """Decide the next step.  Pages are counted here and taken by ``Engine.step``."""
+        # The common step of a running batch: everybody decodes, nobody can join, and even if
+        # every request opened a page the pools would hold them.  The rules of ``_schedule`` give
+        # exactly this plan then, after many more questions.
+        running = self.running
+        if (
+            running and len(running) <= self.max_num_batched_tokens
+            and all(pool.free_count >= len(running) for pool in self.cache.pools)
+            and (not self.waiting or len(running) >= self.max_num_seqs or self.cache.free_slots == 0)
+            and all(len(r.prompt) + len(r.output) - r.num_computed == 1 for r in running)
+        ):
+            return StepPlan(entries=[ScheduledEntry(r, [r.last_token], True) for r in running])
+        return self._schedule()
+
+    def _schedule(self) -> StepPlan:
         plan = StepPlan()
         budget = self.max_num_batched_tokens
         free = [pool.free_count for pool in self.cache.pools]
@@ -165,7 +192,7 @@ class Scheduler:
         i = 0
         while i < len(decoding) and budget > 0:
             req = decoding[i]
-            if req not in self.running:  # preempted a moment ago
+            if req.state != RUNNING:  # preempted a moment ago
                 i += 1
                 continue
             pages = self._pages_for(req, 1)
@@ -181,17 +208,18 @@ class Scheduler:
                     free[g] = self.cache.pools[g].free_count - counted
                 if victim is req:
                     break
-            if req in self.running:
-                plan.entries.append(ScheduledEntry(req, [req.tokens[-1]], samples=True))
+            if req.state == RUNNING:
+                plan.entries.append(ScheduledEntry(req, [req.last_token], samples=True))
                 take(pages)
                 budget -= 1
             i += 1
 
         # (2) prompts already started, in order of admission
+        planned = {id(e.request) for e in plan.entries}
         for req in self.running:
             if budget <= 0:
                 break
-            if req.remaining <= 1 or any(e.request is req for e in plan.entries):
+            if req.remaining <= 1 or id(req) in planned:
                 continue
             n = min(req.remaining, budget, self.prefill_chunk)
             while n > 0 and not fits(self._pages_for(req, n)):
@@ -234,7 +262,7 @@ class Scheduler:
         return max(min(n - 1, room), 0)
 
     def _add_portion(self, plan: StepPlan, req: Request, n: int) -> None:
-        toks = req.tokens[req.num_computed : req.num_computed + n]
+        toks = req.token_slice(req.num_computed, req.num_computed + n)
         plan.entries.append(ScheduledEntry(req, toks, samples=(n == req.remaining)))
 
     # ------------------------------------------------------------------ after the step
