@@ -832,6 +832,71 @@ def test_gemm_wide_takes_strided_rows_and_says_its_limits():
         _ops().gemm_wide(x, w, torch.float32, 1, 1, 4)
 
 
+@pytest.mark.parametrize("m, n, k, splits", [(64, 4096, 1024, 4), (20, 2048, 512, 8), (33, 72, 384, 2), (17, 8192, 256, 3)])
+@pytest.mark.parametrize("weight_dtype", [torch.bfloat16, torch.float32])
+def test_rmsnorm_adds_up_a_split_product_as_the_reduce_kernel_would(m, n, k, splits, weight_dtype):
+    """A product left as the sums of its splits, taken as the delta of the norm: bit for bit what
+    the product's own second kernel followed by the norm gives (same order of additions, same
+    roundings), for the whole batch, with the sum returned, and for gathered rows."""
+    ops = _ops()
+    torch.manual_seed(5)
+    x = torch.randn(m, k).bfloat16().to(DEV)
+    w = (torch.randn(n, k) * 0.05).bfloat16().to(DEV)
+    h = torch.randn(m, n).bfloat16().to(DEV)
+    g = (1 + 0.1 * torch.randn(n)).to(weight_dtype).to(DEV)
+    whole = ops.gemm_wide(x, w, torch.bfloat16, 1, splits, 3)
+    left = ops.gemm_wide(x, w, torch.bfloat16, 1, splits, 3, leave_split=True)
+    assert isinstance(left, ops.SplitSums) and left.shape == (m, n) and left.partial.shape[0] == min(splits, k // 128)
+    assert torch.equal(left.resolve(), whole)
+    want_h, want_y = ops.rmsnorm(h, g, 1e-5, delta=whole, return_sum=True)
+    got_h, got_y = ops.rmsnorm(h, g, 1e-5, delta=left, return_sum=True)
+    assert torch.equal(got_h, want_h) and torch.equal(got_y, want_y)
+    rows = _i32([m - 1, 0, 3, 3])
+    assert torch.equal(ops.rmsnorm(h, g, 1e-5, delta=left, rows=rows), ops.rmsnorm(h, g, 1e-5, delta=whole, rows=rows))
+    # against the formula
+    ref = plain.rms_norm((h.float() + whole.float()).bfloat16().float().cpu(), g.float().cpu(), 1e-5)
+    torch.testing.assert_close(got_y.float().cpu(), ref, rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_rmsnorm_adds_the_splits_first_where_its_kernel_does_not_take_the_width():
+    ops = _ops()
+    torch.manual_seed(6)
+    x = torch.randn(24, 256).bfloat16().to(DEV)
+    w = (torch.randn(100, 256) * 0.05).bfloat16().to(DEV)  # 100 columns: no multiple of 8
+    h = torch.randn(24, 100).bfloat16().to(DEV)
+    g = torch.ones(100, dtype=torch.bfloat16, device=DEV)
+    left = ops.gemm_wide(x, w, torch.bfloat16, 1, 2, 2, leave_split=True)
+    want = ops.rmsnorm(h, g, 1e-6, delta=ops.gemm_wide(x, w, torch.bfloat16, 1, 2, 2))
+    assert torch.equal(ops.rmsnorm(h, g, 1e-6, delta=left), want)
+
+
+def test_linear_to_sum_leaves_a_product_split_only_where_it_was_tuned_to_be_split():
+    ops = _ops()
+    torch.manual_seed(7)
+    w = (torch.randn(96, 512, device=DEV) * 0.05).bfloat16()
+    x = torch.randn(40, 512, device=DEV).bfloat16()
+    want = (x.float() @ w.float().T).cpu()
+    key = (96, 512, 64, "sum")
+    saved = ops._LINEAR_CHOICE.get(key, "absent")
+    try:
+        for choice, split in ((None, False), (("wide", 1, 1, 3), False), (("wide", 1, 4, 3), True), (("wide", 2, 2, 2), True)):
+            ops._LINEAR_CHOICE[key] = choice
+            got = ops.linear_to_sum(x, w)
+            assert isinstance(got, ops.SplitSums) == split, choice
+            if split:
+                got = got.resolve()
+            torch.testing.assert_close(got.float().cpu(), want, rtol=2 ** -7, atol=0.05)
+        small = ops.linear_to_sum(x[:3], w)  # few rows: the streaming kernel, which adds its splits inside the block
+        assert isinstance(small, torch.Tensor)
+        f32 = ops.linear_to_sum(x.float(), w.float())
+        assert isinstance(f32, torch.Tensor) and f32.dtype == torch.float32
+    finally:
+        if saved == "absent":
+            ops._LINEAR_CHOICE.pop(key, None)
+        else:
+            ops._LINEAR_CHOICE[key] = saved
+
+
 def test_tune_linear_measures_the_wide_kernel_from_17_rows_on():
     ops = _ops()
     torch.manual_seed(0)

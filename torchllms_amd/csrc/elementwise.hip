@@ -202,6 +202,92 @@ TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, 
   return tl_check_launch("rmsnorm");
 }
 
+// The same for a delta that arrives as the 32-bit partial sums of a matrix product split along K
+// (partial[s][row][i], s = 0 .. splits - 1): they are added in the order of the splits and rounded
+// to bfloat16, as the kernel that would otherwise finish the product does, and then the row goes the
+// way of rmsnorm_vec_kernel.  One launch instead of two.
+template <typename WT>
+__global__ void __launch_bounds__(kNormThreads)
+rmsnorm_split_kernel(const bf16_t* __restrict__ x, const float* __restrict__ partial, int splits, size_t split_stride,
+                     const int32_t* __restrict__ rows, const WT* __restrict__ weight, bf16_t* __restrict__ h_out,
+                     bf16_t* __restrict__ y, int hidden, float eps) {
+  constexpr int VEC = 8;
+  constexpr int MAXV = 4;
+  __shared__ float scratch[kNormThreads / kWave];
+  const int r = blockIdx.x;
+  const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+  const int n_vec = hidden / VEC;
+  const uint4* xr = reinterpret_cast<const uint4*>(x + s * hidden);
+  const float4* pr = reinterpret_cast<const float4*>(partial + s * hidden);
+  union V { uint4 u; bf16_t e[VEC]; };
+  float v[MAXV][VEC];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < MAXV; ++it) {
+    const int c = threadIdx.x + it * kNormThreads;
+    if (c < n_vec) {
+      V xin;
+      xin.u = xr[c];
+      float d[VEC] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int k = 0; k < splits; ++k) {
+        const float4 lo = pr[k * (split_stride / 4) + 2 * c], hi = pr[k * (split_stride / 4) + 2 * c + 1];
+        d[0] += lo.x; d[1] += lo.y; d[2] += lo.z; d[3] += lo.w;
+        d[4] += hi.x; d[5] += hi.y; d[6] += hi.z; d[7] += hi.w;
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float f = to_f32(from_f32<bf16_t>(to_f32(xin.e[e]) + to_f32(from_f32<bf16_t>(d[e]))));
+        v[it][e] = f;
+        ss += f * f;
+      }
+    }
+  }
+  ss = block_sum<kNormThreads / kWave>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+  uint4* yr = reinterpret_cast<uint4*>(y + (size_t)r * hidden);
+  uint4* hr = h_out ? reinterpret_cast<uint4*>(h_out + (size_t)r * hidden) : nullptr;
+#pragma unroll
+  for (int it = 0; it < MAXV; ++it) {
+    const int c = threadIdx.x + it * kNormThreads;
+    if (c < n_vec) {
+      V out, hs;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        hs.e[e] = from_f32<bf16_t>(v[it][e]);
+        const float n = to_f32(from_f32<bf16_t>(v[it][e] * inv));
+        out.e[e] = from_f32<bf16_t>(n * to_f32(weight[c * VEC + e]));
+      }
+      yr[c] = out.u;
+      if (hr) hr[c] = hs.u;
+    }
+  }
+}
+
+// RMS norm of x + sum of the splits, bfloat16 x / h_out / y [.., hidden]; partial: 32-bit, split s of
+// row r at partial + s * split_stride + r * hidden (split_stride in elements, a multiple of 4).
+// hidden must be a multiple of 8 and at most 8 * 4 * 256.
+TL_EXPORT int tl_rmsnorm_split(const void* x, const float* partial, int splits, int64_t split_stride, const int32_t* rows,
+                               const void* weight, int weight_dtype, void* h_out, void* y, int n_rows, int hidden,
+                               float eps, hipStream_t stream) {
+  TL_REQUIRE(n_rows >= 0 && hidden > 0 && splits >= 1, "rmsnorm_split: bad sizes n_rows=%d hidden=%d splits=%d", n_rows, hidden, splits);
+  TL_REQUIRE(!(rows && h_out), "rmsnorm_split: h_out cannot be combined with a row gather");
+  if (hidden % 8 != 0 || hidden / 8 > kNormThreads * 4)
+    return tl_fail(TL_ERR_UNSUPPORTED, "rmsnorm_split: hidden=%d must be a multiple of 8 and at most %d", hidden, 8 * 4 * kNormThreads);
+  TL_REQUIRE(split_stride % 4 == 0 && ((uintptr_t)partial % 16) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
+                 (!h_out || (uintptr_t)h_out % 16 == 0),
+             "rmsnorm_split: tensors must start on 16-byte boundaries");
+  if (n_rows == 0) return TL_OK;
+  if (weight_dtype == TL_BF16)
+    rmsnorm_split_kernel<bf16_t><<<n_rows, kNormThreads, 0, stream>>>((const bf16_t*)x, partial, splits, (size_t)split_stride, rows,
+                                                                      (const bf16_t*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps);
+  else if (weight_dtype == TL_F32)
+    rmsnorm_split_kernel<float><<<n_rows, kNormThreads, 0, stream>>>((const bf16_t*)x, partial, splits, (size_t)split_stride, rows,
+                                                                     (const float*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps);
+  else
+    return tl_fail(TL_ERR_ARG, "rmsnorm_split: unsupported weight dtype %d", weight_dtype);
+  return tl_check_launch("rmsnorm_split");
+}
+
 // ----------------------------------------------------------------------------- rotary + KV write
 // qkv: [n_tokens, (Hq + 2 Hkv) * dh], each row = q heads | k heads | v heads.
 // For token t at position p: angle_i = float(p) * inv_freq[i], i < rotary_dim/2 (32-bit), and

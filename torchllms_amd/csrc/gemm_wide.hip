@@ -257,6 +257,7 @@ struct Launch {
   int M, N, K;
   int out_dtype;
   int splits;          // blocks along K
+  bool reduce;         // false: the splits' sums stay in `partial` (always written then) and C is not touched
   bool gated;
   const QkvArgs* qkv;  // non-null: the split product ends in the query/key/value epilogue
   hipStream_t stream;
@@ -275,13 +276,15 @@ int launch_kernel(const Launch& l) {
   const int steps_total = l.K / kStepK;
   const int steps_per_split = (steps_total + l.splits - 1) / l.splits;
   const int used = (steps_total + steps_per_split - 1) / steps_per_split;  // no split is empty
-  const bool split = used > 1 || l.qkv != nullptr;  // the query/key/value epilogue lives in the second kernel
+  // the query/key/value epilogue lives in the second kernel; a caller that adds the splits itself gets
+  // them even when there is only one
+  const bool split = used > 1 || l.qkv != nullptr || !l.reduce;
   const int block_cols = GATED ? S::kBlockRows / 2 : S::kBlockRows;
   const dim3 grid((l.N + block_cols - 1) / block_cols, used);
   gemm_wide_kernel<MC, NCW, STAGES, OutT, GATED><<<grid, kWaves * kWave, S::kLdsBytes, l.stream>>>(
       l.A, l.lda, l.W, l.ldw, (OutT*)l.C, l.ldc, split ? l.partial : nullptr, l.M, l.N, l.K, steps_per_split);
   int rc = tl_check_launch("gemm_wide");
-  if (rc != TL_OK || !split) return rc;
+  if (rc != TL_OK || !split || !l.reduce) return rc;
   if (l.qkv != nullptr) {
     const size_t quads = (size_t)l.M * (l.N / 4);
     gemm_wide_reduce_qkv_kernel<<<(unsigned)((quads + 255) / 256), 256, 0, l.stream>>>(l.partial, (bf16_t*)l.C, l.ldc, l.M,
@@ -321,7 +324,7 @@ int run(Launch l, int strips_per_wave, int stages) {
   TL_REQUIRE(strips_per_wave == 1 || strips_per_wave == 2, "gemm_wide: strips_per_wave must be 1 or 2");
   TL_REQUIRE(l.splits >= 1 && l.splits <= 64, "gemm_wide: k_splits must be 1..64");
   TL_REQUIRE(stages == 2 || stages == 3, "gemm_wide: stages must be 2 or 3");
-  const bool needs_partial = l.splits > 1 || l.qkv != nullptr;
+  const bool needs_partial = l.splits > 1 || l.qkv != nullptr || !l.reduce;
   TL_REQUIRE(!needs_partial || (l.partial != nullptr && ((uintptr_t)l.partial % 16) == 0),
              "gemm_wide: a split product needs the 16-byte aligned partial buffer");
   if (l.M == 0) return TL_OK;
@@ -336,10 +339,36 @@ int run(Launch l, int strips_per_wave, int stages) {
 // of 128.  strips_per_wave: 1 or 2 (a block owns 64 or 128 columns).  k_splits >= 1: blocks along
 // K; with more than one, `partial` must hold k_splits * M * N floats.  stages: 2 or 3 buffers of LDS
 // (a buffer is 4 KB for every 16 rows of A, 32 or 64 of them, plus 16 KB for every strip per wave).
+// reduce = 0: the second kernel is left out; `partial` then holds tl_gemm_wide_splits(K, k_splits)
+// slices [M, N] for the caller to add (in their order, for the same result), and C is not touched.
 TL_EXPORT int tl_gemm_wide(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
-                           int out_dtype, int strips_per_wave, int k_splits, int stages, void* partial, hipStream_t stream) {
-  Launch l{(const bf16_t*)A, lda, (const bf16_t*)W, ldw, C, ldc, (float*)partial, M, N, K, out_dtype, k_splits, false, nullptr, stream};
+                           int out_dtype, int strips_per_wave, int k_splits, int stages, int reduce, void* partial,
+                           hipStream_t stream) {
+  Launch l{(const bf16_t*)A, lda, (const bf16_t*)W, ldw, C, ldc, (float*)partial, M, N, K, out_dtype, k_splits, reduce != 0, false, nullptr, stream};
   return run(l, strips_per_wave, stages);
+}
+
+// How many splits a product over K with `k_splits` asked for really has (no split is empty).
+TL_EXPORT int tl_gemm_wide_splits(int K, int k_splits) {
+  if (K <= 0 || k_splits <= 0) return 0;
+  const int steps_total = K / kStepK;
+  const int steps_per_split = (steps_total + k_splits - 1) / k_splits;
+  return steps_per_split > 0 ? (steps_total + steps_per_split - 1) / steps_per_split : 0;
+}
+
+// C [M, N] (bfloat16 or 32-bit) = the sum of `splits` slices [M, N] of `partial`, added in their order.
+TL_EXPORT int tl_gemm_wide_reduce(const void* partial, void* C, int ldc, int M, int N, int splits, int out_dtype,
+                                  hipStream_t stream) {
+  TL_REQUIRE(M >= 0 && N > 0 && splits >= 1 && ldc >= N, "gemm_wide_reduce: bad sizes M=%d N=%d splits=%d", M, N, splits);
+  TL_REQUIRE(out_dtype == TL_BF16 || out_dtype == TL_F32, "gemm_wide_reduce: out_dtype must be 0 or 1");
+  if (M == 0) return TL_OK;
+  const size_t total = (size_t)M * N;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (out_dtype == TL_BF16)
+    gemm_wide_reduce_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const float*)partial, (bf16_t*)C, ldc, M, N, splits);
+  else
+    gemm_wide_reduce_kernel<float><<<blocks, 256, 0, stream>>>((const float*)partial, (float*)C, ldc, M, N, splits);
+  return tl_check_launch("gemm_wide_reduce");
 }
 
 // The gated pair of products: W [2 N, K] = gate rows | up rows; C [M, N] bfloat16 =
@@ -347,7 +376,7 @@ TL_EXPORT int tl_gemm_wide(const void* A, int lda, const void* W, int ldw, void*
 // would be if each were stored in bfloat16.  A block owns 32 or 64 columns (strips_per_wave 1 or 2).
 TL_EXPORT int tl_gemm_wide_glu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
                                int strips_per_wave, int stages, hipStream_t stream) {
-  Launch l{(const bf16_t*)A, lda, (const bf16_t*)W, ldw, C, ldc, nullptr, M, N, K, TL_BF16, 1, true, nullptr, stream};
+  Launch l{(const bf16_t*)A, lda, (const bf16_t*)W, ldw, C, ldc, nullptr, M, N, K, TL_BF16, 1, true, true, nullptr, stream};
   return run(l, strips_per_wave, stages);
 }
 
@@ -365,6 +394,6 @@ TL_EXPORT int tl_gemm_wide_qkv(const void* A, int lda, const void* W, int ldw, v
                           slot_mapping, page_size, C, ldc, &qa);
   if (rc != TL_OK) return rc;
   const int N = (n_q_heads + 2 * n_kv_heads) * head_dim;
-  Launch l{(const bf16_t*)A, lda, (const bf16_t*)W, ldw, C, ldc, (float*)partial, M, N, K, TL_BF16, k_splits, false, &qa, stream};
+  Launch l{(const bf16_t*)A, lda, (const bf16_t*)W, ldw, C, ldc, (float*)partial, M, N, K, TL_BF16, k_splits, true, false, &qa, stream};
   return run(l, strips_per_wave, stages);
 }

@@ -7,7 +7,7 @@ an exception is raised.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_uint64, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_uint64, c_void_p
 from typing import Dict, Optional
 
 from . import build as _build
@@ -21,11 +21,13 @@ _P = c_void_p
 _I = c_int
 _F = c_float
 _U64 = c_uint64
+_I64 = c_int64
 
 # name -> argument types (every function returns int status)
 _CORE_SIGNATURES = {
     "tl_embed": [_P, _P, _P, _I, _I, _I, _P],
     "tl_rmsnorm": [_P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _I, _P],
+    "tl_rmsnorm_split": [_P, _P, _I, _I64, _P, _P, _I, _P, _P, _I, _I, _F, _P],
     "tl_rope_table": [_P, _P, _I, _I, _P, _P],
     "tl_rope_kv_write": [_P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _P],
     "tl_silu_mul": [_P, _P, _I, _I, _I, _P],
@@ -35,7 +37,9 @@ _CORE_SIGNATURES = {
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "tl_gemm_stream_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _P],
-    "tl_gemm_wide": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P],
+    "tl_gemm_wide": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P],
+    "tl_gemm_wide_splits": [_I, _I],
+    "tl_gemm_wide_reduce": [_P, _P, _I, _I, _I, _I, _I, _P],
     "tl_gemm_wide_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "tl_gemm_wide_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P],
     "tl_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P],

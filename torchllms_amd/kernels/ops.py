@@ -63,10 +63,17 @@ def rmsnorm(
     rows: Optional[torch.Tensor] = None,
     return_sum: bool = False,
 ):
-    """RMS norm of ``x (+ delta)`` row by row, optionally of the rows ``rows`` only.
+    """RMS norm of ``x (+ delta)`` row by row, optionally of the rows ``rows`` only.  ``delta`` may be
+    a ``SplitSums``: the kernel then adds the splits itself (where it takes the width, else they are
+    added first).
 
     Returns ``y`` or, with ``return_sum``, ``(x + delta, y)``.
     """
+    if isinstance(delta, SplitSums):
+        hidden = x.shape[-1]
+        if x.dtype == torch.bfloat16 and hidden % 8 == 0 and hidden <= 8192 and delta.shape == tuple(x.shape):
+            return _rmsnorm_split(x, weight, eps, delta, rows, return_sum)
+        delta = delta.resolve()
     _gpu(x, weight, delta, rows)
     _i32(rows, "rows")
     if x.dim() != 2 or not x.is_contiguous():
@@ -85,6 +92,29 @@ def rmsnorm(
         core().tl_rmsnorm(
             x.data_ptr(), _ptr(delta), _ptr(rows), weight.data_ptr(), dtype_code(weight.dtype),
             _ptr(h_out), y.data_ptr(), n, hidden, float(eps), dtype_code(x.dtype), _stream(),
+        )
+    )
+    return (h_out, y) if return_sum else y
+
+
+def _rmsnorm_split(x, weight, eps, delta: "SplitSums", rows, return_sum):
+    _gpu(x, weight, rows)
+    _i32(rows, "rows")
+    if x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("rmsnorm input must be a contiguous [rows, hidden] tensor")
+    hidden = x.shape[1]
+    if weight.shape != (hidden,) or not weight.is_contiguous():
+        raise KernelError(f"rmsnorm weight must have shape ({hidden},), got {tuple(weight.shape)}")
+    if rows is not None and return_sum:
+        raise KernelError("rmsnorm cannot return the sum together with a row gather")
+    n = x.shape[0] if rows is None else rows.numel()
+    y = torch.empty((n, hidden), dtype=x.dtype, device=x.device)
+    h_out = torch.empty_like(x) if return_sum else None
+    part = delta.partial
+    check(
+        core().tl_rmsnorm_split(
+            x.data_ptr(), part.data_ptr(), part.shape[0], part.stride(0), _ptr(rows), weight.data_ptr(),
+            dtype_code(weight.dtype), _ptr(h_out), y.data_ptr(), n, hidden, float(eps), _stream(),
         )
     )
     return (h_out, y) if return_sum else y
@@ -265,20 +295,53 @@ def _wide_shapes(x: torch.Tensor, w: torch.Tensor, what: str) -> None:
         raise KernelError(f"{what}: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
 
 
+class SplitSums:
+    """A matrix product that was split along K and not yet added up: ``partial`` float32
+    [splits, rows, columns].  The product is the sum of the slices in their order, rounded to
+    ``dtype``; ``rmsnorm`` takes it as ``delta`` and adds the slices while it reads them, which
+    saves the kernel that would otherwise do nothing else."""
+
+    def __init__(self, partial: torch.Tensor, dtype: torch.dtype):
+        self.partial = partial
+        self.dtype = dtype
+
+    @property
+    def shape(self):
+        return tuple(self.partial.shape[1:])
+
+    def resolve(self) -> torch.Tensor:
+        splits, m, n = self.partial.shape
+        out = torch.empty((m, n), dtype=self.dtype, device=self.partial.device)
+        check(core().tl_gemm_wide_reduce(self.partial.data_ptr(), out.data_ptr(), out.stride(0), m, n, splits, dtype_code(self.dtype), _stream()))
+        return out
+
+
 def gemm_wide(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, strips_per_wave: int = 1,
-              k_splits: int = 1, stages: int = 3) -> torch.Tensor:
+              k_splits: int = 1, stages: int = 3, leave_split: bool = False):
     """``x @ w.T`` for at most 64 rows of bfloat16 ``x`` (K a multiple of 128) with the kernel whose
     blocks share their slice of ``x`` through LDS; ``k_splits`` > 1 cuts K over several blocks whose
-    32-bit partial sums a second kernel adds."""
+    32-bit partial sums a second kernel adds, or, with ``leave_split``, come back as ``SplitSums``."""
     _wide_shapes(x, w, "gemm_wide")
     m, k = x.shape
     n = w.shape[0]
+    if leave_split:
+        if n % 4:
+            raise KernelError("gemm_wide: split sums need a number of columns that is a multiple of 4")
+        used = core().tl_gemm_wide_splits(k, k_splits)
+        partial = torch.empty((max(used, 1), m, n), dtype=torch.float32, device=x.device)
+        check(
+            core().tl_gemm_wide(
+                x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), None, n, m, n, k,
+                dtype_code(out_dtype), strips_per_wave, k_splits, stages, 0, partial.data_ptr(), _stream(),
+            )
+        )
+        return SplitSums(partial, out_dtype)
     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
     partial = torch.empty((k_splits, m, n), dtype=torch.float32, device=x.device) if k_splits > 1 else None
     check(
         core().tl_gemm_wide(
             x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k,
-            dtype_code(out_dtype), strips_per_wave, k_splits, stages, _ptr(partial), _stream(),
+            dtype_code(out_dtype), strips_per_wave, k_splits, stages, 1, _ptr(partial), _stream(),
         )
     )
     return out
@@ -433,9 +496,11 @@ STREAM_WAVE_CHOICES = (0, 4)
 #: (strips per wave, splits of K, buffers) that ``tune_linear`` tries from 17 rows on: whole-K
 #: launches for matrices with many rows, splits of K for those with few
 WIDE_CHOICES = ((1, 1, 3), (2, 1, 3), (1, 4, 3), (1, 8, 3), (2, 8, 3))
-#: how a product is used: alone, or as the first half of ``linear_glu`` / ``qkv_rope_store``, whose
-#: second half (gate, rotation and cache write) some kernels take into themselves
-LINEAR_USES = ("plain", "glu", "qkv")
+#: how a product is used: alone; as the first half of ``linear_glu`` / ``qkv_rope_store``, whose
+#: second half (gate, rotation and cache write) some kernels take into themselves; or ("sum",
+#: ``linear_to_sum``) as a term of the residual sum, where the norm that follows adds up a split
+#: product for nothing
+LINEAR_USES = ("plain", "glu", "qkv", "sum")
 #: microseconds that a small kernel between large ones costs in a replayed decode step (measured);
 #: ``tune_linear`` charges it to a candidate that leaves the second half of a fused use to a kernel
 #: of its own
@@ -451,8 +516,8 @@ def _row_bucket(m: int) -> int:
 
 def _fuses_tail(choice, use: str) -> bool:
     """Whether the kernel of ``choice`` does the second half of ``use`` itself."""
-    if use == "plain" or choice is None:
-        return use == "plain"
+    if use in ("plain", "sum") or choice is None:
+        return use in ("plain", "sum")
     if choice[0] == "stream":
         return True
     return choice[2] == 1 if use == "glu" else choice[2] > 1  # the gate ends a whole product, the rotation a split one
@@ -555,19 +620,20 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         else:
             candidates = []
         for choice in candidates:
-            t = cost(bucket, choice, lambda w: _run_choice(choice, x, w, out_dtype))
+            t = cost(bucket, choice, lambda w: _run_choice(choice, x, w, out_dtype, leave_split=use == "sum"))
             if t < best_time:
                 best, best_time = choice, t
         _LINEAR_CHOICE[(n, k, bucket, use)] = best
 
 
-def _run_choice(choice, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+def _run_choice(choice, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, leave_split: bool = False):
     if choice is None:
         y = torch.nn.functional.linear(x, w)
         return y if y.dtype == out_dtype else y.to(out_dtype)
     if choice[0] == "stream":
         return gemm_stream(x, w, out_dtype, choice[1])
-    return gemm_wide(x, w, out_dtype, choice[1], choice[2], choice[3])
+    leave_split = leave_split and choice[2] > 1 and w.shape[0] % 4 == 0
+    return gemm_wide(x, w, out_dtype, choice[1], choice[2], choice[3], leave_split)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
@@ -581,6 +647,16 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     _gpu(x, w)
     out_dtype = out_dtype or x.dtype
     return _run_choice(linear_choice(x, w), x, w, out_dtype)
+
+
+def linear_to_sum(x: torch.Tensor, w: torch.Tensor):
+    """``x @ w.T`` for a result that is only ever added to the residual stream by ``rmsnorm(...,
+    delta=...)``: a tensor, or ``SplitSums`` when the product was split along K, which that
+    ``rmsnorm`` adds up while it reads them."""
+    if x.dtype == torch.float32:
+        return gemm_f32(x, w)
+    _gpu(x, w)
+    return _run_choice(linear_choice(x, w, "sum"), x, w, x.dtype, leave_split=True)
 
 
 def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:

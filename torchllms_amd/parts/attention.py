@@ -82,7 +82,7 @@ class Attention(Mixer):
         self.position.to(self.wo.device)
 
     def linear_weights(self):
-        return [(self.wqkv, "qkv"), self.wo]
+        return [(self.wqkv, "qkv"), (self.wo, "sum")]
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
         n_kv_in_row = 0 if self.shares_kv else self.num_kv_heads
@@ -118,4 +118,4 @@ class Attention(Mixer):
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
             ctx, g, self.window, self.softmax_scale,
         )
-        return ops.linear(attn, self.wo)
+        return ops.linear_to_sum(attn, self.wo)

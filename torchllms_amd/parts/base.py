@@ -81,7 +81,19 @@ class Part:
 
 
 class Norm(Part):
-    """y = norm(x).  ``forward_add`` fuses the residual sum that precedes the norm."""
+    """y = norm(x).  ``forward_add`` fuses the residual sum that precedes the norm.
+
+    A mixer or feed-forward whose last matrix product was split along K may hand its result on as
+    ``kernels.ops.SplitSums`` (the slices not yet added) instead of a tensor.  Whoever passes a delta
+    to a norm passes it through ``norm.delta(...)`` first: a norm whose kernel adds the slices while it
+    reads them sets ``takes_split_sums``; for every other norm they are added up there."""
+
+    takes_split_sums = False
+
+    def delta(self, delta):
+        if delta is not None and not isinstance(delta, torch.Tensor) and not self.takes_split_sums:
+            return delta.resolve()
+        return delta
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError

@@ -12,8 +12,8 @@ class PreNormBlock(Block):
     norm that reads it; the last one is handed on as ``delta``."""
 
     def forward(self, h, delta, ctx, cache):
-        h, y = self.mixer_norm.forward_add(h, delta)
+        h, y = self.mixer_norm.forward_add(h, self.mixer_norm.delta(delta))
         a = self.mixer.forward(y, ctx, cache)
-        h, y = self.ffn_norm.forward_add(h, a)
+        h, y = self.ffn_norm.forward_add(h, self.ffn_norm.delta(a))
         f = self.feed_forward.forward(y, ctx)
         return h, f

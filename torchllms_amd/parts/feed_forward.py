@@ -31,7 +31,7 @@ class SwiGLU(FeedForward):
         self.w2 = tensors["w2.weight"].contiguous()
 
     def linear_weights(self):
-        return [(self.w13, "glu"), self.w2]
+        return [(self.w13, "glu"), (self.w2, "sum")]
 
     def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        return ops.linear(ops.linear_glu(x, self.w13), self.w2)
+        return ops.linear_to_sum(ops.linear_glu(x, self.w13), self.w2)

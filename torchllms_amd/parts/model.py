@@ -112,5 +112,5 @@ class Model:
             h, delta = self.blocks[run.layer].forward(h, delta, ctx, view)
         if ctx.logit_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=h.device)
-        x = self.final_norm.forward_rows(h, delta, ctx.logit_rows)
+        x = self.final_norm.forward_rows(h, self.final_norm.delta(delta), ctx.logit_rows)
         return self.head.forward(x)
