@@ -525,6 +525,25 @@ def test_sample_temperature_matches_the_plain_rule(vocab):
         assert got[r] == plain.sample_with_exponentials(logits[r], 1.5, -torch.log(u), top_k=3)
 
 
+@pytest.mark.parametrize("vocab, rows", [(128256, 8), (128256, 64), (40000, 3), (16388, 5)])
+def test_sample_with_several_blocks_a_row_draws_what_one_block_draws(vocab, rows):
+    """Few rows of a large vocabulary are cut into pieces for blocks of their own (a vector of
+    zeros as top-k keeps the one-block kernel): the same tokens, greedy rows and ties included,
+    and the plain rule's token."""
+    ops = _ops()
+    assert ops.sample_chunks(rows, vocab) > 1 and ops.sample_chunks(512, vocab) == 1 and ops.sample_chunks(4, 5000) == 1
+    torch.manual_seed(3)
+    logits = torch.randn(rows, vocab) * 3
+    logits[1, vocab - 1] = logits[1, 9000] = 40.0  # a tie across pieces in a greedy row
+    temps = [0.7, 0.0, 1.3] + [0.9] * (rows - 3)
+    seeds, steps = list(range(11, 11 + rows)), list(range(rows))
+    many = _sample(logits, temps, seeds, steps)
+    one = _sample(logits, temps, seeds, steps, top_k=[0] * rows)
+    assert many.tolist() == one.tolist() and many[1] == 9000
+    u = ops.philox_uniform(seeds[2], steps[2], vocab, DEV).cpu()
+    assert many[2] == plain.sample_with_exponentials(logits[2], 1.3, -torch.log(u))
+
+
 def test_sample_mixed_rows_and_tiny_temperature():
     torch.manual_seed(0)
     logits = torch.randn(4, 200)

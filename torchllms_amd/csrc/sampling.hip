@@ -1,4 +1,6 @@
-// Next-token choice from 32-bit logits, one block per row.
+// Next-token choice from 32-bit logits, one block per row, or several blocks per row and a second
+// kernel that picks among their candidates (same result: maxima and the race's winner do not depend
+// on the order in which elements are visited).
 //   temperature == 0 : argmax(logits), the lowest index among equal maxima.
 //   temperature  > 0 : x = logits / max(temperature, 1e-5); optionally everything below the k-th
 //                      largest x is dropped (ties kept); the token is argmax_i exp(x_i - max x) / q_i
@@ -113,6 +115,38 @@ __device__ __forceinline__ Best row_best(const float* __restrict__ x, int vocab,
   return b;
 }
 
+// The race over indices [lo, hi) of a row scaled by 1 / tdiv, with maximum m of the scaled row:
+// each thread handles whole groups of four indices, so one generator call serves four draws; an
+// aligned row gives the four logits in one 16-byte load.  lo is a multiple of 4.
+__device__ __forceinline__ Best race(const float* __restrict__ x, int lo, int hi, float tdiv, float m, float pivot,
+                                     uint64_t seed, uint64_t step, int tid) {
+  constexpr int kNone = 0x7fffffff;
+  Best b = {-INFINITY, kNone};
+  const bool wide = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+  for (int i4 = lo + tid * 4; i4 < hi; i4 += kThreads * 4) {
+    uint32_t r[4];
+    philox4(seed, (uint32_t)i4 >> 2, step, r);
+    float xs[4];
+    if (wide && i4 + 3 < hi) {
+      const float4 v = *reinterpret_cast<const float4*>(x + i4);
+      xs[0] = v.x; xs[1] = v.y; xs[2] = v.z; xs[3] = v.w;
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) xs[u] = i4 + u < hi ? x[i4 + u] : -INFINITY;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i4 + u;
+      if (i >= hi) break;
+      const float xi = xs[u] / tdiv;
+      if (xi < pivot) continue;
+      const float q = -logf(uniform_open(r[u]));
+      b = better(b, Best{expf(xi - m) / q, i});
+    }
+  }
+  return b;
+}
+
 __global__ void __launch_bounds__(kThreads)
 sample_kernel(const float* __restrict__ logits, int row_stride, int vocab,
               const float* __restrict__ temperature, const int32_t* __restrict__ top_k,
@@ -175,33 +209,52 @@ sample_kernel(const float* __restrict__ logits, int row_stride, int vocab,
 
   const uint64_t seed = seeds[row];
   const uint64_t step = steps[row];
-  Best b = {-INFINITY, kNone};
-  // each thread handles whole groups of four indices, so one generator call serves four draws; an
-  // aligned row gives the four logits in one 16-byte load
-  const bool wide = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
-  for (int i4 = tid * 4; i4 < vocab; i4 += kThreads * 4) {
-    uint32_t r[4];
-    philox4(seed, (uint32_t)i4 >> 2, step, r);
-    float xs[4];
-    if (wide && i4 + 3 < vocab) {
-      const float4 v = *reinterpret_cast<const float4*>(x + i4);
-      xs[0] = v.x; xs[1] = v.y; xs[2] = v.z; xs[3] = v.w;
-    } else {
-#pragma unroll
-      for (int u = 0; u < 4; ++u) xs[u] = i4 + u < vocab ? x[i4 + u] : -INFINITY;
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int i = i4 + u;
-      if (i >= vocab) break;
-      const float xi = xs[u] / tdiv;
-      if (xi < pivot) continue;
-      const float q = -logf(uniform_open(r[u]));
-      b = better(b, Best{expf(xi - m) / q, i});
-    }
-  }
+  Best b = race(x, 0, vocab, tdiv, m, pivot, seed, step, tid);
   b = block_best(b, best_scratch);
   if (tid == 0) out[row] = b.idx;
+}
+
+// Several blocks per row (no top-k): block (chunk, row) finds the row's maximum by itself (the row
+// is read from L2 by all but the first to come) and runs the race, or the argmax, over its chunk of
+// `chunk_len` indices (a multiple of 4); candidates[row][chunk] receives its winner.
+__global__ void __launch_bounds__(kThreads)
+sample_chunks_kernel(const float* __restrict__ logits, int row_stride, int vocab, const float* __restrict__ temperature,
+                     const uint64_t* __restrict__ seeds, const uint64_t* __restrict__ steps, int chunk_len,
+                     Best* __restrict__ candidates) {
+  __shared__ Best best_scratch[kWaves];
+  const int row = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const float* x = logits + (size_t)row * row_stride;
+  const float temp = temperature[row];
+  const int tid = threadIdx.x;
+  const int lo = chunk * chunk_len;
+  const int hi = min(lo + chunk_len, vocab);
+  Best b;
+  if (temp == 0.f) {
+    b = row_best(x + lo, hi - lo, tid);  // (lo * 4 bytes is a multiple of 16: the chunk is aligned as the row is)
+    if (b.idx != 0x7fffffff) b.idx += lo;
+  } else {
+    const float tdiv = fmaxf(temp, 1e-5f);
+    const float m = block_best(row_best(x, vocab, tid), best_scratch).val / tdiv;
+    b = race(x, lo, hi, tdiv, m, -INFINITY, seeds[row], steps[row], tid);
+  }
+  b = block_best(b, best_scratch);
+  if (tid == 0) candidates[(size_t)row * gridDim.x + chunk] = b;
+}
+
+__global__ void __launch_bounds__(kWave)
+sample_pick_kernel(const Best* __restrict__ candidates, int chunks, int32_t* __restrict__ out) {
+  const int row = blockIdx.x;
+  Best b = {-INFINITY, 0x7fffffff};
+  for (int c = threadIdx.x; c < chunks; c += kWave) b = better(b, candidates[(size_t)row * chunks + c]);
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    Best o;
+    o.val = __shfl_xor(b.val, off, kWave);
+    o.idx = __shfl_xor(b.idx, off, kWave);
+    b = better(b, o);
+  }
+  if (threadIdx.x == 0) out[row] = b.idx;
 }
 
 __global__ void philox_uniform_kernel(uint64_t seed, uint64_t step, float* out, int n) {
@@ -221,6 +274,27 @@ TL_EXPORT int tl_sample(const float* logits, int row_stride, int n_rows, int voc
   if (n_rows == 0) return TL_OK;
   sample_kernel<<<n_rows, kThreads, 0, stream>>>(logits, row_stride, vocab, temperature, top_k, seeds, steps, out);
   return tl_check_launch("sample");
+}
+
+// The same choice without top-k, every row cut into `chunks` pieces that blocks of their own work
+// on: for few rows of a large vocabulary, where one block per row leaves most of the GPU idle.
+// candidates: workspace of n_rows * chunks * 8 bytes.  The tokens equal tl_sample's.
+TL_EXPORT int tl_sample_chunks(const float* logits, int row_stride, int n_rows, int vocab, const float* temperature,
+                               const uint64_t* seeds, const uint64_t* steps, int chunks, void* candidates,
+                               int32_t* out, hipStream_t stream) {
+  TL_REQUIRE(n_rows >= 0 && vocab > 0 && row_stride >= vocab, "sample_chunks: bad sizes");
+  TL_REQUIRE(temperature && seeds && steps && out && candidates, "sample_chunks: null argument");
+  TL_REQUIRE(chunks >= 1 && chunks <= 1024 && n_rows <= 65535, "sample_chunks: chunks must be 1..1024, rows at most 65535");
+  TL_REQUIRE(row_stride % 4 == 0 && ((uintptr_t)logits % 16) == 0, "sample_chunks: rows must start on 16-byte boundaries");
+  if (n_rows == 0) return TL_OK;
+  const int chunk_len = ((vocab + chunks - 1) / chunks + 3) / 4 * 4;
+  const int used = (vocab + chunk_len - 1) / chunk_len;  // no chunk is empty
+  sample_chunks_kernel<<<dim3(used, n_rows), kThreads, 0, stream>>>(logits, row_stride, vocab, temperature, seeds, steps,
+                                                                   chunk_len, (Best*)candidates);
+  int rc = tl_check_launch("sample_chunks");
+  if (rc != TL_OK) return rc;
+  sample_pick_kernel<<<n_rows, kWave, 0, stream>>>((const Best*)candidates, used, out);
+  return tl_check_launch("sample_pick");
 }
 
 // The uniforms the sampler uses for (seed, step), indices 0..n-1; for tests of the sampler.
