@@ -78,6 +78,14 @@ class Engine:
         self.vocab_size = self.spec.vocab_size
         self.max_model_len = int(max_model_len or self.spec.max_positions)
         self.page_size = page_size
+        if dtype == torch.bfloat16 and tune_kernels:
+            # which matrix-product kernel serves decode steps best is measured, not guessed; before
+            # the pool is sized, so that what the measurement borrows is free again for pages
+            from ..kernels import ops
+
+            for (shape, use), group in self.model.linear_weights().items():
+                ops.tune_linear(group, torch.float32 if group[0] is self.model.head.weight else torch.bfloat16, use)
+            torch.cuda.empty_cache()
         groups, states = group_layers(self.model.cache_needs())
         if num_pages is None:
             per_page = CacheManager.bytes_per_page(groups, page_size, dtype)
@@ -97,12 +105,6 @@ class Engine:
         # the last step's plan when every row of it brought one token: (request ids, wanted places,
         # layout); a decode step that follows it with the same requests is planned from it
         self._last_decode = None
-        if dtype == torch.bfloat16 and tune_kernels:
-            # which matrix-product kernel serves decode steps best is measured, not guessed
-            from ..kernels import ops
-
-            for (shape, use), group in self.model.linear_weights().items():
-                ops.tune_linear(group, torch.float32 if group[0] is self.model.head.weight else torch.bfloat16, use)
         # decode steps are replayed from HIP graphs when every mixer's launches are fixed by the
         # step's shape alone
         from .graphs import DecodeGraphs
