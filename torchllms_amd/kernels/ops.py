@@ -569,7 +569,7 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     # read, not written, before every replay: written lines would still be on their way to HBM
     # while the products are timed
-    flush = torch.zeros(_TUNE_FLUSH_BYTES // 4, dtype=torch.int32, device=device)
+    flush = torch.zeros(_TUNE_FLUSH_BYTES // 4, dtype=torch.float32, device=device)  # (summed without a conversion pass)
 
     def clock(fn) -> float:
         for i in range(2):  # loads the kernel's code and lets it ask for its LDS before the recording
