@@ -29,8 +29,6 @@ namespace {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 4;
 constexpr int kStepK = 128;            // k per step: 16 pieces of 8 elements
