@@ -1,0 +1,60 @@
+"""Host-side decisions about kernel launches (CPU): key splits of the decode attention, pieces of
+a sampled row, and which matrix-product kernel a tuned table sends a product to."""
+
+import torch
+
+from torchllms_amd.kernels import ops
+
+
+def test_decode_splits_cover_the_range_with_about_512_blocks():
+    for n_tokens in (1, 2, 3, 8, 17, 64, 200):
+        for n_kv_heads in (1, 2, 8):
+            for longest in (1, 15, 256, 1000, 8192, 70000, 131072):
+                for uneven in (False, True):
+                    split, n_splits = ops.plan_decode_splits(n_tokens, n_kv_heads, longest, uneven=uneven)
+                    assert split % 64 == 0 and split >= 256
+                    assert n_splits >= 1 and (n_splits - 1) * split < max(longest, 1) <= n_splits * split
+                    if uneven:
+                        assert split <= 1024
+                    elif n_splits > 1:
+                        # no more blocks than asked for, unless the shortest split allowed is reached
+                        assert split == 256 or n_tokens * n_kv_heads * n_splits <= 512 + n_tokens * n_kv_heads
+
+
+def test_a_sampled_row_is_cut_only_when_rows_are_few_and_long():
+    assert ops.sample_chunks(1, 128256) == 15 and ops.sample_chunks(8, 128256) == 15
+    assert ops.sample_chunks(64, 128256) == 4 and ops.sample_chunks(256, 128256) == 1
+    assert ops.sample_chunks(1, 8191) == 1 and ops.sample_chunks(1, 32000) == 3 and ops.sample_chunks(0, 128256) == 15
+
+
+def test_the_tuned_table_decides_per_shape_rows_and_use():
+    w = torch.zeros(96, 256, dtype=torch.bfloat16)
+    x = torch.zeros(40, 256, dtype=torch.bfloat16)
+    keys = [(96, 256, b, use) for b in (8, 64) for use in ops.LINEAR_USES]
+    saved = {k: ops._LINEAR_CHOICE[k] for k in keys if k in ops._LINEAR_CHOICE}
+    try:
+        for k in keys:
+            ops._LINEAR_CHOICE.pop(k, None)
+        assert ops.linear_choice(x, w) is None  # 40 rows, never measured: the library
+        assert ops.linear_choice(x[:8], w) == ("stream", 0)  # 8 rows, never measured: the size rule
+        ops._LINEAR_CHOICE[(96, 256, 64, "plain")] = ("wide", 1, 2, 3)
+        ops._LINEAR_CHOICE[(96, 256, 64, "glu")] = ("wide", 2, 1, 3)
+        ops._LINEAR_CHOICE[(96, 256, 8, "plain")] = None
+        assert ops.linear_choice(x, w) == ("wide", 1, 2, 3) and ops.linear_choice(x, w, "glu") == ("wide", 2, 1, 3)
+        assert ops.linear_choice(x, w, "qkv") is None and ops.linear_choice(x[:8], w) is None
+        assert ops.linear_choice(x[:33], w) == ("wide", 1, 2, 3)  # 33 to 64 rows share a bucket
+        assert ops.linear_choice(torch.zeros(65, 256, dtype=torch.bfloat16), w) is None  # too many rows
+        assert ops.linear_choice(torch.zeros(40, 192, dtype=torch.bfloat16), torch.zeros(96, 192, dtype=torch.bfloat16)) is None  # K % 128
+        assert ops.linear_choice(x.float(), w.float()) is None
+    finally:
+        for k in keys:
+            ops._LINEAR_CHOICE.pop(k, None)
+        ops._LINEAR_CHOICE.update(saved)
+
+
+def test_which_candidates_are_charged_a_kernel_of_their_own_for_the_second_half():
+    stream, whole, split = ("stream", 4), ("wide", 2, 1, 3), ("wide", 1, 4, 3)
+    for choice in (None, stream, whole, split):
+        assert ops._fuses_tail(choice, "plain") and ops._fuses_tail(choice, "sum")
+    assert [ops._fuses_tail(c, "glu") for c in (None, stream, whole, split)] == [False, True, True, False]
+    assert [ops._fuses_tail(c, "qkv") for c in (None, stream, whole, split)] == [False, True, False, True]
