@@ -189,7 +189,8 @@ def main(argv=None) -> int:
     main_r = results[args.batch]
     achieved = main_r["bytes"] / main_r["sec"] / 1e9
     line = {
-        "metric": "decode tok/s at batch 8, Llama-3.1-8B shape (plus batch 1/64 and prefill tok/s at 2048 tokens)",
+        "metric": f"decode tok/s at batch {args.batch}, Llama-3.1-8B shape (plus batch {'/'.join(str(b) for b in batches[1:]) or 'none'}"
+                  f" and prefill tok/s at {args.prefill_tokens} tokens)",
         "value": round(main_r["tps"], 2),
         "unit": "tokens/s",
         "n_gpus": 1,

@@ -767,12 +767,15 @@ def test_tune_linear_remembers_a_choice_for_every_row_bucket():
 @pytest.mark.parametrize(
     "m, n, k",
     [(64, 4096, 4096), (32, 6144, 4096), (17, 200, 128), (64, 4100, 384), (33, 72, 2048), (48, 1000, 1024), (5, 64, 256),
-     (64, 128, 14336), (49, 130, 640)],
+     (64, 128, 14336), (49, 130, 640), (128, 4096, 4096), (65, 200, 384), (100, 1000, 1024), (127, 72, 2048)],
 )
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_wide(m, n, k, out_dtype):
-    """Both row tiles (32 and 64), N that is no multiple of a block's columns, one step of K and
-    many, every block shape, splits of K that divide the steps and that do not, both buffer counts."""
+    """All row tiles (32, 64 and 128), N that is no multiple of a block's columns, one step of K and
+    many, every block shape, splits of K that divide the steps and that do not, both buffer counts
+    (three buffers of the largest tile with two strips do not fit LDS and are refused)."""
+    from torchllms_amd.kernels.lib import KernelError
+
     torch.manual_seed(0)
     x = torch.randn(m, k).bfloat16()
     w = (torch.randn(n, k) * 0.05).bfloat16()
@@ -781,11 +784,15 @@ def test_gemm_wide(m, n, k, out_dtype):
     for strips in (1, 2):
         for splits in (1, 2, 3, 8):
             for stages in (2, 3):
+                if not _ops().wide_fits(m, strips, stages):
+                    with pytest.raises(KernelError, match="do not fit into LDS"):
+                        _ops().gemm_wide(x.to(DEV), w.to(DEV), out_dtype, strips, splits, stages)
+                    continue
                 got = _ops().gemm_wide(x.to(DEV), w.to(DEV), out_dtype, strips, splits, stages).float().cpu()
                 assert (got.double() - want).abs().max().item() <= tol, f"strips={strips} splits={splits} stages={stages}"
 
 
-@pytest.mark.parametrize("m, f, k", [(64, 14336, 4096), (32, 1000, 256), (17, 40, 128), (50, 72, 1152)])
+@pytest.mark.parametrize("m, f, k", [(64, 14336, 4096), (32, 1000, 256), (17, 40, 128), (50, 72, 1152), (128, 4096, 2048), (77, 200, 384)])
 def test_gemm_wide_glu_equals_the_product_followed_by_the_gate(m, f, k):
     """The same roundings as the two kernels it replaces (see the streaming kernel's test)."""
     torch.manual_seed(1)
@@ -794,6 +801,8 @@ def test_gemm_wide_glu_equals_the_product_followed_by_the_gate(m, f, k):
     ref = torch.nn.functional.silu(x.float() @ w[:f].float().T) * (x.float() @ w[f:].float().T)
     for strips in (1, 2):
         for stages in (2, 3):
+            if not _ops().wide_fits(m, strips, stages):
+                continue
             want = _ops().silu_mul(_ops().gemm_wide(x, w, torch.bfloat16, strips, 1, stages))
             got = _ops().gemm_wide_glu(x, w, strips, stages)
             torch.testing.assert_close(got.float(), want.float(), rtol=2 ** -6, atol=2 ** -8 * want.float().abs().max().item(), msg=f"strips={strips}")
@@ -802,7 +811,8 @@ def test_gemm_wide_glu_equals_the_product_followed_by_the_gate(m, f, k):
 
 
 @pytest.mark.parametrize("m, hq, hkv, dh, rot, page, k", [(64, 32, 8, 128, 128, 16, 4096), (32, 4, 4, 64, 64, 16, 256),
-                                                           (23, 6, 3, 48, 24, 4, 384), (40, 5, 1, 20, 0, 8, 128)])
+                                                           (23, 6, 3, 48, 24, 4, 384), (40, 5, 1, 20, 0, 8, 128),
+                                                           (128, 8, 2, 64, 64, 16, 1024), (90, 6, 3, 48, 24, 4, 384)])
 @pytest.mark.parametrize("with_pages", [True, False])
 def test_gemm_wide_qkv_equals_product_then_rotary_kernel(m, hq, hkv, dh, rot, page, k, with_pages):
     """The split product whose second kernel rotates and scatters, against product and rotary
@@ -814,7 +824,7 @@ def test_gemm_wide_qkv_equals_product_then_rotary_kernel(m, hq, hkv, dh, rot, pa
     pos = torch.randint(0, 9000, (m,))
     inv_freq = plain.rope_inverse_frequencies(rot, 500000.0, None).to(DEV) if rot else None
     table = _ops().rope_table(_i32(pos.tolist()), inv_freq) if rot else None
-    n_pages = 80
+    n_pages = 160
     slots = torch.randperm(n_pages * page)[:m].tolist()
     slots[1] = -1
     sm = _i32(slots) if with_pages else None
@@ -843,8 +853,8 @@ def test_gemm_wide_takes_strided_rows_and_says_its_limits():
     w = torch.randn(70, 256).bfloat16().to(DEV)
     got = _ops().gemm_wide(x, w, torch.float32, 2, 2).cpu()
     torch.testing.assert_close(got, (x.float() @ w.float().T).cpu(), rtol=1e-4, atol=1e-3)
-    with pytest.raises(KernelError, match="exceeds 64"):
-        _ops().gemm_wide(torch.zeros(65, 256, dtype=torch.bfloat16, device=DEV), w)
+    with pytest.raises(KernelError, match="exceeds 128"):
+        _ops().gemm_wide(torch.zeros(129, 256, dtype=torch.bfloat16, device=DEV), w)
     with pytest.raises(KernelError, match="multiple of 128"):
         _ops().gemm_wide(torch.zeros(20, 64, dtype=torch.bfloat16, device=DEV), w[:, :64].contiguous())
     with pytest.raises(KernelError, match="stages"):

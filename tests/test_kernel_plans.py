@@ -30,7 +30,7 @@ def test_a_sampled_row_is_cut_only_when_rows_are_few_and_long():
 def test_the_tuned_table_decides_per_shape_rows_and_use():
     w = torch.zeros(96, 256, dtype=torch.bfloat16)
     x = torch.zeros(40, 256, dtype=torch.bfloat16)
-    keys = [(96, 256, b, use) for b in (8, 64) for use in ops.LINEAR_USES]
+    keys = [(96, 256, b, use) for b in (8, 64, 128) for use in ops.LINEAR_USES]
     saved = {k: ops._LINEAR_CHOICE[k] for k in keys if k in ops._LINEAR_CHOICE}
     try:
         for k in keys:
@@ -43,7 +43,8 @@ def test_the_tuned_table_decides_per_shape_rows_and_use():
         assert ops.linear_choice(x, w) == ("wide", 1, 2, 3) and ops.linear_choice(x, w, "glu") == ("wide", 2, 1, 3)
         assert ops.linear_choice(x, w, "qkv") is None and ops.linear_choice(x[:8], w) is None
         assert ops.linear_choice(x[:33], w) == ("wide", 1, 2, 3)  # 33 to 64 rows share a bucket
-        assert ops.linear_choice(torch.zeros(65, 256, dtype=torch.bfloat16), w) is None  # too many rows
+        assert ops.linear_choice(torch.zeros(65, 256, dtype=torch.bfloat16), w) is None  # the next bucket, never measured
+        assert ops.linear_choice(torch.zeros(129, 256, dtype=torch.bfloat16), w) is None  # too many rows
         assert ops.linear_choice(torch.zeros(40, 192, dtype=torch.bfloat16), torch.zeros(96, 192, dtype=torch.bfloat16)) is None  # K % 128
         assert ops.linear_choice(x.float(), w.float()) is None
     finally:
@@ -58,3 +59,8 @@ def test_which_candidates_are_charged_a_kernel_of_their_own_for_the_second_half(
         assert ops._fuses_tail(choice, "plain") and ops._fuses_tail(choice, "sum")
     assert [ops._fuses_tail(c, "glu") for c in (None, stream, whole, split)] == [False, True, True, False]
     assert [ops._fuses_tail(c, "qkv") for c in (None, stream, whole, split)] == [False, True, False, True]
+
+
+def test_which_launches_of_the_wide_kernel_fit_lds():
+    assert ops.wide_fits(64, 2, 3) and ops.wide_fits(128, 1, 3) and ops.wide_fits(128, 2, 2) and not ops.wide_fits(128, 2, 3)
+    assert ops.wide_fits(20, 2, 3) and ops.wide_fits(65, 1, 2)

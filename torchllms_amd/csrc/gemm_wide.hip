@@ -1,4 +1,4 @@
-// C[M, N] = A[M, K] * W[N, K]^T for 17 to 64 rows, bfloat16 inputs, 32-bit accumulation: the matrix
+// C[M, N] = A[M, K] * W[N, K]^T for 17 to 128 rows, bfloat16 inputs, 32-bit accumulation: the matrix
 // products of decode steps with many requests.  Their cost is still reading W once from HBM, but
 // the rows of A are now a quarter of a megabyte and more, so the blocks must share what they read
 // of A instead of each wave fetching it for its own strip of columns.
@@ -313,7 +313,7 @@ int launch_rows(int ncw, int stages, const Launch& l) {
 
 int run(Launch l, int strips_per_wave, int stages) {
   TL_REQUIRE(l.M >= 0 && l.N > 0 && l.K > 0, "gemm_wide: bad sizes M=%d N=%d K=%d", l.M, l.N, l.K);
-  if (l.M > 64) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_wide: M=%d exceeds 64", l.M);
+  if (l.M > 128) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_wide: M=%d exceeds 128", l.M);
   if (l.K % kStepK) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_wide: K=%d is not a multiple of %d", l.K, kStepK);
   TL_REQUIRE(l.lda >= l.K && l.ldw >= l.K && l.ldc >= l.N, "gemm_wide: leading dimensions too small");
   TL_REQUIRE(l.lda % 8 == 0 && l.ldw % 8 == 0 && ((uintptr_t)l.A % 16) == 0 && ((uintptr_t)l.W % 16) == 0,
@@ -327,16 +327,18 @@ int run(Launch l, int strips_per_wave, int stages) {
              "gemm_wide: a split product needs the 16-byte aligned partial buffer");
   if (l.M == 0) return TL_OK;
   if (l.M <= 32) return launch_rows<2>(strips_per_wave, stages, l);
-  return launch_rows<4>(strips_per_wave, stages, l);
+  if (l.M <= 64) return launch_rows<4>(strips_per_wave, stages, l);
+  return launch_rows<8>(strips_per_wave, stages, l);
 }
 
 }  // namespace
 
 // A [M, K] and W [N, K] bfloat16, row-major with leading dimensions lda / ldw (multiples of 8, bases
-// 16-byte aligned); C [M, N] bfloat16 (out_dtype 1) or 32-bit (out_dtype 0).  M <= 64, K a multiple
+// 16-byte aligned); C [M, N] bfloat16 (out_dtype 1) or 32-bit (out_dtype 0).  M <= 128, K a multiple
 // of 128.  strips_per_wave: 1 or 2 (a block owns 64 or 128 columns).  k_splits >= 1: blocks along
 // K; with more than one, `partial` must hold k_splits * M * N floats.  stages: 2 or 3 buffers of LDS
-// (a buffer is 4 KB for every 16 rows of A, 32 or 64 of them, plus 16 KB for every strip per wave).
+// (a buffer is 4 KB for every 16 rows of A, 32, 64 or 128 of them, plus 16 KB for every strip per
+// wave; three buffers of 128 rows and two strips do not fit the 160 KB and are refused).
 // reduce = 0: the second kernel is left out; `partial` then holds tl_gemm_wide_splits(K, k_splits)
 // slices [M, N] for the caller to add (in their order, for the same result), and C is not touched.
 TL_EXPORT int tl_gemm_wide(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,

@@ -284,7 +284,7 @@ def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     return out
 
 
-WIDE_MAX_ROWS = 64
+WIDE_MAX_ROWS = 128
 
 
 def _wide_shapes(x: torch.Tensor, w: torch.Tensor, what: str) -> None:
@@ -318,7 +318,7 @@ class SplitSums:
 
 def gemm_wide(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, strips_per_wave: int = 1,
               k_splits: int = 1, stages: int = 3, leave_split: bool = False):
-    """``x @ w.T`` for at most 64 rows of bfloat16 ``x`` (K a multiple of 128) with the kernel whose
+    """``x @ w.T`` for at most 128 rows of bfloat16 ``x`` (K a multiple of 128) with the kernel whose
     blocks share their slice of ``x`` through LDS; ``k_splits`` > 1 cuts K over several blocks whose
     32-bit partial sums a second kernel adds, or, with ``leave_split``, come back as ``SplitSums``."""
     _wide_shapes(x, w, "gemm_wide")
@@ -348,7 +348,7 @@ def gemm_wide(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
 
 
 def gemm_wide_glu(x: torch.Tensor, w: torch.Tensor, strips_per_wave: int = 1, stages: int = 3) -> torch.Tensor:
-    """``silu(x @ gate.T) * (x @ up.T)`` for at most 64 rows of bfloat16 ``x`` and ``w`` [2F, K] =
+    """``silu(x @ gate.T) * (x @ up.T)`` for at most 128 rows of bfloat16 ``x`` and ``w`` [2F, K] =
     gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``."""
     _wide_shapes(x, w, "gemm_wide_glu")
     if w.shape[0] % 2:
@@ -402,7 +402,7 @@ def gemm_wide_qkv(
     k_splits: int = 4,
     stages: int = 3,
 ) -> torch.Tensor:
-    """As ``gemm_stream_qkv`` for at most 64 rows: the product split along K, and the kernel that
+    """As ``gemm_stream_qkv`` for at most 128 rows: the product split along K, and the kernel that
     adds the splits rotates the heads and writes keys and values into their pages."""
     width = _qkv_shapes("gemm_wide_qkv", x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size)
     m, k = x.shape
@@ -477,7 +477,7 @@ def stream_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def wide_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether the kernel for 17 to 64 rows can take this product at all."""
+    """Whether the kernel for 17 to 128 rows can take this product at all."""
     return (
         x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and STREAM_MAX_ROWS < x.shape[0] <= WIDE_MAX_ROWS
         and x.shape[1] % 128 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
@@ -491,11 +491,19 @@ def wide_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
 #:   None                                          the library
 #: Shapes never measured follow the size rule below.
 _LINEAR_CHOICE: dict = {}
-ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64)
+ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128)
 STREAM_WAVE_CHOICES = (0, 4)
 #: (strips per wave, splits of K, buffers) that ``tune_linear`` tries from 17 rows on: whole-K
 #: launches for matrices with many rows, splits of K for those with few
-WIDE_CHOICES = ((1, 1, 3), (2, 1, 3), (1, 4, 3), (1, 8, 3), (2, 8, 3))
+WIDE_CHOICES = ((1, 1, 3), (2, 1, 3), (2, 1, 2), (1, 4, 3), (1, 8, 3), (2, 8, 3), (2, 8, 2))
+
+
+def wide_fits(rows: int, strips_per_wave: int, stages: int) -> bool:
+    """Whether the buffers of such a launch fit the 160 KB of LDS: a buffer holds 4 KB for every 16
+    rows of the row tile (32, 64 or 128) and 16 KB for every strip per wave."""
+    tile = 32 if rows <= 32 else 64 if rows <= 64 else 128
+    return stages * (tile // 16 * 4 + strips_per_wave * 16) <= 160
+
 #: how a product is used: alone; as the first half of ``linear_glu`` / ``qkv_rope_store``, whose
 #: second half (gate, rotation and cache write) some kernels take into themselves; or ("sum",
 #: ``linear_to_sum``) as a term of the residual sum, where the norm that follows adds up a split
@@ -616,7 +624,9 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         if bucket <= STREAM_MAX_ROWS:
             candidates = [("stream", waves) for waves in STREAM_WAVE_CHOICES]
         elif wide_supported(x, weights[0]):
-            candidates = [("wide",) + c for c in WIDE_CHOICES if c[1] <= k // 128]
+            candidates = [("wide",) + c for c in WIDE_CHOICES if c[1] <= k // 128 and wide_fits(bucket, c[0], c[2])]
+            # (two buffers are only tried where three do not fit)
+            candidates = [c for c in candidates if c[3] == 3 or not wide_fits(bucket, c[1], 3)]
         else:
             candidates = []
         for choice in candidates:
@@ -637,7 +647,7 @@ def _run_choice(choice, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16: for up to 64 rows (decode steps)
+    """``x @ w.T``.  float32: the true 32-bit kernel.  bfloat16: for up to 128 rows (decode steps)
     one of the two MFMA kernels that are built around reading ``w`` once, or the BLAS library's
     matrix product, whichever was measured faster for the shape (``tune_linear``); for more rows the
     library, as the reference uses its library's (torchllms/models/networks.py:474-493).
@@ -693,7 +703,7 @@ def qkv_rope_store(
     """Projection into query | key | value heads, rotation of queries and keys by position, keys
     and values appended to their pages; returns the row-major [n, (Hq + 2 Hkv) * dh] buffer whose
     query part the attention kernels read.  Fused into the product's own kernels where one of the
-    decode kernels serves it (at most 64 bfloat16 rows, no bias, interleaved pairs, head size a
+    decode kernels serves it (at most 128 bfloat16 rows, no bias, interleaved pairs, head size a
     multiple of 4), else product, bias and rotary kernels in turn."""
     if x.dtype == torch.bfloat16:
         _gpu(x, w)
