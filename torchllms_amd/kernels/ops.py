@@ -552,8 +552,9 @@ _TUNE_FLUSH_BYTES = 512 << 20  # twice the 256 MB of last-level cache
 def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "plain", iters: int = 8, report=None) -> None:
     """Measure, for matrices of one shape and every row bucket, which bfloat16 kernel and launch is
     fastest on this GPU, and remember it.  ``weights``: the model's tensors of that shape; ``use``:
-    one of ``LINEAR_USES``.  The plain product is what is timed; a candidate that cannot take the
-    second half of a fused use into itself is charged the kernel that has to follow it.
+    one of ``LINEAR_USES``.  "glu" times the whole gated product as ``linear_glu`` would run it,
+    "sum" a product that may stay split; for "qkv" the plain product is timed and a candidate that
+    cannot take rotation and cache write into itself is charged the kernel that has to follow it.
 
     Timing is made like a decode step: the launches are recorded into a HIP graph and replayed (a
     product that needs two kernels is then charged what a second graph node costs, not what a
@@ -571,6 +572,8 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         return
     if use not in LINEAR_USES:
         raise ValueError(f"use must be one of {LINEAR_USES}, got {use!r}")
+    if use == "glu" and n % 2:
+        raise ValueError(f"a gated matrix holds gate rows and as many up rows, got {n} rows")
     if all((n, k, bucket, use) in _LINEAR_CHOICE for bucket in ROW_BUCKETS):
         return
     device = weights[0].device
@@ -605,7 +608,7 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         return best
 
     def cost(bucket, choice, fn) -> float:
-        tail = 0.0 if _fuses_tail(choice, use) else _TAIL_KERNEL_US * 1e-3 * iters
+        tail = _TAIL_KERNEL_US * 1e-3 * iters if use == "qkv" and not _fuses_tail(choice, use) else 0.0
         t = clock(fn) + tail
         if report is not None:
             report(bucket, choice, t / iters * 1e3)
@@ -616,11 +619,12 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
             continue
         x = torch.randn((bucket, k), device=device, dtype=torch.float32).to(torch.bfloat16)
 
-        def library(w):
-            y = torch.nn.functional.linear(x, w)
-            return y if y.dtype == out_dtype else y.to(out_dtype)
+        def run(choice):
+            if use == "glu":
+                return lambda w: _run_glu(choice, x, w)
+            return lambda w: _run_choice(choice, x, w, out_dtype, leave_split=use == "sum")
 
-        best, best_time = None, cost(bucket, None, library)
+        best, best_time = None, cost(bucket, None, run(None))
         if bucket <= STREAM_MAX_ROWS:
             candidates = [("stream", waves) for waves in STREAM_WAVE_CHOICES]
         elif wide_supported(x, weights[0]):
@@ -630,7 +634,7 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         else:
             candidates = []
         for choice in candidates:
-            t = cost(bucket, choice, lambda w: _run_choice(choice, x, w, out_dtype, leave_split=use == "sum"))
+            t = cost(bucket, choice, run(choice))
             if t < best_time:
                 best, best_time = choice, t
         _LINEAR_CHOICE[(n, k, bucket, use)] = best
@@ -675,7 +679,10 @@ def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     if x.dtype != torch.bfloat16:
         return silu_mul(linear(x, w))
     _gpu(x, w)
-    choice = linear_choice(x, w, "glu")
+    return _run_glu(linear_choice(x, w, "glu"), x, w)
+
+
+def _run_glu(choice, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     if choice is not None and choice[0] == "stream":
         return gemm_stream_glu(x, w, choice[1])
     if choice is not None and choice[0] == "wide" and choice[2] == 1:
