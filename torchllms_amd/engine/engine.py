@@ -109,7 +109,10 @@ class Engine:
         # step's shape alone
         from .graphs import DecodeGraphs
 
-        graph_safe = all(getattr(b.mixer, "graph_safe", False) for b in self.model.blocks)
+        parts = [self.model.embedding, self.model.final_norm, self.model.head]
+        for b in self.model.blocks:
+            parts += [b, b.mixer, b.feed_forward, b.mixer_norm, b.ffn_norm]
+        graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
         self.graphs = DecodeGraphs(self.model, self.cache, self.device, page_size) if (use_graphs and graph_safe) else None
 
     # ------------------------------------------------------------------ construction

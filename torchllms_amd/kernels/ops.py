@@ -316,6 +316,12 @@ class SplitSums:
         return out
 
 
+def resolved(x):
+    """``x`` as a tensor: a ``SplitSums`` is added up, a tensor is returned as it is.  For code that
+    does arithmetic of its own on what a mixer or feed-forward returned."""
+    return x.resolve() if isinstance(x, SplitSums) else x
+
+
 def gemm_wide(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, strips_per_wave: int = 1,
               k_splits: int = 1, stages: int = 3, leave_split: bool = False):
     """``x @ w.T`` for at most 128 rows of bfloat16 ``x`` (K a multiple of 128) with the kernel whose

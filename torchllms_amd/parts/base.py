@@ -65,6 +65,11 @@ class StateNeed:
 class Part:
     """Base of all parts."""
 
+    #: True only if what the part launches depends on the step's shape alone (no value read back
+    #: to the host, no launch whose size depends on data): a decode step is replayed from a HIP
+    #: graph only when every part of the model says so
+    graph_safe = False
+
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {}
 

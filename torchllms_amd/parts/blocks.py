@@ -11,6 +11,8 @@ class PreNormBlock(Block):
     (reference: torchllms/models/networks.py:635-644).  Each residual sum is fused into the
     norm that reads it; the last one is handed on as ``delta``."""
 
+    graph_safe = True
+
     def forward(self, h, delta, ctx, cache):
         h, y = self.mixer_norm.forward_add(h, self.mixer_norm.delta(delta))
         a = self.mixer.forward(y, ctx, cache)

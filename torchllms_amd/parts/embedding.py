@@ -14,6 +14,8 @@ from .base import EMBEDDINGS, HEADS, Embedding, Head, ParamSpec
 class TokenEmbedding(Embedding):
     """``h = weight[token]``, no scale factor (reference: torchllms/models/networks.py:793,1017)."""
 
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
@@ -33,6 +35,8 @@ class TokenEmbedding(Embedding):
 class LMHead(Head):
     """``logits = x W^T`` with W [vocab, hidden], no bias; with ``tied`` W is the embedding
     matrix (reference: torchllms/models/networks.py:804-809,1047).  Logits are returned in 32-bit."""
+
+    graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int, tied: bool):
         self.vocab_size = vocab_size

@@ -15,6 +15,8 @@ class SwiGLU(FeedForward):
     """``w2( silu(w1 x) * (w3 x) )`` without biases
     (reference: torchllms/models/networks.py:592-605)."""
 
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size

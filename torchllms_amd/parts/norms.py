@@ -15,6 +15,7 @@ class RMSNorm(Norm):
     """``y = cast(x32 * rsqrt(mean(x32^2) + eps)) * weight``: statistics and scaling in 32-bit,
     the weight multiply after the cast back (reference: torchllms/models/networks.py:186-200)."""
 
+    graph_safe = True
     takes_split_sums = True  # ops.rmsnorm adds the slices of a split product while it reads them
 
     def __init__(self, size: int, eps: float):
