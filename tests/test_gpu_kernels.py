@@ -701,7 +701,7 @@ def test_gemm_stream(m, n, k, out_dtype):
         assert (got.double() - want).abs().max().item() <= tol, f"waves={waves}"
 
 
-@pytest.mark.parametrize("m, f, k", [(1, 4096, 1024), (8, 14336, 4096), (5, 100, 136), (16, 688, 96), (12, 24, 8)])
+@pytest.mark.parametrize("m, f, k", [(1, 4096, 1024), (8, 14336, 4096), (5, 100, 136), (16, 688, 96), (12, 24, 8), (3, 13, 264)])
 def test_gemm_stream_glu_equals_the_product_followed_by_the_gate(m, f, k):
     """The same roundings as the two kernels it replaces; the 32-bit sums may differ in their last
     bit (blocks walk K from different starting steps), so single results may move by one rounding."""
@@ -710,9 +710,10 @@ def test_gemm_stream_glu_equals_the_product_followed_by_the_gate(m, f, k):
     w = (torch.randn(2 * f, k) * 0.1).bfloat16().to(DEV)
     for waves in (0, 1, 2, 4, 8):
         want = _ops().silu_mul(_ops().gemm_stream(x, w, torch.bfloat16, waves=waves))
-        got = _ops().gemm_stream_glu(x, w, waves=waves)
-        torch.testing.assert_close(got.float(), want.float(), rtol=2 ** -6, atol=2 ** -8 * want.float().abs().max().item(), msg=f"waves={waves}")
-        assert (got != want).float().mean().item() < 0.05, f"waves={waves}"
+        for cols in (16, 8):  # both shapes of a block: gate and up tiles of 16 columns, or 8 + 8 rows in one tile
+            got = _ops().gemm_stream_glu(x, w, waves=waves, cols=cols)
+            torch.testing.assert_close(got.float(), want.float(), rtol=2 ** -6, atol=2 ** -8 * want.float().abs().max().item(), msg=f"waves={waves} cols={cols}")
+            assert (got != want).float().mean().item() < 0.05, f"waves={waves} cols={cols}"
     ref = torch.nn.functional.silu(x.float() @ w[:f].float().T) * (x.float() @ w[f:].float().T)
     torch.testing.assert_close(_ops().linear_glu(x, w).float(), ref, rtol=2 ** -6, atol=2 ** -6 * ref.abs().max().item())
 
@@ -753,17 +754,21 @@ def test_tune_linear_remembers_a_choice_for_every_row_bucket():
     for key in [k for k in ops._LINEAR_CHOICE if k[:2] == (48, 64)]:
         del ops._LINEAR_CHOICE[key]
     ops.tune_linear(weights)
+    ops.tune_linear(weights, use="glu")
     for bucket in ops.ROW_BUCKETS:
         if bucket <= ops.STREAM_MAX_ROWS:
             assert ops._LINEAR_CHOICE[(48, 64, bucket, "plain")] in (None,) + tuple(("stream", w) for w in ops.STREAM_WAVE_CHOICES)
+            assert ops._LINEAR_CHOICE[(48, 64, bucket, "glu")] in (None,) + tuple(("stream", w, c) for w in ops.STREAM_WAVE_CHOICES for c in (8, 16))
         else:
             assert ops._LINEAR_CHOICE[(48, 64, bucket, "plain")] is None  # K = 64 is no multiple of 128: the library
     x = torch.randn(5, 64, device=DEV).bfloat16()
     got = ops.linear(x, weights[0]).float().cpu()
     torch.testing.assert_close(got, (x.float() @ weights[0].float().T).cpu(), rtol=2 ** -7, atol=0.1)
+    glu = (torch.nn.functional.silu(x.float() @ weights[0][:24].float().T) * (x.float() @ weights[0][24:].float().T)).cpu()
+    torch.testing.assert_close(ops.linear_glu(x, weights[0]).float().cpu(), glu, rtol=2 ** -6, atol=0.1)
 
 
-# ----------------------------------------------------------------------------- shared-activation matrix product (17 to 64 rows)
+# ----------------------------------------------------------------------------- shared-activation matrix product (17 to 128 rows)
 @pytest.mark.parametrize(
     "m, n, k",
     [(64, 4096, 4096), (32, 6144, 4096), (17, 200, 128), (64, 4100, 384), (33, 72, 2048), (48, 1000, 1024), (5, 64, 256),

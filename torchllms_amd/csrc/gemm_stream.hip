@@ -14,7 +14,12 @@
 //     fetched and transposed the same way (only as many groups of four rows as M needs).
 //   * the LDS rows are 272 bytes apart: the 16 lanes that read one 16-byte piece of 16 different
 //     rows then fall on different banks.
-//   * gated variant (GLU): W = gate rows | up rows; a block computes the same 16 columns of both
+//   * gated variant (GLU), in two shapes.  Half: the block's 16 rows of W are 8 gate rows and the 8 up
+//     rows of the same columns, so the launch looks like the plain product's (as many blocks, each
+//     fetching as much) and costs the same; the lanes that hold gate sums fetch the up sums from the
+//     lanes 32 further on.  With 16 rows of A, whose fetch every block repeats, twice as many blocks
+//     cost more than they gain, hence the other shape.  Full:
+//     W = gate rows | up rows; a block computes the same 16 columns of both
 //     products from one fetch of A and stores silu(gate) * up, with the roundings of the unfused
 //     sequence (both products rounded to bfloat16, the activation rounded, then the product).
 //   * query/key/value variant (QKV): the columns are query heads | key heads | value heads; query and
@@ -39,10 +44,11 @@ constexpr int kTileElems = 16 * kPitch;
 __device__ __forceinline__ short4_t lo_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[0], v[1]}); }
 __device__ __forceinline__ short4_t hi_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[2], v[3]}); }
 
-enum Epilogue { kPlain = 0, kGated = 1, kQkv = 2 };
+enum Epilogue { kPlain = 0, kGated = 1, kQkv = 2, kGatedHalf = 3 };
 
 // MR: groups of four rows of A that are fetched (M <= 4 * MR).  WAVES: waves per block = splits of K.
-// EPI kGated: W holds 2 N rows, gate rows then up rows; C[M, N] = silu(A gate^T) * (A up^T).
+// EPI kGated, kGatedHalf: W holds 2 N rows, gate rows then up rows; C[M, N] = silu(A gate^T) * (A up^T);
+// a block owns 16 (kGated) or 8 (kGatedHalf) columns of C.
 template <int MR, int WAVES, typename OutT, int EPI>
 __global__ void __launch_bounds__(WAVES* kWave)
 gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
@@ -59,7 +65,8 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   const int g4 = lane / 16;   // operand layout: piece within a group of four
   const int q = lane / 16;    // fetch layout: row within a group of four
   const int piece = lane % 16;  // fetch layout: 16-byte piece of the row's 256 bytes
-  const int n0 = blockIdx.x * kStrip;
+  constexpr bool HALF = EPI == kGatedHalf;
+  const int n0 = blockIdx.x * (HALF ? kStrip / 2 : kStrip);
   bf16_t* w_lds = lds + (size_t)wave * kWaveElems;
   bf16_t* a_lds = w_lds + kTileElems;
 
@@ -75,8 +82,11 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
 #pragma unroll
   for (int t = 0; t < NW; ++t)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      wsrc[4 * t + j] = W + ((size_t)t * N + min(n0 + 4 * j + q, N - 1)) * ldw + 8 * piece;
+    for (int j = 0; j < 4; ++j) {
+      // half: tile rows 0..7 are gate rows n0.., rows 8..15 the up rows of the same columns
+      const size_t row = HALF ? (size_t)(j / 2) * N + min(n0 + 4 * (j % 2) + q, N - 1) : (size_t)t * N + min(n0 + 4 * j + q, N - 1);
+      wsrc[4 * t + j] = W + row * ldw + 8 * piece;
+    }
   const bf16_t* asrc[MR];
 #pragma unroll
   for (int j = 0; j < MR; ++j) {
@@ -195,6 +205,23 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
       const float sums[4] = {acc[0][0], acc[0][1], acc[0][2], acc[0][3]};
       qkv_finish(sums, n16, n, qa, reinterpret_cast<bf16_t*>(C), ldc);
     }
+  } else if constexpr (HALF) {
+    // lanes with g4 < 2 hold the gate sums of columns n0 + 4 g4 + i, the lanes 32 further on the up
+    // sums of the same columns (every lane takes part in the exchange)
+    float up[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) up[i] = __shfl(acc[0][i], (lane + 32) % kWave, kWave);
+    if (n16 < M && g4 < 2) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 4 * g4 + i;
+        if (n >= N) continue;
+        const float g = to_f32(from_f32<OutT>(acc[0][i]));
+        const float u = to_f32(from_f32<OutT>(up[i]));
+        const float act = to_f32(from_f32<OutT>(g / (1.0f + expf(-g))));
+        C[(size_t)n16 * ldc + n] = from_f32<OutT>(act * u);
+      }
+    }
   } else if (n16 < M) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -223,7 +250,8 @@ int launch_typed(const bf16_t* A, int lda, const bf16_t* W, int ldw, OutT* C, in
     if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "gemm_stream: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     raised = true;
   }
-  const dim3 grid((N + kStrip - 1) / kStrip);
+  constexpr int kCols = EPI == kGatedHalf ? kStrip / 2 : kStrip;  // columns of C per block
+  const dim3 grid((N + kCols - 1) / kCols);
   gemm_stream_kernel<MR, WAVES, OutT, EPI><<<grid, WAVES * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, qa);
   return tl_check_launch("gemm_stream");
 }
@@ -232,6 +260,7 @@ template <int MR, int WAVES>
 int launch(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N, int K,
            int out_dtype, int epi, const QkvArgs& qa, hipStream_t stream) {
   if (epi == kGated) return launch_typed<MR, WAVES, bf16_t, kGated>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
+  if (epi == kGatedHalf) return launch_typed<MR, WAVES, bf16_t, kGatedHalf>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
   if (epi == kQkv) return launch_typed<MR, WAVES, bf16_t, kQkv>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
   if (out_dtype == TL_BF16) return launch_typed<MR, WAVES, bf16_t, kPlain>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
   return launch_typed<MR, WAVES, float, kPlain>(A, lda, W, ldw, (float*)C, ldc, M, N, K, qa, stream);
@@ -260,7 +289,8 @@ int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M,
   if (M == 0) return TL_OK;
   if (waves == 0) {
     // enough waves to keep loads in flight on 256 CUs: about 4096 in all, at least two steps each
-    const int strips = (N + kStrip - 1) / kStrip;
+    const int cols = epi == kGatedHalf ? kStrip / 2 : kStrip;
+    const int strips = (N + cols - 1) / cols;
     const int steps = (K + kStepK - 1) / kStepK;
     waves = 1;
     while (waves < 8 && strips * waves < 4096 && steps >= 2 * waves * 2) waves *= 2;
@@ -285,10 +315,11 @@ TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, voi
 
 // The gated pair of products: W [2 N, K] = gate rows | up rows; C [M, N] bfloat16 =
 // silu(A gate^T) * (A up^T), rounded as the two products, the activation and the final product
-// would be if each were stored in bfloat16.
+// would be if each were stored in bfloat16.  cols: 16 or 8 columns of C per block.
 TL_EXPORT int tl_gemm_stream_glu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
-                                 int K, int waves, hipStream_t stream) {
-  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, kGated, QkvArgs{}, stream);
+                                 int K, int waves, int cols, hipStream_t stream) {
+  TL_REQUIRE(cols == 8 || cols == 16, "gemm_stream_glu: cols must be 8 or 16");
+  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, cols == 8 ? kGatedHalf : kGated, QkvArgs{}, stream);
 }
 
 // The query/key/value projection with the rotary kernel's work in its epilogue.  W [(Hq + 2 Hkv) *

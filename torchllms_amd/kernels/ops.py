@@ -424,9 +424,10 @@ def gemm_wide_qkv(
     return out
 
 
-def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0) -> torch.Tensor:
+def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0, cols: int = 16) -> torch.Tensor:
     """``silu(x @ gate.T) * (x @ up.T)`` for at most 16 rows of bfloat16 ``x`` and ``w`` [2F, K] =
-    gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``."""
+    gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``.  ``cols``: 16
+    or 8 columns of the result per block (8: a launch shaped like the plain product's)."""
     _gpu(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("gemm_stream_glu takes bfloat16 tensors")
@@ -437,7 +438,7 @@ def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0) -> torch.T
     out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     check(
         core().tl_gemm_stream_glu(
-            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k, waves, _stream(),
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k, waves, cols, _stream(),
         )
     )
     return out
@@ -492,7 +493,8 @@ def wide_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 #: measured choice of bfloat16 kernel by (n, k, row bucket, use); filled by ``tune_linear``:
-#:   ("stream", waves)                             the weight-streaming kernel (waves 0 = its own rule)
+#:   ("stream", waves[, cols])                     the weight-streaming kernel (waves 0 = its own rule;
+#:                                                 cols: columns per block of the gated form, 8 or 16)
 #:   ("wide", strips_per_wave, k_splits, stages)   the kernel whose blocks share the activations
 #:   None                                          the library
 #: Shapes never measured follow the size rule below.
@@ -631,7 +633,9 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
             return lambda w: _run_choice(choice, x, w, out_dtype, leave_split=use == "sum")
 
         best, best_time = None, cost(bucket, None, run(None))
-        if bucket <= STREAM_MAX_ROWS:
+        if bucket <= STREAM_MAX_ROWS and use == "glu":
+            candidates = [("stream", waves, cols) for waves in STREAM_WAVE_CHOICES for cols in (8, 16)]
+        elif bucket <= STREAM_MAX_ROWS:
             candidates = [("stream", waves) for waves in STREAM_WAVE_CHOICES]
         elif wide_supported(x, weights[0]):
             candidates = [("wide",) + c for c in WIDE_CHOICES if c[1] <= k // 128 and wide_fits(bucket, c[0], c[2])]
@@ -690,7 +694,7 @@ def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 def _run_glu(choice, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     if choice is not None and choice[0] == "stream":
-        return gemm_stream_glu(x, w, choice[1])
+        return gemm_stream_glu(x, w, choice[1], choice[2] if len(choice) > 2 else 16)
     if choice is not None and choice[0] == "wide" and choice[2] == 1:
         return gemm_wide_glu(x, w, choice[1], choice[3])
     return silu_mul(_run_choice(choice, x, w, x.dtype))
