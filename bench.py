@@ -2,6 +2,7 @@
 bfloat16 weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
+                    [--shape 8b|1b|70b] [--workload decode|serve]
 
 A step is one decode step of the whole batch: ``Engine.step`` on one token per request followed by
 the sampling kernel and the copy of the chosen tokens to the host, as generation does it.  The
@@ -10,6 +11,11 @@ which costs a decode step the same reads.  One JSON line is printed: ``value`` i
 second at the default batch; ``prefill`` times one 2,048-token prompt; ``roofline`` sets the decode
 step's unavoidable reads (every weight once, the live requests' cache) against HBM's 8 TB/s;
 ``points`` holds decode at batch 1 and 64.
+
+``--shape`` takes the layer sizes of Llama-3.2-1B or Llama-3.1-70B instead (the default is the
+headline's 8B).  ``--workload serve`` runs the scheduler instead of fixed batches: 64 requests at
+once, prompts of 128 to 4,096 random tokens, 512 tokens generated for each at temperature 0.7; its
+line reports generated tokens a second over the whole run, prefill included.
 """
 
 from __future__ import annotations
@@ -32,6 +38,17 @@ LLAMA_8B = dict(
 )
 
 
+SHAPES = {
+    "8b": LLAMA_8B,
+    "1b": dict(LLAMA_8B, hidden_size=2048, num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               intermediate_size=8192, tie_word_embeddings=True,
+               rope_scaling=dict(LLAMA_8B["rope_scaling"], factor=32.0)),
+    "70b": dict(LLAMA_8B, hidden_size=8192, num_hidden_layers=80, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+                intermediate_size=28672),
+}
+SHAPE_NAMES = {"8b": "Llama-3.1-8B shape", "1b": "Llama-3.2-1B shape", "70b": "Llama-3.1-70B shape"}
+
+
 def parse_args(argv=None):
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -44,6 +61,10 @@ def parse_args(argv=None):
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     p.add_argument("--page-size", type=int, default=16)
+    p.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the headline's)")
+    p.add_argument("--workload", default="decode", choices=["decode", "serve"])
+    p.add_argument("--requests", type=int, default=64, help="serve: requests running at once")
+    p.add_argument("--new-tokens", type=int, default=512, help="serve: tokens generated for every request")
     return p.parse_args(argv)
 
 
@@ -150,20 +171,76 @@ def prefill_flops(cfg, n_layers, T):
     return n_layers * (T * per_token + attn) + 2 * D * V
 
 
+def serve_run(args, shape) -> int:
+    """The continuous-batching workload: every request is admitted at once, prompts are cut into
+    portions under the token budget beside the running requests' decode tokens."""
+    import random
+
+    import torch
+
+    from torchllms_amd.config import LlamaConfig
+    from torchllms_amd.engine import Engine
+    from torchllms_amd.inference.llm import GenerationLoop
+    from torchllms_amd.sampling import Sampler, SamplingParams
+
+    n_layers = args.layers or shape["num_hidden_layers"]
+    cfg = LlamaConfig.from_dict(dict(shape, num_hidden_layers=n_layers))
+    longest, budget = 4096, 4096
+    engine = Engine.from_random(cfg, seed=0, dtype=args.dtype, draw_on_device=True, page_size=args.page_size,
+                                max_seqs=args.requests, max_model_len=longest + args.new_tokens)
+    rng = random.Random(0)
+    prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(128, longest))] for _ in range(args.requests)]
+    params = [SamplingParams(temperature=0.7, max_new_tokens=args.new_tokens, seed=i) for i in range(args.requests)]
+    loop = GenerationLoop(engine, Sampler(), max_num_seqs=args.requests, max_num_batched_tokens=budget,
+                          max_model_len=longest + args.new_tokens)
+    steps = [0]
+
+    def count(plan):
+        steps[0] += 1
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    requests = loop.run(prompts, params, count)
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    generated = sum(len(r.output) for r in requests)
+    prompt_tokens = sum(len(p) for p in prompts)
+    engine.cache.check_invariants()
+    print(json.dumps({
+        "metric": f"generated tok/s, {args.requests} requests at once, prompts of 128..{longest} tokens, {args.new_tokens} new tokens each, {SHAPE_NAMES[args.shape]}",
+        "value": round(generated / sec, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps[0], "warmup": 0,
+        "ms_per_step": round(sec / steps[0] * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: random-init weights, random token ids",
+        "config": {"model": SHAPE_NAMES[args.shape], "global_batch": args.requests, "seq_len": longest + args.new_tokens,
+                   "parallelism": "single GPU", "n_layers": n_layers, "n_layers_full": shape["num_hidden_layers"],
+                   "hidden_size": cfg.hidden_size, "n_heads": cfg.num_attention_heads, "n_kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+                   "page_size": args.page_size, "token_budget": budget, "temperature": 0.7},
+        "seconds": round(sec, 3), "prompt_tokens": prompt_tokens, "generated_tokens": generated,
+        "total_tokens_per_s": round((prompt_tokens + generated) / sec, 1),
+        "preemptions": loop.scheduler.stats["preemptions"],
+    }))
+    return 0
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
         return 2
+    shape = SHAPES[args.shape]
+    if args.workload == "serve":
+        return serve_run(args, shape)
     import torch
 
     from torchllms_amd.config import LlamaConfig
     from torchllms_amd.engine import Engine
     from torchllms_amd.sampling import Sampler
 
-    full_layers = LLAMA_8B["num_hidden_layers"]
+    full_layers = shape["num_hidden_layers"]
     n_layers = args.layers or full_layers
-    cfg = LlamaConfig.from_dict(dict(LLAMA_8B, num_hidden_layers=n_layers))
+    cfg = LlamaConfig.from_dict(dict(shape, num_hidden_layers=n_layers))
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
     max_batch = max(batches)
     pages_per_req = -(-args.context // args.page_size) + 1
@@ -189,7 +266,7 @@ def main(argv=None) -> int:
     main_r = results[args.batch]
     achieved = main_r["bytes"] / main_r["sec"] / 1e9
     line = {
-        "metric": f"decode tok/s at batch {args.batch}, Llama-3.1-8B shape (plus batch {'/'.join(str(b) for b in batches[1:]) or 'none'}"
+        "metric": f"decode tok/s at batch {args.batch}, {SHAPE_NAMES[args.shape]} (plus batch {'/'.join(str(b) for b in batches[1:]) or 'none'}"
                   f" and prefill tok/s at {args.prefill_tokens} tokens)",
         "value": round(main_r["tps"], 2),
         "unit": "tokens/s",
@@ -203,7 +280,7 @@ def main(argv=None) -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: random-init weights, random token ids, cache of earlier context filled with random values",
         "config": {
-            "model": "Llama-3.1-8B shape",
+            "model": SHAPE_NAMES[args.shape],
             "global_batch": args.batch,
             "seq_len": args.context,
             "parallelism": "single GPU",
@@ -217,7 +294,7 @@ def main(argv=None) -> int:
             "vocab_size": cfg.vocab_size,
             "page_size": args.page_size,
             "prefill_tokens": args.prefill_tokens,
-            "rope": "llama3 factor 8 theta 5e5",
+            "rope": f"llama3 factor {shape['rope_scaling']['factor']:g} theta 5e5",
         },
         "prefill": {
             "value": round(args.prefill_tokens / pre_sec, 1),
