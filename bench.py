@@ -65,6 +65,7 @@ def parse_args(argv=None):
     p.add_argument("--workload", default="decode", choices=["decode", "serve"])
     p.add_argument("--requests", type=int, default=64, help="serve: requests running at once")
     p.add_argument("--new-tokens", type=int, default=512, help="serve: tokens generated for every request")
+    p.add_argument("--no-look-ahead", action="store_true", help="plan every decode step when it runs, not during the step before")
     return p.parse_args(argv)
 
 
@@ -108,8 +109,10 @@ def fill_context(engine, rids, n_tokens, seed=0):
             flat[lo : lo + chunk].normal_(0.0, 1.0, generator=g)
 
 
-def decode_run(engine, sampler, batch, context, steps, warmup, vocab):
-    """Time ``steps`` decode steps of ``batch`` requests whose context ends at ``context`` tokens."""
+def decode_run(engine, sampler, batch, context, steps, warmup, vocab, look_ahead=True):
+    """Time ``steps`` decode steps of ``batch`` requests whose context ends at ``context`` tokens.
+    A step is what the generation loop does for one: run the batch, sample, read the tokens; with
+    ``look_ahead`` the next step's plan is made while the GPU runs this one, as the loop does."""
     import torch
 
     from torchllms_amd.engine import StepEntry
@@ -124,10 +127,17 @@ def decode_run(engine, sampler, batch, context, steps, warmup, vocab):
     params = [SamplingParams(temperature=0.0, seed=i) for i in range(batch)]
     tokens = [(7 * i + 3) % vocab for i in range(batch)]
 
+    prepared = None
+
     def one_step(k):
-        nonlocal tokens
-        logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(rids, tokens)])
-        tokens = sampler(logits, params, [k] * batch)
+        nonlocal tokens, prepared
+        entries = [StepEntry(r, [t], [0]) for r, t in zip(rids, tokens)]
+        logits = engine.step_prepared(prepared, entries) if prepared is not None else None
+        if logits is None:
+            logits = engine.step(entries)
+        pending = sampler.launch(logits, params, [k] * batch)
+        prepared = engine.prepare_decode() if look_ahead else None
+        tokens = pending.tolist()
 
     for k in range(prime + warmup):
         one_step(k)
@@ -192,7 +202,7 @@ def serve_run(args, shape) -> int:
     prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(128, longest))] for _ in range(args.requests)]
     params = [SamplingParams(temperature=0.7, max_new_tokens=args.new_tokens, seed=i) for i in range(args.requests)]
     loop = GenerationLoop(engine, Sampler(), max_num_seqs=args.requests, max_num_batched_tokens=budget,
-                          max_model_len=longest + args.new_tokens)
+                          max_model_len=longest + args.new_tokens, look_ahead=not args.no_look_ahead)
     steps = [0]
 
     def count(plan):
@@ -219,7 +229,7 @@ def serve_run(args, shape) -> int:
                    "page_size": args.page_size, "token_budget": budget, "temperature": 0.7},
         "seconds": round(sec, 3), "prompt_tokens": prompt_tokens, "generated_tokens": generated,
         "total_tokens_per_s": round((prompt_tokens + generated) / sec, 1),
-        "preemptions": loop.scheduler.stats["preemptions"],
+        "preemptions": loop.scheduler.stats["preemptions"], "prepared_steps": loop.stats["prepared_steps"],
     }))
     return 0
 
@@ -256,7 +266,7 @@ def main(argv=None) -> int:
     results = {}
     for b in batches:
         steps = args.steps if b == args.batch else max(args.steps // 2, 4)
-        sec, mean_ctx = decode_run(engine, sampler, b, args.context, steps, args.warmup, cfg.vocab_size)
+        sec, mean_ctx = decode_run(engine, sampler, b, args.context, steps, args.warmup, cfg.vocab_size, not args.no_look_ahead)
         step_bytes = wbytes + b * cfg.hidden_size * elt + b * mean_ctx * kv_per_token
         results[b] = dict(sec=sec, tps=b / sec, bytes=step_bytes)
 

@@ -99,6 +99,33 @@ def test_preemption_on_the_gpu_changes_nothing(model_b):
     tight.engine.cache.check_invariants()
 
 
+@pytest.mark.parametrize("precision", ["float32", "bfloat16"])
+def test_preparing_the_next_step_ahead_changes_no_token(model_b, precision):
+    """Seven requests of different lengths and budgets, three at a time, some ending on a stop
+    token: with the next decode step prepared during the current one, the tokens are those of the
+    loop that plans every step when it runs, and most decode steps did run prepared."""
+    from torchllms_amd.inference import LLM
+
+    folder, cfg, _ = model_b
+    prompts = [random_tokens(n, cfg["vocab_size"], 300 + n) for n in (3, 50, 17, 8, 33, 1, 25)]
+    llm = LLM(str(folder), precision=precision, max_len=160, max_bsz=3, page_size=8, max_num_batched_tokens=32)
+    assert llm.engine.graphs is not None
+    llm.look_ahead = False
+    base = llm.generate(prompt_token_ids=prompts, temperature=0.9, max_new_tokens=60, seed=5)
+    assert llm.last_stats["prepared_steps"] == 0
+    stops = [base[1].token_ids[20], base[4].token_ids[41]]  # end two of them early
+    want = llm.generate(prompt_token_ids=prompts, temperature=0.9, max_new_tokens=60, seed=5, stop_token_ids=stops)
+    steps = llm.last_stats["steps"]
+    assert any(r.stop_reason is not None for r in want) and any(r.stop_reason is None for r in want)
+    llm.look_ahead = True
+    got = llm.generate(prompt_token_ids=prompts, temperature=0.9, max_new_tokens=60, seed=5, stop_token_ids=stops)
+    assert [r.token_ids for r in got] == [r.token_ids for r in want]
+    assert [r.stop_reason for r in got] == [r.stop_reason for r in want]
+    assert llm.last_stats["steps"] == steps and llm.last_stats["prepared_steps"] > steps // 3
+    llm.engine.cache.check_invariants()
+    assert llm.engine.cache.live == []
+
+
 def test_generate_command_line(model_b, tmp_path):
     folder, cfg, weights = model_b
     prompts = [random_tokens(n, cfg["vocab_size"], 90 + n) for n in (4, 11)]

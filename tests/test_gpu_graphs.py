@@ -74,3 +74,61 @@ def test_context_cap_buckets():
     from torchllms_amd.engine.graphs import context_cap
 
     assert [context_cap(n) for n in (1, 512, 513, 1024, 5000, 8192)] == [512, 512, 1024, 1024, 8192, 8192]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prepared_decode_steps_match_plain_steps(tmp_path, dtype):
+    """Decode steps prepared one step ahead (plan made and uploaded before the tokens are known)
+    give the logits of steps planned when they run, across pages' edges and the context cap's
+    step from 512 to 1024, and a preparation that no longer fits is refused."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    cfg = TINY["B"]
+    folder = make_folder(tmp_path / "m", cfg, seed=33, dtype=torch.bfloat16, sharpen=True)
+    plain = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=4, max_model_len=1100)
+    ahead = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=4, max_model_len=1100)
+    vocab = cfg["vocab_size"]
+    toks = {r: random_tokens(600, vocab, 900 + i) for i, r in enumerate("abc")}
+    start = {"a": 470, "b": 23, "c": 7}
+    for eng in (plain, ahead):
+        for r in toks:
+            eng.admit(r)
+        eng.step([StepEntry(r, toks[r][: start[r]], []) for r in toks])
+    used = 0
+    prepared = None
+    for step in range(70):
+        entries = [StepEntry(r, [toks[r][start[r] + step]], [0]) for r in toks]
+        want = plain.step(entries).float().cpu()
+        got = ahead.step_prepared(prepared, entries) if prepared is not None else None
+        used += got is not None
+        if got is None:
+            got = ahead.step(entries)
+        prepared = ahead.prepare_decode()  # before the step's result is read, as the loop does
+        got = got.float().cpu()
+        if dtype == "float32":
+            assert torch.equal(want, got), step
+        else:
+            assert (want - got).abs().max().item() <= 2 ** -6 * max(want.abs().max().item(), 1.0), step
+    # a shape runs eagerly twice and is recorded at its third step; from then on every step is
+    # prepared, but for the same three steps after request a passes 512 tokens
+    assert used >= 70 - 2 * 4
+    assert plain.cache.num_tokens("a") == ahead.cache.num_tokens("a") == 540
+    # other entries than the prepared ones, or a request gone: refused, nothing run
+    steps_before = ahead.steps_run
+    assert prepared is not None
+    two = [StepEntry(r, [1], [0]) for r in "ab"]
+    assert ahead.step_prepared(prepared, two) is None
+    swapped = [StepEntry(r, [1], [0]) for r in "bac"]
+    assert ahead.step_prepared(prepared, swapped) is None
+    unwanted = [StepEntry(r, [1], []) for r in "abc"]
+    assert ahead.step_prepared(prepared, unwanted) is None
+    ahead.free("c")
+    assert ahead.step_prepared(prepared, [StepEntry(r, [1], [0]) for r in "abc"]) is None
+    assert ahead.steps_run == steps_before
+    assert ahead.prepare_decode() is None  # the last decode step's requests are not all there
+    for eng in (plain, ahead):
+        for r in toks:
+            if eng.cache.has(r):
+                eng.free(r)
+        eng.cache.check_invariants()
+        assert eng.cache.free_pages() == 160

@@ -237,3 +237,90 @@ def test_the_short_cut_for_decode_steps_plans_what_the_rules_plan():
     sched._schedule, sched.schedule = counted_rules, checked_schedule
     reqs = loop.run(prompts, [SamplingParams(max_new_tokens=rng.randint(2, 15)) for _ in prompts])
     assert all(r.finished for r in reqs) and state["short_cuts"] > 10 and state["by_rules"] >= 3
+
+
+class AheadEngine(FakeEngine):
+    """A fake engine that can prepare the next decode step as the real one does: it takes that
+    step's pages early, and uses the preparation only for the very step it was made for."""
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self._decoded = None
+        self.prepared = self.used = 0
+
+    def step(self, entries):
+        out = super().step(entries)
+        self._decoded = [e.rid for e in entries] if all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries) else None
+        return out
+
+    def prepare_decode(self):
+        if self._decoded is None:
+            return None
+        need = sum(self.cache.new_pages_needed(r, 1) for r in self._decoded)
+        if need > self.cache.free_pages():
+            return None
+        for r in self._decoded:
+            self.cache.extend(r, 1)
+        self.prepared += 1
+        return (list(self._decoded), self.cache.epoch)
+
+    def step_prepared(self, prepared, entries):
+        rids, epoch = prepared
+        if epoch != self.cache.epoch or [e.rid for e in entries] != rids:
+            return None
+        if any(len(e.tokens) != 1 or list(e.want) != [0] for e in entries):
+            return None
+        self.used += 1
+        return self.step(entries)
+
+
+class LaunchingSampler:
+    def __call__(self, logits, params, steps):
+        return greedy(logits, params, steps)
+
+    def launch(self, logits, params, steps):
+        return logits.argmax(-1)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_preparing_the_next_decode_step_changes_no_decision(seed):
+    """With an engine that prepares the next decode step during the current one (and takes its
+    pages early) the loop runs the same steps, preempts the same requests and gives the same
+    tokens as without; requests end on stop tokens and budgets, join late, and pools are tight."""
+    rng = random.Random(100 + seed)
+    n = rng.randint(3, 10)
+    prompts = [[1] * rng.randint(1, 30) for _ in range(n)]
+    news = [rng.randint(1, 24) for _ in range(n)]
+    stops = [(rng.randrange(VOCAB),) if rng.random() < 0.5 else () for _ in range(n)]
+    page = rng.choice([2, 4, 8])
+    longest = max(len(p) + m for p, m in zip(prompts, news))
+    pages, seqs, live = -(-longest // page) + rng.randint(0, 6), rng.randint(1, 4), rng.randint(1, 4)
+    budget, chunk = rng.choice([4, 5, 16, 64]), rng.choice([None, 3, 7])
+    runs = []
+    for make, sampler, ahead in ((FakeEngine, greedy, False), (AheadEngine, LaunchingSampler(), True), (AheadEngine, LaunchingSampler(), False)):
+        eng = make(num_pages=pages, page_size=page, max_seqs=seqs)
+        loop = GenerationLoop(eng, sampler, live, budget, 256, chunk, look_ahead=ahead)
+        reqs = loop.run(prompts, [SamplingParams(max_new_tokens=m, stop_token_ids=s) for m, s in zip(news, stops)])
+        assert eng.cache.live == []
+        eng.cache.check_invariants()
+        calls = [[(rid[2], start, k) for rid, start, k in call] for call in eng.calls]
+        runs.append(([r.output for r in reqs], [r.stop_reason for r in reqs], calls, loop.scheduler.stats["preemptions"]))
+        if ahead:
+            assert loop.stats["prepared_steps"] == eng.used
+        elif make is AheadEngine:
+            assert eng.prepared == 0
+    assert runs[0] == runs[1] == runs[2]
+
+
+def test_prepared_steps_are_used_and_dropped():
+    """Two requests decode side by side: all their decode steps but the first run prepared, until
+    one ends on its stop token; the step after that is planned anew."""
+    eng = AheadEngine(num_pages=32, page_size=4, max_seqs=2)
+    loop = GenerationLoop(eng, LaunchingSampler(), 2, 64, 256)
+    reqs = loop.run([[1] * 3, [1] * 5], [SamplingParams(max_new_tokens=12, stop_token_ids=(9,)), SamplingParams(max_new_tokens=12)])
+    assert reqs[0].output == [3, 4, 5, 6, 7, 8, 9] and len(reqs[1].output) == 12
+    # steps: 1 prefill, 11 decode steps; prepared were all decode steps but the first one, the one
+    # after the first request ended (its preparation no longer fits), and none after the last
+    assert len(eng.calls) == 12
+    assert eng.used == 11 - 2
+    assert eng.prepared == eng.used + 1  # one was made in vain

@@ -47,6 +47,15 @@ def require_gpu(device) -> torch.device:
     return device
 
 
+class PreparedDecode:
+    """A decode step whose plan is made and uploaded but for its tokens (``Engine.prepare_decode``)."""
+
+    __slots__ = ("rids", "wants", "previous", "layout", "graph", "epoch")
+
+    def __init__(self, rids, wants, previous, layout, graph, epoch):
+        self.rids, self.wants, self.previous, self.layout, self.graph, self.epoch = rids, wants, previous, layout, graph, epoch
+
+
 class Engine:
     def __init__(
         self,
@@ -166,29 +175,44 @@ class Engine:
         if last is None or len(entries) != len(last[0]):
             return None
         rids, wants, prev, epoch = last
+        toks = []
+        for e, rid, want in zip(entries, rids, wants):
+            if e.rid != rid or len(e.tokens) != 1 or list(e.want) != want:
+                return None
+            toks.append(e.tokens[0])
+        if min(toks) < 0 or max(toks) >= self.vocab_size:
+            return None
+        layout = self._next_decode_layout()
+        if layout is not None:
+            layout.tokens[:] = toks
+        return layout
+
+    def _next_decode_layout(self) -> Optional[StepLayout]:
+        """What ``_plan_next_decode`` knows before it has seen the tokens: the plan of the next
+        decode step of the last decode step's requests, with zeros for token ids.  Takes the pages
+        that the step needs; None, with nothing taken, when it cannot be."""
+        last = self._last_decode
+        if last is None:
+            return None
+        rids, wants, prev, epoch = last
         cache = self.cache
         if epoch != cache.epoch:
             return None
-        n = len(entries)
+        n = len(rids)
         held = prev.kv_lens.tolist()
         page = self.page_size
         get = cache.get
-        toks = []
         need = 0
-        for e, rid, want, have in zip(entries, rids, wants, held):
-            if e.rid != rid or len(e.tokens) != 1 or list(e.want) != want:
-                return None
+        for rid, have in zip(rids, held):
             live = get(rid)
             if live is None or live.num_tokens != have:
                 return None
-            toks.append(e.tokens[0])
             if have % page == 0:  # the new token opens a page
                 need += cache.new_pages_needed(rid, 1)
-        if min(toks) < 0 or max(toks) >= self.vocab_size or max(held) + 1 > self.max_model_len:
+        if max(held) + 1 > self.max_model_len:
             return None
         if any(need > pool.free_count for pool in cache.pools):
             return None
-        tokens = np.asarray(toks, dtype=np.int32)
         positions = prev.kv_lens.copy()  # the new token's position = tokens held so far
         fresh = (positions % page) == 0  # rows whose new token opens a page; the others have room
         for i in np.nonzero(fresh)[0]:
@@ -204,16 +228,66 @@ class Engine:
                 bt = wider
                 for i in np.nonzero(fresh)[0]:
                     blk = int(positions[i]) // page
-                    bt[i, blk] = cache.block_table(entries[i].rid, g)[blk]
+                    bt[i, blk] = cache.block_table(rids[i], g)[blk]
                     sm[i] = bt[i, blk] * page
             tables.append(bt)
             slots.append(sm)
         return StepLayout(
-            n_tokens=n, n_seqs=n, n_decode=n, row_of_entry=prev.row_of_entry, tokens=tokens, positions=positions,
-            token_seq=prev.token_seq, qo_indptr=prev.qo_indptr, kv_lens=positions + 1, slot_ids=prev.slot_ids,
-            logit_rows=prev.logit_rows, block_tables=tables, slot_mappings=slots, page_size=page, max_q_len=1,
-            max_kv_len=int(positions.max()) + 1,
+            n_tokens=n, n_seqs=n, n_decode=n, row_of_entry=prev.row_of_entry, tokens=np.zeros(n, dtype=np.int32),
+            positions=positions, token_seq=prev.token_seq, qo_indptr=prev.qo_indptr, kv_lens=positions + 1,
+            slot_ids=prev.slot_ids, logit_rows=prev.logit_rows, block_tables=tables, slot_mappings=slots, page_size=page,
+            max_q_len=1, max_kv_len=int(positions.max()) + 1,
         )
+
+    # ------------------------------------------------------------------ one step ahead
+    def prepare_decode(self) -> Optional["PreparedDecode"]:
+        """Call after a decode step, while the GPU is still busy with it: everything of the next
+        decode step of the same requests (one token each, the same wanted places) that does not
+        depend on the tokens is done now, the plan made, its pages taken, the upload buffer filled.
+        ``step_prepared`` then only needs the tokens.  None when there is nothing to prepare: the
+        last step was no decode step, pages are short, a window releases pages, the step's shape has
+        no recorded graph yet.  A preparation that is never used costs nothing but the pages it took
+        early, which their requests keep, and would have taken with the step anyway."""
+        if self.graphs is None or self._windowed or self._last_decode is None:
+            return None
+        rids, wants, prev, epoch = self._last_decode
+        if epoch != self.cache.epoch:
+            return None
+        layout = self._next_decode_layout()
+        if layout is None:
+            return None
+        graph = self.graphs.recorded(layout)
+        if graph is None:
+            return None  # the pages are taken all the same; the step finds them when it is planned
+        graph.pack(layout)
+        return PreparedDecode(rids, wants, prev, layout, graph, self.cache.epoch)
+
+    @torch.inference_mode()
+    def step_prepared(self, prepared: "PreparedDecode", entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """``step(entries)`` by way of what ``prepare_decode`` prepared.  Returns the logits, or
+        None, with nothing run, when the entries are not the step that was prepared (other
+        requests, more tokens, other wanted places) or the preparation is out of date (another step
+        ran, requests came or went): ``step`` then does the whole work."""
+        last = self._last_decode
+        if last is None or last[2] is not prepared.previous or prepared.epoch != self.cache.epoch:
+            return None
+        if len(entries) != len(prepared.rids):
+            return None
+        tokens = prepared.layout.tokens
+        for i, (e, rid, want) in enumerate(zip(entries, prepared.rids, prepared.wants)):
+            if e.rid != rid or len(e.tokens) != 1 or list(e.want) != want:
+                return None
+            if not 0 <= e.tokens[0] < self.vocab_size:
+                return None  # step() says what is wrong with it
+            tokens[i] = e.tokens[0]
+        prepared.graph.set_tokens(tokens)
+        logits = prepared.graph.launch()
+        for rid in prepared.rids:
+            self.cache.advance(rid, 1)
+        self._last_decode = (prepared.rids, prepared.wants, prepared.layout, self.cache.epoch)
+        self.steps_run += 1
+        self.tokens_run += len(prepared.rids)
+        return logits
 
     def plan(self, entries: Sequence[StepEntry]) -> StepLayout:
         """Reserve pages for the step's tokens (all or nothing) and lay the step out."""

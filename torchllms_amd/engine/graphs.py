@@ -57,12 +57,25 @@ class DecodeGraph:
         self.logits = None
         self.replays = 0
 
-    def _load(self, layout: StepLayout) -> None:
+    def pack(self, layout: StepLayout) -> None:
+        """The plan into the pinned buffer.  May run while an earlier replay is still busy on the
+        GPU: that replay reads the device buffer, which only ``_upload`` touches."""
         if self.replays or self.graph is not None:
             self.copied.synchronize()  # the pinned buffer is free again
         pack_into(self.host_np, layout, self.shapes, self.offsets)
+
+    def set_tokens(self, tokens) -> None:
+        """The token ids of an already packed plan (they are the first section of the buffer)."""
+        off = self.offsets[0]
+        self.host_np[off : off + len(tokens)] = tokens
+
+    def _upload(self) -> None:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
+
+    def _load(self, layout: StepLayout) -> None:
+        self.pack(layout)
+        self._upload()
 
     def first_run(self, layout: StepLayout) -> torch.Tensor:
         """Run the step eagerly (this is the step's real execution), then record the same launches."""
@@ -90,7 +103,12 @@ class DecodeGraph:
         return result
 
     def replay(self, layout: StepLayout) -> torch.Tensor:
-        self._load(layout)
+        self.pack(layout)
+        return self.launch()
+
+    def launch(self) -> torch.Tensor:
+        """Upload the packed plan and replay."""
+        self._upload()
         self.graph.replay()
         self.replays += 1
         return self.logits.clone()
@@ -115,10 +133,17 @@ class DecodeGraphs:
         self.seen: Dict[Tuple[int, int, int, bool], int] = {}
         self.pool = None
 
+    def key_of(self, layout: StepLayout) -> Tuple[int, int, int, bool]:
+        return (layout.n_seqs, int(layout.logit_rows.size), context_cap(layout.max_kv_len), layout.decode_uneven)
+
+    def recorded(self, layout: StepLayout):
+        """The recording that would replay this plan, or None."""
+        g = self.graphs.get(self.key_of(layout))
+        return g if g is not None and g.graph is not None else None
+
     def run(self, layout: StepLayout) -> torch.Tensor:
-        cap = context_cap(layout.max_kv_len)
-        uneven = layout.decode_uneven
-        key = (layout.n_seqs, int(layout.logit_rows.size), cap, uneven)
+        key = self.key_of(layout)
+        cap, uneven = key[2], key[3]
         g = self.graphs.get(key)
         if g is not None:
             return g.replay(layout)

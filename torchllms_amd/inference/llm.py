@@ -34,23 +34,45 @@ class GenerationLoop:
     ``(logits, params, steps) -> token ids``; nothing else."""
 
     def __init__(self, engine, sampler, max_num_seqs: int, max_num_batched_tokens: int, max_model_len: int,
-                 prefill_chunk: Optional[int] = None):
+                 prefill_chunk: Optional[int] = None, look_ahead: bool = True):
         from ..engine.scheduler import Scheduler
 
         self.engine = engine
         self.sampler = sampler
+        self.look_ahead = look_ahead
+        self.stats = {"prepared_steps": 0}
         self.scheduler = Scheduler(engine.cache, max_num_seqs, max_num_batched_tokens, max_model_len, prefill_chunk)
 
     def run(self, prompts: Sequence[Sequence[int]], params: Sequence[SamplingParams], on_step=None):
-        """Generate for every prompt; returns the finished ``Request`` objects in input order."""
+        """Generate for every prompt; returns the finished ``Request`` objects in input order.
+
+        While the GPU runs a decode step, an engine that can (``prepare_decode``) prepares the next
+        one for the case that the same requests decode again; the scheduler still decides every
+        step, and the preparation is used only when its plan is that case."""
         sched = self.scheduler
         requests = [sched.add(("gen", id(self), i), p, sp) for i, (p, sp) in enumerate(zip(prompts, params))]
+        prepare = getattr(self.engine, "prepare_decode", None) if self.look_ahead else None
+        launch = getattr(self.sampler, "launch", None)
+        prepared = None
         try:
             while sched.has_work:
                 plan = sched.schedule()
-                logits = self.engine.step(plan.step_entries())
+                entries = plan.step_entries()
+                logits = None
+                if prepared is not None:
+                    logits = self.engine.step_prepared(prepared, entries)  # None: it is another step
+                    self.stats["prepared_steps"] += logits is not None
+                if logits is None:
+                    logits = self.engine.step(entries)
+                prepared = None
                 sampling = [e.request for e in plan.entries if e.samples]
-                tokens = self.sampler(logits, [r.params for r in sampling], [len(r.output) for r in sampling])
+                counters = [len(r.output) for r in sampling]
+                if prepare is not None and launch is not None and _decodes_on(plan):
+                    pending = launch(logits, [r.params for r in sampling], counters)
+                    prepared = prepare()  # the GPU is busy with the step meanwhile
+                    tokens = pending.tolist()
+                else:
+                    tokens = self.sampler(logits, [r.params for r in sampling], counters)
                 sched.update(plan, tokens)
                 if on_step is not None:
                     on_step(plan)
@@ -61,6 +83,14 @@ class GenerationLoop:
                     sched.abort(r)
             raise
         return requests
+
+
+def _decodes_on(plan) -> bool:
+    """Is the plan a decode step after which every request surely decodes again (none reaches its
+    token budget with this step's token; a stop token may still end one)?"""
+    return bool(plan.entries) and all(
+        len(e.tokens) == 1 and e.samples and len(e.request.output) + 1 < e.request.budget for e in plan.entries
+    )
 
 
 class LLM:
@@ -82,12 +112,14 @@ class LLM:
         max_num_batched_tokens: int = 2048,
         tokenizer=None,
         seed: int = 0,
+        look_ahead: bool = True,
     ):
         """``ckpt_paths``: the model folder (config.json + safetensors), or a list whose first
         entry is that folder or a file in it.  ``precision``: "bfloat16" or "float32"; None takes
         config.json's ``torch_dtype``.  ``max_len`` bounds prompt + generated tokens of a request,
         ``max_bsz`` the requests running at once.  ``model_kwargs`` may override ``max_seq_len``
-        (reference: throughput_bench.py:1057-1060)."""
+        (reference: throughput_bench.py:1057-1060).  ``look_ahead``: prepare the next decode step
+        while the GPU runs the current one (the tokens are the same either way)."""
         from ..engine.engine import Engine
         from ..sampling.sampler import Sampler
 
@@ -117,6 +149,7 @@ class LLM:
         self.batched = batched
         self.device = device
         self.seed = seed
+        self.look_ahead = look_ahead
         self.max_num_batched_tokens = max_num_batched_tokens
         self.template: Optional[ChatTemplate] = get_template(template_config)
         if tokenizer is None and (folder / "tokenizer.json").is_file():
@@ -179,9 +212,9 @@ class LLM:
         live = self.max_bsz if not batch_size else min(batch_size, self.max_bsz)
         if not self.batched:
             live = 1
-        loop = GenerationLoop(self.engine, self.sampler, live, self.max_num_batched_tokens, self.max_len)
+        loop = GenerationLoop(self.engine, self.sampler, live, self.max_num_batched_tokens, self.max_len, look_ahead=self.look_ahead)
         finished = loop.run(ids, params)
-        self.last_stats = dict(loop.scheduler.stats)
+        self.last_stats = dict(loop.scheduler.stats, **loop.stats)
         out = []
         for r in finished:
             text = self.tokenizer.decode(r.output) if self.tokenizer is not None else ""

@@ -30,9 +30,15 @@ class Sampler:
         self._counters = None
 
     def __call__(self, logits: torch.Tensor, params: Sequence[SamplingParams], steps: Sequence[int]) -> List[int]:
+        return self.launch(logits, params, steps).tolist()
+
+    def launch(self, logits: torch.Tensor, params: Sequence[SamplingParams], steps: Sequence[int]) -> torch.Tensor:
+        """Queue the sampling behind the step's kernels and return the token ids as a tensor on the
+        device: the host goes on until it asks for them (``.tolist()``), which it has to do before
+        the next call."""
         n = logits.shape[0]
         if n == 0:
-            return []
+            return torch.empty((0,), dtype=torch.int32)
         if len(params) != n or len(steps) != n:
             raise ValueError("one SamplingParams and one step counter per logits row")
         dev = logits.device
@@ -51,7 +57,7 @@ class Sampler:
         self._pinned[:n] = torch.as_tensor([int(s) for s in steps], dtype=torch.int64)
         counters = self._counters[:n]
         counters.copy_(self._pinned[:n], non_blocking=True)
-        return ops.sample(logits, temperature, seeds, counters, top_k).tolist()
+        return ops.sample(logits, temperature, seeds, counters, top_k)
 
 
 def _as_i64(x: int) -> int:
