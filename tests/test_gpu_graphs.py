@@ -132,3 +132,24 @@ def test_prepared_decode_steps_match_plain_steps(tmp_path, dtype):
                 eng.free(r)
         eng.cache.check_invariants()
         assert eng.cache.free_pages() == 160
+
+
+def test_an_engine_of_other_sizes_can_be_built_after_steps_were_recorded(tmp_path):
+    """Building a bfloat16 engine measures its product kernels in recorded graphs; that has to work
+    after another engine has recorded decode steps (torch keeps capture state between graphs, and a
+    capture inside inference mode followed by one outside it is refused)."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    first = Engine.from_folder(make_folder(tmp_path / "a", TINY["A"], seed=1), dtype="bfloat16", page_size=8, num_pages=16, max_seqs=2)
+    first.admit("a")
+    first.step([StepEntry("a", [1, 2, 3], [])])
+    for t in range(6):
+        first.step([StepEntry("a", [4 + t], [0])])
+    assert any(g.graph is not None for g in first.graphs.graphs.values())
+    other = dict(TINY["A"], hidden_size=72, intermediate_size=200, head_dim=16, vocab_size=264)  # sizes no other test has
+    second = Engine.from_folder(make_folder(tmp_path / "b", other, seed=2), dtype="bfloat16", page_size=8, num_pages=16, max_seqs=2)
+    second.admit("b")
+    logits = second.step([StepEntry("b", [5, 6, 7], [2])])
+    assert logits.shape == (1, 264) and bool(torch.isfinite(logits).all())
+    for t in range(4):
+        first.step([StepEntry("a", [20 + t], [0])])  # the first engine's recordings still replay

@@ -957,7 +957,7 @@ def test_tune_linear_measures_the_wide_kernel_from_17_rows_on():
 
 
 # ----------------------------------------------------------------------------- prefill attention (MFMA)
-def _prefill(rows, hq, hkv, dh, page, window=0, seed=0):
+def _prefill(rows, hq, hkv, dh, page, window=0, seed=0, key_groups=1):
     """Run the prefill kernel on a batch: ``rows`` = [(tokens cached after the step, new queries)].
     Returns (got, want): outputs for all new tokens, row after row."""
     torch.manual_seed(seed)
@@ -984,10 +984,10 @@ def _prefill(rows, hq, hkv, dh, page, window=0, seed=0):
     n = qo[-1]
     wide = torch.cat([torch.cat(qs), torch.randn(n, 2 * hkv * dh).bfloat16()], dim=1).to(DEV)
     qpt = ops.prefill_queries_per_tile(hq, hkv, dh)
-    trow, tq0 = ops.prefill_tiles(qo, 0, len(rows), qpt, kv, window, hkv)  # in the balanced order the engine uses
+    trow, tq0 = ops.prefill_tiles(qo, 0, len(rows), qpt, kv, window, hkv, key_groups)  # in the balanced order the engine uses
     out = torch.zeros(n, hq * dh, dtype=torch.bfloat16, device=DEV)
     ops.attention_prefill(wide, hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32(qo), _i32(kv), _i32(tables), _i32(trow), _i32(tq0),
-                          window, dh ** -0.5, out)
+                          window, dh ** -0.5, out, key_groups=key_groups)
     return out.float().cpu(), torch.cat(wants)
 
 
@@ -1005,14 +1005,18 @@ def _prefill(rows, hq, hkv, dh, page, window=0, seed=0):
         (2, 2, 64, 16, [(1, 1), (2, 2), (17, 16)]),
     ],
 )
-def test_attention_prefill(hq, hkv, dh, page, rows):
-    got, want = _prefill(rows, hq, hkv, dh, page)
+@pytest.mark.parametrize("key_groups", [1, 2])
+def test_attention_prefill(hq, hkv, dh, page, rows, key_groups):
+    """``key_groups`` = 2: two sets of waves per block take every second tile of keys each and add
+    up at the end; a row of fewer keys than two tiles leaves the second set without any."""
+    got, want = _prefill(rows, hq, hkv, dh, page, key_groups=key_groups)
     torch.testing.assert_close(got, want, rtol=2 ** -6, atol=2 ** -6)
 
 
+@pytest.mark.parametrize("key_groups", [1, 2])
 @pytest.mark.parametrize("window", [1, 7, 64, 100])
-def test_attention_prefill_window(window):
-    got, want = _prefill([(260, 260), (300, 40)], 4, 2, 64, 8, window=window)
+def test_attention_prefill_window(window, key_groups):
+    got, want = _prefill([(260, 260), (300, 40)], 4, 2, 64, 8, window=window, key_groups=key_groups)
     torch.testing.assert_close(got, want, rtol=2 ** -6, atol=2 ** -6)
 
 
@@ -1033,9 +1037,10 @@ def test_attention_prefill_sharp_scores_find_the_right_key():
         k_pages, v_pages, table = _paged(k, v, page, n_pages, dtype=torch.bfloat16)
         qpt = ops.prefill_queries_per_tile(hq, hkv, dh)
         trow, tq0 = ops.prefill_tiles([0, S], 0, 1, qpt)
-        out = torch.zeros(S, hq * dh, dtype=torch.bfloat16, device=DEV)
-        ops.attention_prefill(q.reshape(S, hq * dh).to(DEV), hq, hkv, dh, k_pages, v_pages, _i32([0, S]), _i32([S]), _i32([table]),
-                              _i32(trow), _i32(tq0), 0, dh ** -0.5, out)
         want = v[tgt].float().repeat_interleave(hq // hkv, dim=1).reshape(S, hq * dh)
-        err = (out.float().cpu() - want).abs().amax(dim=1)
-        assert err.max().item() < 3e-2, f"distance {dist}: first bad query {int((err >= 3e-2).nonzero()[0])}"
+        for key_groups in (1, 2):
+            out = torch.zeros(S, hq * dh, dtype=torch.bfloat16, device=DEV)
+            ops.attention_prefill(q.reshape(S, hq * dh).to(DEV), hq, hkv, dh, k_pages, v_pages, _i32([0, S]), _i32([S]), _i32([table]),
+                                  _i32(trow), _i32(tq0), 0, dh ** -0.5, out, key_groups=key_groups)
+            err = (out.float().cpu() - want).abs().amax(dim=1)
+            assert err.max().item() < 3e-2, f"distance {dist}, {key_groups} key groups: first bad query {int((err >= 3e-2).nonzero()[0])}"

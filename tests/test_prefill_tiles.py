@@ -3,7 +3,13 @@ tokens, ordered so that the launch is balanced."""
 
 import random
 
-from torchllms_amd.kernels.ops import PREFILL_RESIDENT_BLOCKS, prefill_tiles
+from torchllms_amd.kernels.ops import (
+    PREFILL_RESIDENT_BLOCKS,
+    PREFILL_SPLIT_BLOCKS,
+    prefill_key_groups,
+    prefill_tile_count,
+    prefill_tiles,
+)
 
 
 def _cost(row, q0, qo, kv, qpt, window):
@@ -26,9 +32,10 @@ def test_tiles_are_a_partition_whatever_the_order():
             qo.append(qo[-1] + q)
         qpt = rng.choice([8, 16, 32, 128])
         window = rng.choice([0, 0, 7, 100])
-        rows, q0s = prefill_tiles(qo, first, n_rows, qpt, kv, window, rng.choice([1, 8]))
+        rows, q0s = prefill_tiles(qo, first, n_rows, qpt, kv, window, rng.choice([1, 8]), rng.choice([1, 2]))
         want = sorted((r, q0) for r in range(first, n_rows) for q0 in range(0, q_lens[r], qpt))
         assert sorted(zip(rows, q0s)) == want
+        assert prefill_tile_count(qo, first, n_rows, qpt) == len(want)
         plain_rows, plain_q0s = prefill_tiles(qo, first, n_rows, qpt)  # without lengths: in natural order
         assert list(zip(plain_rows, plain_q0s)) == want
 
@@ -51,3 +58,14 @@ def test_a_long_launch_starts_its_longest_tiles_first():
     costs = [_cost(r, q, qo, kv, qpt, 0) for r, q in zip(rows, q0s)]
     assert costs == sorted(costs, reverse=True)
     assert rows[0] == 1 and rows[-1] == 1 and 0 in rows  # the short row's tiles lie where their length puts them
+
+
+def test_two_sets_of_waves_for_launches_that_fit_at_once_and_then_longest_first():
+    qo, kv, qpt, heads = [0, 2048], [2048], 32, 8
+    n = prefill_tile_count(qo, 0, 1, qpt)
+    assert n * heads <= PREFILL_SPLIT_BLOCKS and prefill_key_groups(n, heads) == 2
+    rows, q0s = prefill_tiles(qo, 0, 1, qpt, kv, 0, heads, key_groups=2)
+    costs = [_cost(r, q, qo, kv, qpt, 0) for r, q in zip(rows, q0s)]
+    assert costs == sorted(costs, reverse=True)
+    assert prefill_key_groups(prefill_tile_count([0, 8192], 0, 1, qpt), heads) == 1
+    assert prefill_key_groups(PREFILL_SPLIT_BLOCKS // heads + 1, heads) == 1

@@ -50,8 +50,7 @@ static_assert(DH == 32 || DH == 64 || DH == 128 || DH == 256, "prefill kernel: h
 typedef short short4_t __attribute__((ext_vector_type(4)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 4;
-constexpr int kThreads = kWaves * kWave;
+constexpr int kWaves = 4;                   // waves that share the columns of a block
 constexpr int NC = DH <= 128 ? 2 : 1;        // MFMA column blocks per wave
 constexpr int kCols = kWaves * NC * 16;      // columns per block
 constexpr int KT = DH <= 128 ? 64 : 32;       // keys per LDS tile
@@ -109,6 +108,21 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(float2_t{a, b}, bf16x2_t));
 }
 
+// Target builtins that the kernel's own body uses stand in device functions: the host pass, which
+// only needs the kernel's stub, does not know them.
+__device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ void wait_for_loads() { __builtin_amdgcn_s_waitcnt(0); }
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// The block's LDS: [group][buffer][keys | values][kTileElems].  It is declared here and not in the
+// kernel: a __shared__ array whose size depends on a template parameter of the kernel itself keeps
+// this compiler from emitting the kernel's host stub.
+template <int GROUPS>
+__device__ __forceinline__ bf16_t* tile_memory() {
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[GROUPS * 2 * 2 * kTileElems];
+  return tiles;
+}
+
 // W consecutive 32-bit words from LDS (W = 1, 2, 4 or 8)
 template <int W>
 __device__ __forceinline__ void lds_words(const bf16_t* src, uint32_t* dst) {
@@ -129,15 +143,19 @@ __device__ __forceinline__ void lds_words(const bf16_t* src, uint32_t* dst) {
 }
 
 // RP: query heads per kv head, rounded up to a power of two.  WINDOWED: whether queries have a lower
-// bound on the keys they see; without one the test against it is compiled out.
-template <int RP, bool WINDOWED>
-__global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a) {
-  __shared__ __attribute__((aligned(16))) bf16_t tiles[2][2][kTileElems];  // [buffer][keys | values]
+// bound on the keys they see; without one the test against it is compiled out.  GROUPS: 1, or 2 sets
+// of kWaves waves that take the same columns and every second tile of keys each, and add up what
+// they have at the end through LDS: a block's chain of tiles is half as long, which is what a launch
+// needs whose blocks all fit the GPU at once and whose time is therefore that of its longest block.
+template <int RP, bool WINDOWED, int GROUPS>
+__global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) attn_prefill_kernel(PrefillArgs a) {
   constexpr int QB = kCols / RP;  // queries per block
 
   const int tile = blockIdx.y;  // the host lists the tiles in the order that balances the launch
   const int kvh = blockIdx.x;
-  const int wave = threadIdx.x / kWave;
+  const int grp = GROUPS == 1 ? 0 : wave_uniform(threadIdx.x / (kWaves * kWave));
+  bf16_t* const tiles = tile_memory<GROUPS>() + grp * 4 * kTileElems;  // this group's [buffer][keys | values]
+  const int wave = (threadIdx.x / kWave) % kWaves;  // within the group
   const int lane = threadIdx.x % kWave;
   const int n16 = lane % 16;
   const int g4 = lane / 16;
@@ -220,12 +238,12 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
       const int blk = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
       const int off = a.page_shift >= 0 ? key & (a.page_size - 1) : key % a.page_size;
       const size_t at = ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH + 8 * piece;
-      __builtin_amdgcn_global_load_lds(a.k_pages + at, &tiles[buffer][0][first * DH], 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(a.v_pages + at, &tiles[buffer][1][first * DH], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(a.k_pages + at, &tiles[(2 * buffer) * kTileElems + first * DH], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(a.v_pages + at, &tiles[(2 * buffer + 1) * kTileElems + first * DH], 16, 0, 0);
     }
   };
 
-  dma(tile_begin, 0);
+  dma(tile_begin + grp * KT, 0);
   int buffer = 0;
   // One tile of keys: wait for it, start the next one's loads, work it off.  `masked`: whether some
   // column may not see some key of the tile; where every column sees every key the tests are
@@ -235,9 +253,9 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
     // has finished with the tile before, whose buffer the next tile's loads may now overwrite
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    dma(base + KT, buffer ^ 1);  // unconditional (keys are clamped): no wait has to cover a path without it
-    const bf16_t* k_lds = tiles[buffer][0];
-    const bf16_t* v_lds = tiles[buffer][1];
+    dma(base + GROUPS * KT, buffer ^ 1);  // unconditional (keys are clamped): no wait has to cover a path without it
+    const bf16_t* k_lds = tiles + (2 * buffer) * kTileElems;
+    const bf16_t* v_lds = tiles + (2 * buffer + 1) * kTileElems;
 
     if (base > wave_hi || base + KT - 1 < wave_lo) return;  // nothing here for this wave's columns
 
@@ -358,11 +376,57 @@ __global__ void __launch_bounds__(kThreads, 2) attn_prefill_kernel(PrefillArgs a
   // columns of the block: they run in a loop of their own, without masks.  The two loops are code
   // one after the other, not two arms of a branch inside one loop, which is what keeps the register
   // count where it was.
-  int base = tile_begin;
+  // Every wave of the block passes the same number of barriers: with two groups both make as many
+  // steps, and the second one's last tile may lie past the last key (then it only waits and loads).
+  const int n_steps = ((key_hi - tile_begin) / KT + GROUPS) / GROUPS;
+  int base = tile_begin + grp * KT;
+  int step = 0;
   if (!WINDOWED) {
-    for (; base + KT - 1 <= pos0 + q0; base += KT, buffer ^= 1) work_tile(base, std::false_type{});
+    for (; step < n_steps && base + KT - 1 <= pos0 + q0; ++step, base += GROUPS * KT, buffer ^= 1)
+      work_tile(base, std::false_type{});
   }
-  for (; base <= key_hi; base += KT, buffer ^= 1) work_tile(base, std::true_type{});
+  for (; step < n_steps; ++step, base += GROUPS * KT, buffer ^= 1) work_tile(base, std::true_type{});
+
+  if constexpr (GROUPS == 2) {
+    // The second group hands its maxima, sums and outputs to the first through the memory of the
+    // tiles (nobody reads a tile any more, and the last, unused load has landed).  Value i of thread
+    // t lies at i * 256 + t: consecutive lanes, consecutive words.
+    constexpr int kPerLane = NC * (2 + 4 * DT);
+    static_assert(kPerLane * kWaves * kWave * sizeof(float) <= GROUPS * 4 * kTileElems * sizeof(bf16_t),
+                  "the tiles' memory is too small for the exchange");
+    float* xch = reinterpret_cast<float*>(tile_memory<GROUPS>()) + (wave * kWave + lane);
+    constexpr int kStride = kWaves * kWave;
+    wait_for_loads();
+    __syncthreads();
+    if (grp == 1) {
+#pragma unroll
+      for (int i = 0; i < NC; ++i) {
+        float* x = xch + i * (2 + 4 * DT) * kStride;
+        x[0] = m_run[i];
+        x[kStride] = l_part[i];
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) x[(2 + 4 * t + r) * kStride] = acc[i][t][r];
+      }
+    }
+    __syncthreads();
+    if (grp == 1) return;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const float* x = xch + i * (2 + 4 * DT) * kStride;
+      const float m_other = x[0];
+      const float m_new = fmaxf(m_run[i], m_other);
+      // a group that has met no visible key of a column has maximum -inf and nothing to add
+      const float mine = m_run[i] == -INFINITY ? 0.f : exp2_fast(m_run[i] - m_new);
+      const float other = m_other == -INFINITY ? 0.f : exp2_fast(m_other - m_new);
+      l_part[i] = l_part[i] * mine + x[kStride] * other;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[i][t][r] = acc[i][t][r] * mine + x[(2 + 4 * t + r) * kStride] * other;
+    }
+  }
 
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
@@ -407,7 +471,7 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
                               const void* v_pages, const int32_t* qo_indptr, const int32_t* kv_lens,
                               const int32_t* block_table, int bt_stride, const int32_t* tile_row,
                               const int32_t* tile_q0, int n_tiles, int n_q_heads, int n_kv_heads, int head_dim,
-                              int page_size, int window, float scale, hipStream_t stream) {
+                              int page_size, int window, float scale, int key_groups, hipStream_t stream) {
   if (head_dim != DH) return variant_fail(TL_ERR_ARG, "attn_prefill: built for head_dim %d, called with %d", DH, head_dim);
   if (n_tiles < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || page_size <= 0 || bt_stride <= 0 || window < 0)
     return variant_fail(TL_ERR_ARG, "attn_prefill: bad sizes");
@@ -419,6 +483,7 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   if (!(scale > 0.f)) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: softmax scale %g must be positive", (double)scale);
   if (q_stride % 8 || ((uintptr_t)q % 16) || out_stride % 8 || ((uintptr_t)out % 16))
     return variant_fail(TL_ERR_ARG, "attn_prefill: queries and outputs need 16-byte aligned rows");
+  if (key_groups != 1 && key_groups != 2) return variant_fail(TL_ERR_ARG, "attn_prefill: key_groups must be 1 or 2, got %d", key_groups);
   if (n_tiles == 0) return TL_OK;
   PrefillArgs a;
   a.q = (const bf16_t*)q; a.q_stride = q_stride; a.out = (bf16_t*)out; a.out_stride = out_stride;
@@ -432,10 +497,16 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   a.scale_log2e = scale * 1.4426950408889634f;
   dim3 grid(n_kv_heads, n_tiles);  // consecutive blocks share a query tile: their loads of q overlap
   const bool windowed = window > 0;
-#define TL_PREFILL_LAUNCH(rp)                                                      \
-  do {                                                                             \
-    if (windowed) attn_prefill_kernel<rp, true><<<grid, kThreads, 0, stream>>>(a);  \
-    else attn_prefill_kernel<rp, false><<<grid, kThreads, 0, stream>>>(a);          \
+  const int threads = kWaves * kWave;
+#define TL_PREFILL_LAUNCH(rp)                                                                      \
+  do {                                                                                             \
+    if (key_groups == 2) {                                                                         \
+      if (windowed) attn_prefill_kernel<rp, true, 2><<<grid, 2 * threads, 0, stream>>>(a);         \
+      else attn_prefill_kernel<rp, false, 2><<<grid, 2 * threads, 0, stream>>>(a);                 \
+    } else {                                                                                       \
+      if (windowed) attn_prefill_kernel<rp, true, 1><<<grid, threads, 0, stream>>>(a);             \
+      else attn_prefill_kernel<rp, false, 1><<<grid, threads, 0, stream>>>(a);                     \
+    }                                                                                              \
   } while (0)
   if (R == 1) TL_PREFILL_LAUNCH(1);
   else if (R == 2) TL_PREFILL_LAUNCH(2);

@@ -77,8 +77,11 @@ class DecodeGraph:
         self.pack(layout)
         self._upload()
 
+    @torch.inference_mode()
     def first_run(self, layout: StepLayout) -> torch.Tensor:
-        """Run the step eagerly (this is the step's real execution), then record the same launches."""
+        """Run the step eagerly (this is the step's real execution), then record the same launches.
+        In inference mode whoever calls: so is every other capture of this package (see
+        ``ops.tune_linear`` for why they must agree)."""
         self._load(layout)
         ctx = make_context(layout, self.dev, self.shapes, self.offsets, decode_longest=self.cap, decode_uneven=self.uneven)
         logits = self.model.forward(ctx, self.cache)

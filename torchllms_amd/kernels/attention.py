@@ -64,13 +64,15 @@ def paged_attention(
             key = ("prefill_tiles", qpt, window, n_kv_heads)
             tiles = ctx.scratch.get(key)
             if tiles is None:
-                rows, q0s = ops.prefill_tiles(ctx.host.qo_indptr, n_dec, ctx.host.n_seqs, qpt, ctx.host.kv_lens, window, n_kv_heads)
+                host = ctx.host
+                key_groups = ops.prefill_key_groups(ops.prefill_tile_count(host.qo_indptr, n_dec, host.n_seqs, qpt), n_kv_heads)
+                rows, q0s = ops.prefill_tiles(host.qo_indptr, n_dec, host.n_seqs, qpt, host.kv_lens, window, n_kv_heads, key_groups)
                 both = torch.tensor([rows, q0s], dtype=torch.int32).to(qkv.device)
-                tiles = (both[0], both[1])
+                tiles = (both[0], both[1], key_groups)
                 ctx.scratch[key] = tiles
             ops.attention_prefill(
                 qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.qo_indptr, ctx.kv_lens,
-                ctx.block_tables[group], tiles[0], tiles[1], window, scale, out,
+                ctx.block_tables[group], tiles[0], tiles[1], window, scale, out, key_groups=tiles[2],
             )
         else:
             ops.attention_generic(

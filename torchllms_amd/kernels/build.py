@@ -190,7 +190,7 @@ register_variant("attn_decode", "attention_decode.hip", "TL_HEAD_DIM")
 register_variant("attn_prefill", "attention_prefill.hip", "TL_HEAD_DIM")
 
 #: sizes compiled ahead of time by ``build_all`` (tests, the smoke run and the benchmark use these)
-PREBUILT_VARIANTS: Dict[str, Iterable[int]] = {"attn_decode": (32, 64, 128), "attn_prefill": (32, 64, 128)}
+PREBUILT_VARIANTS: Dict[str, Iterable[int]] = {"attn_decode": (32, 64, 128, 256), "attn_prefill": (32, 64, 128, 256)}
 
 
 def build_all(force: bool = False) -> List[Path]:

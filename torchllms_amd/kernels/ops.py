@@ -557,6 +557,11 @@ def linear_choice(x: torch.Tensor, w: torch.Tensor, use: str = "plain"):
 _TUNE_FLUSH_BYTES = 512 << 20  # twice the 256 MB of last-level cache
 
 
+# In inference mode like the engine's steps: torch keeps the random generator's capture state in
+# tensors that live as long as any graph does and are updated in place at every capture; were they
+# made by a step's capture (inference tensors), a later capture outside inference mode would be
+# refused, so every capture of this package runs inside it.
+@torch.inference_mode()
 def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "plain", iters: int = 8, report=None) -> None:
     """Measure, for matrices of one shape and every row bucket, which bfloat16 kernel and launch is
     fastest on this GPU, and remember it.  ``weights``: the model's tensors of that shape; ``use``:
@@ -919,7 +924,7 @@ def attention_decode(
 
 # ----------------------------------------------------------------------------- prefill attention (bfloat16, MFMA)
 _PREFILL_SIGNATURES = {
-    "tl_attn_prefill": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "tl_attn_prefill": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
 }
 PREFILL_HEAD_DIMS = (32, 64, 128, 256)
 
@@ -941,10 +946,25 @@ def prefill_queries_per_tile(n_q_heads: int, n_kv_heads: int, head_dim: int) -> 
 
 #: blocks of the prefill kernel that the GPU holds at once: 256 CUs, two blocks each
 PREFILL_RESIDENT_BLOCKS = 512
+#: launches of up to this many blocks run with two sets of waves per block (measured at head size
+#: 128: 512 blocks 87 -> 72 us, 1,024 blocks even, 2,048 blocks 800 -> 890 us)
+PREFILL_SPLIT_BLOCKS = 768
+
+
+def prefill_key_groups(n_tiles: int, n_kv_heads: int) -> int:
+    """Sets of waves per block of the prefill kernel.  A launch whose blocks all fit the GPU at once
+    takes as long as its longest block; with two sets of waves, each with every second tile of keys,
+    that block's chain is half as long.  A launch of many more blocks keeps the CUs busy anyway, and
+    there two independent blocks on a CU overlap better than two sets of waves in step."""
+    return 2 if n_tiles * n_kv_heads <= PREFILL_SPLIT_BLOCKS else 1
+
+
+def prefill_tile_count(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int) -> int:
+    return sum(-(-(int(qo_indptr[r + 1]) - int(qo_indptr[r])) // queries_per_tile) for r in range(first_row, n_rows))
 
 
 def prefill_tiles(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int, kv_lens=None, window: int = 0,
-                  n_kv_heads: int = 1):
+                  n_kv_heads: int = 1, key_groups: int = 1):
     """Host lists ``(tile_row, tile_q0)`` that cut rows ``first_row .. n_rows-1`` into query tiles.
 
     With ``kv_lens`` the tiles are put in the order that balances the launch: a tile's cost is the
@@ -952,7 +972,8 @@ def prefill_tiles(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int,
     Blocks are handed to the CUs in launch order.  When there are far more blocks than fit at once,
     longest first lets short ones fill the gaps at the end; when about all fit at once, the first
     half of the launch takes the long tiles in descending order and the second half the short ones in
-    ascending order, so that the blocks that meet on a CU have complementary lengths."""
+    ascending order, so that the blocks that meet on a CU have complementary lengths.  With two sets
+    of waves a block (``key_groups`` = 2) a CU holds one block at a time: longest first."""
     rows, q0s, costs = [], [], []
     for r in range(first_row, n_rows):
         q_len = int(qo_indptr[r + 1]) - int(qo_indptr[r])
@@ -966,7 +987,7 @@ def prefill_tiles(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int,
     if kv_lens is None or len(rows) < 2:
         return rows, q0s
     order = sorted(range(len(rows)), key=lambda i: -costs[i])
-    if len(rows) * n_kv_heads <= 2 * PREFILL_RESIDENT_BLOCKS:
+    if key_groups == 1 and len(rows) * n_kv_heads <= 2 * PREFILL_RESIDENT_BLOCKS:
         half = (len(order) + 1) // 2
         order = order[:half] + order[half:][::-1]
     return [rows[i] for i in order], [q0s[i] for i in order]
@@ -987,9 +1008,11 @@ def attention_prefill(
     window: int,
     scale: float,
     out: torch.Tensor,
+    key_groups: int = 1,
 ) -> torch.Tensor:
     """Causal attention of the rows named by the tile lists (see ``prefill_tiles``) with the MFMA
-    prefill kernel.  Token t of ``qkv`` / ``out`` is token t of ``qo_indptr``'s numbering."""
+    prefill kernel.  Token t of ``qkv`` / ``out`` is token t of ``qo_indptr``'s numbering.
+    ``key_groups`` = 2: two sets of waves per block share a tile's keys between them."""
     _gpu(qkv, k_pages, v_pages, qo_indptr, kv_lens, block_table, tile_row, tile_q0, out)
     for t, what in ((qo_indptr, "qo_indptr"), (kv_lens, "kv_lens"), (tile_row, "tile_row"), (tile_q0, "tile_q0")):
         _i32(t, what)
@@ -1015,7 +1038,7 @@ def attention_prefill(
             qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
             qo_indptr.data_ptr(), kv_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
             tile_row.data_ptr(), tile_q0.data_ptr(), tile_row.numel(), n_q_heads, n_kv_heads, head_dim, page_size,
-            window, float(scale), _stream(),
+            window, float(scale), int(key_groups), _stream(),
         ),
         lib,
         "tl_variant_last_error",
