@@ -296,57 +296,63 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
   }
 }
 
-// Merge of the splits: one wave per (token, query head); lane -> channels.
+// Merge of the splits: one wave per (token, query head); lane -> channels.  The kernel runs between
+// two large ones, where every load misses all caches, and is as long as its chain of dependent loads:
+// so the token's position, the statistics of the first 64 splits (lane s: split s) and the outputs of
+// the first eight are all asked for at the top, before anything is known about how many splits are
+// valid (every slot of the workspace exists; what an invalid one holds is not used).  Each output
+// still adds its splits in ascending order.
 __global__ void __launch_bounds__(kWave) attn_decode_merge_kernel(DecodeArgs a, int n_q_heads) {
+  constexpr int NC = (DH + kWave - 1) / kWave;
+  constexpr int kAhead = 8;  // splits whose outputs are in flight together
   const int t = blockIdx.x;
   const int qh = blockIdx.y;
   const int lane = threadIdx.x;
-  const int p = a.positions[t];
-  const int lo = (a.window > 0 && p - a.window + 1 > 0) ? p - a.window + 1 : 0;
-  const int lo_al = lo & ~(kTile - 1);
-  const int n_valid = min((p - lo_al) / a.split_size + 1, a.n_splits);
   const size_t slot0 = ((size_t)t * n_q_heads + qh) * a.n_splits;
-  // lane s (and s + 64, ...) reads the statistics of split s; the maximum is reduced over the wave
-  float M = -INFINITY;
-  for (int s = lane; s < n_valid; s += kWave) M = fmaxf(M, a.ws_ml[(slot0 + s) * 2]);
-  M = wave_max(M);
-  float L = 0.f;
-  for (int s = lane; s < n_valid; s += kWave)
-    L += a.ws_ml[(slot0 + s) * 2 + 1] * __builtin_amdgcn_exp2f(a.ws_ml[(slot0 + s) * 2] - M);
-  L = wave_sum(L);
-  constexpr int NC = (DH + kWave - 1) / kWave;
-  float o[NC];
+  const int p = a.positions[t];
+  const int mine = min(lane, a.n_splits - 1);
+  const float m_mine = a.ws_ml[(slot0 + mine) * 2];
+  const float l_mine = a.ws_ml[(slot0 + mine) * 2 + 1];
+  float v[kAhead][NC];
+  auto fetch = [&](int first) {
 #pragma unroll
-  for (int c = 0; c < NC; ++c) o[c] = 0.f;
-  int s = 0;
-  for (; s + 4 <= n_valid; s += 4) {  // four splits' loads in flight at a time
-    float f[4], v[4][NC];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      f[u] = a.ws_ml[(slot0 + s + u) * 2];
+    for (int u = 0; u < kAhead; ++u) {
+      const size_t at = (slot0 + min(first + u, a.n_splits - 1)) * DH;
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const int d = lane + c * kWave;
-        v[u][c] = d < DH ? a.ws_o[(slot0 + s + u) * DH + d] : 0.f;
+        v[u][c] = a.ws_o[at + (d < DH ? d : 0)];
       }
     }
+  };
+  fetch(0);
+  const int lo = (a.window > 0 && p - a.window + 1 > 0) ? p - a.window + 1 : 0;
+  const int lo_al = lo & ~(kTile - 1);
+  const int n_valid = min((p - lo_al) / a.split_size + 1, a.n_splits);
+  float M = lane < n_valid ? m_mine : -INFINITY;
+  for (int s = lane + kWave; s < n_valid; s += kWave) M = fmaxf(M, a.ws_ml[(slot0 + s) * 2]);
+  M = wave_max(M);
+  float L = lane < n_valid ? l_mine * __builtin_amdgcn_exp2f(m_mine - M) : 0.f;
+  for (int s = lane + kWave; s < n_valid; s += kWave)
+    L += a.ws_ml[(slot0 + s) * 2 + 1] * __builtin_amdgcn_exp2f(a.ws_ml[(slot0 + s) * 2] - M);
+  L = wave_sum(L);
+  float o[NC];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const float w = __builtin_amdgcn_exp2f(f[u] - M);
+  for (int c = 0; c < NC; ++c) o[c] = 0.f;
+  for (int s = 0; s < n_valid; s += kAhead) {
+    if (s > 0) fetch(s);
 #pragma unroll
-      for (int c = 0; c < NC; ++c) o[c] += v[u][c] * w;
+    for (int u = 0; u < kAhead; ++u) {
+      const int split = s + u;
+      // the split's maximum: from the lane that holds it, or from memory past the first 64
+      const float m_u = split < kWave ? __shfl(m_mine, split, kWave) : a.ws_ml[(slot0 + min(split, a.n_splits - 1)) * 2];
+      const float w = split < n_valid ? __builtin_amdgcn_exp2f(m_u - M) : 0.f;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) o[c] += split < n_valid ? v[u][c] * w : 0.f;
     }
   }
-  for (; s < n_valid; ++s) {
-    const float w = __builtin_amdgcn_exp2f(a.ws_ml[(slot0 + s) * 2] - M);
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      const int d = lane + c * kWave;
-      if (d < DH) o[c] += a.ws_o[(slot0 + s) * DH + d] * w;
-    }
-  }
-#pragma unroll
-  for (int c = 0; c < (DH + kWave - 1) / kWave; ++c) {
+  for (int c = 0; c < NC; ++c) {
     const int d = lane + c * kWave;
     if (d < DH) a.out[(size_t)t * a.out_stride + (size_t)qh * DH + d] = from_f32<bf16_t>(o[c] / L);
   }

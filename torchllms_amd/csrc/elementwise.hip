@@ -95,51 +95,63 @@ rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ delta, const int32
 }
 
 // Fast path: rows whose length is a multiple of the 16-byte vector and at most kNormThreads * 4 vectors
-// long are read with 16-byte loads and kept in registers between the two passes.
-template <typename T, typename WT>
+// long are read with 16-byte loads and kept in registers between the two passes.  NV = vectors per
+// thread.  Between two large kernels every load here misses all caches, so the kernel's time is its
+// chain of dependent loads: everything it will need (row, delta and the weight) is asked for at the
+// top, without a branch in between, and waited for once.
+template <typename T, int VEC>
+struct alignas(16) NormVec {
+  T e[VEC];
+};
+
+template <typename T, typename WT, int NV>
 __global__ void __launch_bounds__(kNormThreads)
 rmsnorm_vec_kernel(const T* __restrict__ x, const T* __restrict__ delta, const int32_t* __restrict__ rows,
                    const WT* __restrict__ weight, T* __restrict__ h_out, T* __restrict__ y, int hidden,
                    float eps) {
   constexpr int VEC = 16 / sizeof(T);
-  constexpr int MAXV = 4;
+  typedef NormVec<T, VEC> V;
+  typedef NormVec<WT, VEC> W;
   __shared__ float scratch[kNormThreads / kWave];
   const int r = blockIdx.x;
   const size_t s = rows ? (size_t)rows[r] : (size_t)r;
   const int n_vec = hidden / VEC;
-  const uint4* xr = reinterpret_cast<const uint4*>(x + s * hidden);
-  const uint4* dr = delta ? reinterpret_cast<const uint4*>(delta + s * hidden) : nullptr;
-  union V { uint4 u; T e[VEC]; };
-  float v[MAXV][VEC];
-  V xin[MAXV], din[MAXV];
+  const V* xr = reinterpret_cast<const V*>(x + s * hidden);
+  const V* dr = reinterpret_cast<const V*>(delta ? delta + s * hidden : x + s * hidden);
+  const W* wr = reinterpret_cast<const W*>(weight);
+  int at[NV];   // a thread past the row's end reads the last vector again and uses nothing of it
 #pragma unroll
-  for (int it = 0; it < MAXV; ++it) {
-    const int c = threadIdx.x + it * kNormThreads;
-    if (c < n_vec) {
-      xin[it].u = xr[c];
-      if (dr) din[it].u = dr[c];
-    }
-  }
+  for (int it = 0; it < NV; ++it) at[it] = min(threadIdx.x + it * kNormThreads, n_vec - 1);
+  V xin[NV], din[NV];
+  W win[NV];
+#pragma unroll
+  for (int it = 0; it < NV; ++it) xin[it] = xr[at[it]];
+#pragma unroll
+  for (int it = 0; it < NV; ++it) din[it] = dr[at[it]];
+#pragma unroll
+  for (int it = 0; it < NV; ++it) win[it] = wr[at[it]];
+  const bool add = delta != nullptr;
+  float v[NV][VEC];
   float ss = 0.f;
 #pragma unroll
-  for (int it = 0; it < MAXV; ++it) {
-    const int c = threadIdx.x + it * kNormThreads;
-    if (c < n_vec) {
+  for (int it = 0; it < NV; ++it) {
+    const bool live = threadIdx.x + it * kNormThreads < n_vec;
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) {
-        float f = to_f32(xin[it].e[e]);
-        if (dr) f = to_f32(from_f32<T>(f + to_f32(din[it].e[e])));
-        v[it][e] = f;
-        ss += f * f;
-      }
+    for (int e = 0; e < VEC; ++e) {
+      float f = to_f32(xin[it].e[e]);
+      const float sum = to_f32(from_f32<T>(f + to_f32(din[it].e[e])));
+      f = add ? sum : f;
+      f = live ? f : 0.f;
+      v[it][e] = f;
+      ss += f * f;
     }
   }
   ss = block_sum<kNormThreads / kWave>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
-  uint4* yr = reinterpret_cast<uint4*>(y + (size_t)r * hidden);
-  uint4* hr = h_out ? reinterpret_cast<uint4*>(h_out + (size_t)r * hidden) : nullptr;
+  V* yr = reinterpret_cast<V*>(y + (size_t)r * hidden);
+  V* hr = h_out ? reinterpret_cast<V*>(h_out + (size_t)r * hidden) : nullptr;
 #pragma unroll
-  for (int it = 0; it < MAXV; ++it) {
+  for (int it = 0; it < NV; ++it) {
     const int c = threadIdx.x + it * kNormThreads;
     if (c < n_vec) {
       V out, hs;
@@ -147,12 +159,26 @@ rmsnorm_vec_kernel(const T* __restrict__ x, const T* __restrict__ delta, const i
       for (int e = 0; e < VEC; ++e) {
         hs.e[e] = from_f32<T>(v[it][e]);
         const float n = to_f32(from_f32<T>(v[it][e] * inv));
-        out.e[e] = from_f32<T>(n * to_f32(weight[c * VEC + e]));
+        out.e[e] = from_f32<T>(n * to_f32(win[it].e[e]));
       }
-      yr[c] = out.u;
-      if (hr) hr[c] = hs.u;
+      yr[c] = out;
+      if (hr) hr[c] = hs;
     }
   }
+}
+
+template <typename T, typename WT>
+static void launch_rmsnorm_vec(const void* x, const void* delta, const int32_t* rows, const void* weight, void* h_out, void* y,
+                               int n_rows, int hidden, float eps, hipStream_t stream) {
+  const int per_thread = (hidden / (16 / (int)sizeof(T)) + kNormThreads - 1) / kNormThreads;
+#define TL_NORM_VEC(NV)                                                                                          \
+  rmsnorm_vec_kernel<T, WT, NV><<<n_rows, kNormThreads, 0, stream>>>((const T*)x, (const T*)delta, rows, (const WT*)weight, \
+                                                                     (T*)h_out, (T*)y, hidden, eps)
+  if (per_thread <= 1) TL_NORM_VEC(1);
+  else if (per_thread == 2) TL_NORM_VEC(2);
+  else if (per_thread == 3) TL_NORM_VEC(3);
+  else TL_NORM_VEC(4);
+#undef TL_NORM_VEC
 }
 
 TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, const void* weight,
@@ -165,17 +191,14 @@ TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, 
   const size_t lds = (size_t)hidden * sizeof(float);
   const int vec = dtype == TL_F32 ? 4 : 8;
   const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0) && (!delta || (uintptr_t)delta % 16 == 0) &&
-                       (!h_out || (uintptr_t)h_out % 16 == 0);
+                       (!h_out || (uintptr_t)h_out % 16 == 0) && ((uintptr_t)weight % 16 == 0);
   if (hidden % vec == 0 && hidden / vec <= kNormThreads * 4 && aligned) {
     if (dtype == TL_F32 && weight_dtype == TL_F32)
-      rmsnorm_vec_kernel<float, float><<<n_rows, kNormThreads, 0, stream>>>(
-          (const float*)x, (const float*)delta, rows, (const float*)weight, (float*)h_out, (float*)y, hidden, eps);
+      launch_rmsnorm_vec<float, float>(x, delta, rows, weight, h_out, y, n_rows, hidden, eps, stream);
     else if (dtype == TL_BF16 && weight_dtype == TL_BF16)
-      rmsnorm_vec_kernel<bf16_t, bf16_t><<<n_rows, kNormThreads, 0, stream>>>(
-          (const bf16_t*)x, (const bf16_t*)delta, rows, (const bf16_t*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps);
+      launch_rmsnorm_vec<bf16_t, bf16_t>(x, delta, rows, weight, h_out, y, n_rows, hidden, eps, stream);
     else if (dtype == TL_BF16 && weight_dtype == TL_F32)
-      rmsnorm_vec_kernel<bf16_t, float><<<n_rows, kNormThreads, 0, stream>>>(
-          (const bf16_t*)x, (const bf16_t*)delta, rows, (const float*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps);
+      launch_rmsnorm_vec<bf16_t, float>(x, delta, rows, weight, h_out, y, n_rows, hidden, eps, stream);
     else
       return tl_fail(TL_ERR_ARG, "rmsnorm: unsupported dtypes x=%d weight=%d", dtype, weight_dtype);
     return tl_check_launch("rmsnorm");
@@ -206,48 +229,81 @@ TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, 
 // (partial[s][row][i], s = 0 .. splits - 1): they are added in the order of the splits and rounded
 // to bfloat16, as the kernel that would otherwise finish the product does, and then the row goes the
 // way of rmsnorm_vec_kernel.  One launch instead of two.
-template <typename WT>
+template <typename WT, int NV>
 __global__ void __launch_bounds__(kNormThreads)
 rmsnorm_split_kernel(const bf16_t* __restrict__ x, const float* __restrict__ partial, int splits, size_t split_stride,
                      const int32_t* __restrict__ rows, const WT* __restrict__ weight, bf16_t* __restrict__ h_out,
                      bf16_t* __restrict__ y, int hidden, float eps) {
   constexpr int VEC = 8;
-  constexpr int MAXV = 4;
+  typedef NormVec<bf16_t, VEC> V;
+  typedef NormVec<WT, VEC> W;
+  typedef NormVec<float, VEC> P;
   __shared__ float scratch[kNormThreads / kWave];
   const int r = blockIdx.x;
   const size_t s = rows ? (size_t)rows[r] : (size_t)r;
   const int n_vec = hidden / VEC;
-  const uint4* xr = reinterpret_cast<const uint4*>(x + s * hidden);
-  const float4* pr = reinterpret_cast<const float4*>(partial + s * hidden);
-  union V { uint4 u; bf16_t e[VEC]; };
-  float v[MAXV][VEC];
-  float ss = 0.f;
+  const V* xr = reinterpret_cast<const V*>(x + s * hidden);
+  const P* pr = reinterpret_cast<const P*>(partial + s * hidden);
+  const W* wr = reinterpret_cast<const W*>(weight);
+  const size_t step = split_stride / VEC;
+  int at[NV];
 #pragma unroll
-  for (int it = 0; it < MAXV; ++it) {
-    const int c = threadIdx.x + it * kNormThreads;
-    if (c < n_vec) {
-      V xin;
-      xin.u = xr[c];
-      float d[VEC] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      for (int k = 0; k < splits; ++k) {
-        const float4 lo = pr[k * (split_stride / 4) + 2 * c], hi = pr[k * (split_stride / 4) + 2 * c + 1];
-        d[0] += lo.x; d[1] += lo.y; d[2] += lo.z; d[3] += lo.w;
-        d[4] += hi.x; d[5] += hi.y; d[6] += hi.z; d[7] += hi.w;
-      }
+  for (int it = 0; it < NV; ++it) at[it] = min(threadIdx.x + it * kNormThreads, n_vec - 1);
+  // row, weight and the first two splits are asked for together; further splits two at a time.  Each
+  // element still adds its splits in their order.
+  V xin[NV];
+  W win[NV];
+  P first[NV], second[NV];
+#pragma unroll
+  for (int it = 0; it < NV; ++it) xin[it] = xr[at[it]];
+#pragma unroll
+  for (int it = 0; it < NV; ++it) first[it] = pr[at[it]];
+  const size_t one = splits > 1 ? step : 0;
+#pragma unroll
+  for (int it = 0; it < NV; ++it) second[it] = pr[one + at[it]];
+#pragma unroll
+  for (int it = 0; it < NV; ++it) win[it] = wr[at[it]];
+  float d[NV][VEC];
+#pragma unroll
+  for (int it = 0; it < NV; ++it)
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      d[it][e] = 0.f + first[it].e[e];
+      if (splits > 1) d[it][e] += second[it].e[e];
+    }
+  for (int k = 2; k < splits; k += 2) {
+    const size_t next = k + 1 < splits ? step : 0;
+#pragma unroll
+    for (int it = 0; it < NV; ++it) first[it] = pr[k * step + at[it]];
+#pragma unroll
+    for (int it = 0; it < NV; ++it) second[it] = pr[k * step + next + at[it]];
+#pragma unroll
+    for (int it = 0; it < NV; ++it)
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
-        const float f = to_f32(from_f32<bf16_t>(to_f32(xin.e[e]) + to_f32(from_f32<bf16_t>(d[e]))));
-        v[it][e] = f;
-        ss += f * f;
+        d[it][e] += first[it].e[e];
+        if (k + 1 < splits) d[it][e] += second[it].e[e];
       }
+  }
+  float v[NV][VEC];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < NV; ++it) {
+    const bool live = threadIdx.x + it * kNormThreads < n_vec;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      float f = to_f32(from_f32<bf16_t>(to_f32(xin[it].e[e]) + to_f32(from_f32<bf16_t>(d[it][e]))));
+      f = live ? f : 0.f;
+      v[it][e] = f;
+      ss += f * f;
     }
   }
   ss = block_sum<kNormThreads / kWave>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
-  uint4* yr = reinterpret_cast<uint4*>(y + (size_t)r * hidden);
-  uint4* hr = h_out ? reinterpret_cast<uint4*>(h_out + (size_t)r * hidden) : nullptr;
+  V* yr = reinterpret_cast<V*>(y + (size_t)r * hidden);
+  V* hr = h_out ? reinterpret_cast<V*>(h_out + (size_t)r * hidden) : nullptr;
 #pragma unroll
-  for (int it = 0; it < MAXV; ++it) {
+  for (int it = 0; it < NV; ++it) {
     const int c = threadIdx.x + it * kNormThreads;
     if (c < n_vec) {
       V out, hs;
@@ -255,16 +311,30 @@ rmsnorm_split_kernel(const bf16_t* __restrict__ x, const float* __restrict__ par
       for (int e = 0; e < VEC; ++e) {
         hs.e[e] = from_f32<bf16_t>(v[it][e]);
         const float n = to_f32(from_f32<bf16_t>(v[it][e] * inv));
-        out.e[e] = from_f32<bf16_t>(n * to_f32(weight[c * VEC + e]));
+        out.e[e] = from_f32<bf16_t>(n * to_f32(win[it].e[e]));
       }
-      yr[c] = out.u;
-      if (hr) hr[c] = hs.u;
+      yr[c] = out;
+      if (hr) hr[c] = hs;
     }
   }
 }
 
+template <typename WT>
+static void launch_rmsnorm_split(const void* x, const float* partial, int splits, size_t split_stride, const int32_t* rows,
+                                 const void* weight, void* h_out, void* y, int n_rows, int hidden, float eps, hipStream_t stream) {
+  const int per_thread = (hidden / 8 + kNormThreads - 1) / kNormThreads;
+#define TL_NORM_SPLIT(NV)                                                                                                \
+  rmsnorm_split_kernel<WT, NV><<<n_rows, kNormThreads, 0, stream>>>((const bf16_t*)x, partial, splits, split_stride, rows, \
+                                                                    (const WT*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps)
+  if (per_thread <= 1) TL_NORM_SPLIT(1);
+  else if (per_thread == 2) TL_NORM_SPLIT(2);
+  else if (per_thread == 3) TL_NORM_SPLIT(3);
+  else TL_NORM_SPLIT(4);
+#undef TL_NORM_SPLIT
+}
+
 // RMS norm of x + sum of the splits, bfloat16 x / h_out / y [.., hidden]; partial: 32-bit, split s of
-// row r at partial + s * split_stride + r * hidden (split_stride in elements, a multiple of 4).
+// row r at partial + s * split_stride + r * hidden (split_stride in elements, a multiple of 8).
 // hidden must be a multiple of 8 and at most 8 * 4 * 256.
 TL_EXPORT int tl_rmsnorm_split(const void* x, const float* partial, int splits, int64_t split_stride, const int32_t* rows,
                                const void* weight, int weight_dtype, void* h_out, void* y, int n_rows, int hidden,
@@ -273,16 +343,14 @@ TL_EXPORT int tl_rmsnorm_split(const void* x, const float* partial, int splits, 
   TL_REQUIRE(!(rows && h_out), "rmsnorm_split: h_out cannot be combined with a row gather");
   if (hidden % 8 != 0 || hidden / 8 > kNormThreads * 4)
     return tl_fail(TL_ERR_UNSUPPORTED, "rmsnorm_split: hidden=%d must be a multiple of 8 and at most %d", hidden, 8 * 4 * kNormThreads);
-  TL_REQUIRE(split_stride % 4 == 0 && ((uintptr_t)partial % 16) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
-                 (!h_out || (uintptr_t)h_out % 16 == 0),
-             "rmsnorm_split: tensors must start on 16-byte boundaries");
+  TL_REQUIRE(split_stride % 8 == 0 && ((uintptr_t)partial % 16) == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
+                 (!h_out || (uintptr_t)h_out % 16 == 0) && ((uintptr_t)weight % 16) == 0,
+             "rmsnorm_split: tensors must start on 16-byte boundaries and splits lie a multiple of 8 elements apart");
   if (n_rows == 0) return TL_OK;
   if (weight_dtype == TL_BF16)
-    rmsnorm_split_kernel<bf16_t><<<n_rows, kNormThreads, 0, stream>>>((const bf16_t*)x, partial, splits, (size_t)split_stride, rows,
-                                                                      (const bf16_t*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps);
+    launch_rmsnorm_split<bf16_t>(x, partial, splits, (size_t)split_stride, rows, weight, h_out, y, n_rows, hidden, eps, stream);
   else if (weight_dtype == TL_F32)
-    rmsnorm_split_kernel<float><<<n_rows, kNormThreads, 0, stream>>>((const bf16_t*)x, partial, splits, (size_t)split_stride, rows,
-                                                                     (const float*)weight, (bf16_t*)h_out, (bf16_t*)y, hidden, eps);
+    launch_rmsnorm_split<float>(x, partial, splits, (size_t)split_stride, rows, weight, h_out, y, n_rows, hidden, eps, stream);
   else
     return tl_fail(TL_ERR_ARG, "rmsnorm_split: unsupported weight dtype %d", weight_dtype);
   return tl_check_launch("rmsnorm_split");

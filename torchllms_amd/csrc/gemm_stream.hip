@@ -98,6 +98,11 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
 #pragma unroll
   for (int t = 0; t < NW; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
+  // what the query/key/value epilogue reads from memory is asked for now and has long arrived when
+  // the walk along K ends (asked for at the end, it would be one more round trip to memory)
+  QkvOperands qkv_operands = {};
+  if constexpr (EPI == kQkv) qkv_operands = qkv_fetch(min(n16, M - 1), n0 + 4 * g4, qa);
+
   auto fetch = [&](int st, u32x4_t* w, u32x4_t* a) {
     const int k0 = st * kStepK;
 #pragma unroll
@@ -203,7 +208,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     const int n = n0 + 4 * g4;
     if (n16 < M && n < N) {
       const float sums[4] = {acc[0][0], acc[0][1], acc[0][2], acc[0][3]};
-      qkv_finish(sums, n16, n, qa, reinterpret_cast<bf16_t*>(C), ldc);
+      qkv_finish(sums, n16, n, qa, reinterpret_cast<bf16_t*>(C), ldc, qkv_operands);
     }
   } else if constexpr (HALF) {
     // lanes with g4 < 2 hold the gate sums of columns n0 + 4 g4 + i, the lanes 32 further on the up

@@ -219,7 +219,11 @@ gemm_wide_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
   }
 }
 
-// C[m][n] = sum over the splits, in their order, of partial[s][m][n].
+// C[m][n] = sum over the splits, in their order, of partial[s][m][n].  These kernels run between two
+// large ones and every load of theirs misses the caches: the splits are asked for several at a time
+// (a split past the last is the last once more, and not added), not one after the other.
+constexpr int kReduceAhead = 8;
+
 template <typename OutT>
 __global__ void __launch_bounds__(256) gemm_wide_reduce_kernel(const float* __restrict__ partial, OutT* __restrict__ C,
                                                                int ldc, int M, int N, int splits) {
@@ -227,7 +231,13 @@ __global__ void __launch_bounds__(256) gemm_wide_reduce_kernel(const float* __re
   const size_t total = (size_t)M * N;
   if (idx >= total) return;
   float sum = 0.f;
-  for (int s = 0; s < splits; ++s) sum += partial[s * total + idx];
+  for (int s = 0; s < splits; s += kReduceAhead) {
+    float part[kReduceAhead];
+#pragma unroll
+    for (int u = 0; u < kReduceAhead; ++u) part[u] = partial[(size_t)min(s + u, splits - 1) * total + idx];
+#pragma unroll
+    for (int u = 0; u < kReduceAhead; ++u) sum = s + u < splits ? sum + part[u] : sum;
+  }
   C[(idx / N) * ldc + idx % N] = from_f32<OutT>(sum);
 }
 
@@ -241,10 +251,18 @@ __global__ void __launch_bounds__(256) gemm_wide_reduce_qkv_kernel(const float* 
   const int m = (int)(idx / quads);
   const int n = 4 * (int)(idx % quads);
   const size_t total = (size_t)M * N;
+  const float* mine = partial + (size_t)m * N + n;
+  const QkvOperands operands = qkv_fetch(m, n, qa);
   float4_t sum = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < splits; ++s) sum += *reinterpret_cast<const float4_t*>(partial + s * total + (size_t)m * N + n);
+  for (int s = 0; s < splits; s += kReduceAhead) {
+    float4_t part[kReduceAhead];
+#pragma unroll
+    for (int u = 0; u < kReduceAhead; ++u) part[u] = *reinterpret_cast<const float4_t*>(mine + (size_t)min(s + u, splits - 1) * total);
+#pragma unroll
+    for (int u = 0; u < kReduceAhead; ++u) sum = s + u < splits ? sum + part[u] : sum;
+  }
   const float sums[4] = {sum[0], sum[1], sum[2], sum[3]};
-  qkv_finish(sums, m, n, qa, C, ldc);
+  qkv_finish(sums, m, n, qa, C, ldc, operands);
 }
 
 struct Launch {

@@ -15,12 +15,35 @@ struct QkvArgs {
   int page_size;
 };
 
+// What the epilogue reads from memory for one thread's four columns: the cosines and sines of its two
+// rotary pairs and its row's place in the pages.  Fetched apart from the arithmetic so that a kernel
+// can ask for them together with everything else it loads (indices are clamped to what exists; what
+// a thread does not need it does not use).
+struct QkvOperands {
+  float2 cs[2];
+  int slot;
+};
+
+__device__ __forceinline__ QkvOperands qkv_fetch(int row, int n, const QkvArgs& qa) {
+  QkvOperands o;
+  const int half = qa.rotary_dim / 2;
+  const int pair = (n % qa.head_dim) / 2;
+  o.cs[0] = o.cs[1] = float2{1.f, 0.f};
+  if (half > 0) {
+    o.cs[0] = qa.cos_sin[(size_t)row * half + min(pair, half - 1)];
+    o.cs[1] = qa.cos_sin[(size_t)row * half + min(pair + 1, half - 1)];
+  }
+  o.slot = qa.k_pages != nullptr ? qa.slot_mapping[row] : -1;
+  return o;
+}
+
 // sums[0..3]: the 32-bit products of row `row` and columns n .. n + 3, which are channels d .. d + 3
 // of one head (the host checks head_dim % 4 == 0): two rotary pairs (interleaved pairing).  They are
 // rounded to bfloat16 first, as the stored product of the unfused sequence would read, rotated in
 // 32-bit, rounded again and stored: queries into C, keys and values into their pages (or into C when
 // there are no pages).
-__device__ __forceinline__ void qkv_finish(const float* sums, int row, int n, const QkvArgs& qa, bf16_t* C, int ldc) {
+__device__ __forceinline__ void qkv_finish(const float* sums, int row, int n, const QkvArgs& qa, bf16_t* C, int ldc,
+                                           const QkvOperands& o) {
   typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
   const int head = n / qa.head_dim;
   const int d = n % qa.head_dim;
@@ -31,7 +54,7 @@ __device__ __forceinline__ void qkv_finish(const float* sums, int row, int n, co
 #pragma unroll
     for (int pi = 0; pi < 2; ++pi) {
       if (d + 2 * pi < qa.rotary_dim) {
-        const float2 cs = qa.cos_sin[(size_t)row * (qa.rotary_dim / 2) + (d / 2 + pi)];
+        const float2 cs = o.cs[pi];
         const float x0 = x[2 * pi], x1 = x[2 * pi + 1];
         x[2 * pi] = x0 * cs.x - x1 * cs.y;
         x[2 * pi + 1] = x1 * cs.x + x0 * cs.y;
@@ -44,7 +67,7 @@ __device__ __forceinline__ void qkv_finish(const float* sums, int row, int n, co
   bf16_t* dst = C + (size_t)row * ldc + n;
   bool store = true;
   if (head >= qa.n_q_heads && qa.k_pages != nullptr) {
-    const int slot = qa.slot_mapping[row];
+    const int slot = o.slot;
     store = slot >= 0;
     const int kvh = head < qa.n_q_heads + qa.n_kv_heads ? head - qa.n_q_heads : head - qa.n_q_heads - qa.n_kv_heads;
     bf16_t* pages = head < qa.n_q_heads + qa.n_kv_heads ? qa.k_pages : qa.v_pages;
@@ -53,6 +76,10 @@ __device__ __forceinline__ void qkv_finish(const float* sums, int row, int n, co
     dst = pages + (((size_t)page * qa.n_kv_heads + kvh) * qa.page_size + off) * qa.head_dim + d;
   }
   if (store) *reinterpret_cast<u32x2_t*>(dst) = packed;
+}
+
+__device__ __forceinline__ void qkv_finish(const float* sums, int row, int n, const QkvArgs& qa, bf16_t* C, int ldc) {
+  qkv_finish(sums, row, n, qa, C, ldc, qkv_fetch(row, n, qa));
 }
 
 // The argument checks of the entry points that take these arguments; fills `qa`.
