@@ -14,10 +14,9 @@
 //     bytes of a key row are one operand); their output layout, taken over two blocks of 16 keys, is
 //     exactly the B-operand layout of P^T in O^T[channel][column] = V^T P^T, so the probabilities
 //     never leave their registers.  Softmax statistics are 32-bit, per column.
-//   * the A operand of the second product wants, per lane, one channel of eight keys.  A lane reads
-//     from each of its eight key rows the DH/16 consecutive channels (DH/16) * n16 ...; the operand of
-//     output block b is channel b of the eight rows (four byte permutes).  Row m of output block b is
-//     therefore channel (DH/16) * m + b: a renaming that makes a lane's results contiguous in memory.
+//   * the A operand of the second product wants, per lane, one channel of eight keys, while the
+//     values lie in LDS key by key.  gfx950's transposing LDS load (ds_read_b64_tr_b16) hands every
+//     lane one channel of four key rows: two of them are an operand, no permutes.
 //   * every column has its own causal limit (its query's position) and window start.
 //
 // Compiled once per head size (-DTL_HEAD_DIM=32|64|128|256).
@@ -56,7 +55,6 @@ constexpr int kCols = kWaves * NC * 16;      // columns per block
 constexpr int KT = DH <= 128 ? 64 : 32;       // keys per LDS tile
 constexpr int KL = DH / 32;                  // 16-byte pieces of a key row per lane
 constexpr int DT = DH / 16;                  // channel tiles of the output
-constexpr int kVWords = DT / 2;              // 32-bit words a lane reads from one value row (DT channels)
 constexpr int kPieces = DH / 8;              // 16-byte pieces in a key/value row
 constexpr int kRowsPerLoad = kWave / kPieces;  // rows that one wave load (64 lanes x 16 bytes) covers
 constexpr int kLoadsPerWave = KT / kRowsPerLoad / kWaves;  // wave loads per tile and operand
@@ -67,8 +65,13 @@ constexpr int kTileElems = KT * DH;          // one operand's tile in LDS, rows 
 constexpr int kRowsPerSweep = DH >= 128 ? 1 : 128 / DH;
 constexpr int kSwizzle = kPieces < 16 ? kPieces : 16;
 __device__ __forceinline__ int swizzle(int row) { return (row / kRowsPerSweep) % kSwizzle; }
-// element offset of piece `piece` of row `row` within a tile
+// element offset of piece `piece` of row `row` within a tile of keys
 __device__ __forceinline__ int tile_at(int row, int piece) { return row * DH + 8 * (piece ^ swizzle(row)); }
+// Values are read by transposing loads (see below): 16 lanes fetch 32 bytes at the same place of four
+// consecutive rows, and these four have to meet different banks.  Rows of 256 bytes and more start on
+// the same bank, rows of 128 bytes on every second: the pair of pieces moves with the row.
+__device__ __forceinline__ int swizzle_v(int row) { return DH >= 128 ? 2 * (row % 8) : DH == 64 ? 2 * ((row / 2) % 4) : 0; }
+__device__ __forceinline__ int tile_at_v(int row, int piece) { return row * DH + 8 * (piece ^ swizzle_v(row)); }
 
 struct PrefillArgs {
   const bf16_t* q;
@@ -123,23 +126,15 @@ __device__ __forceinline__ bf16_t* tile_memory() {
   return tiles;
 }
 
-// W consecutive 32-bit words from LDS (W = 1, 2, 4 or 8)
-template <int W>
-__device__ __forceinline__ void lds_words(const bf16_t* src, uint32_t* dst) {
-  if constexpr (W == 1) {
-    dst[0] = *reinterpret_cast<const uint32_t*>(src);
-  } else if constexpr (W == 2) {
-    const u32x2_t v = *reinterpret_cast<const u32x2_t*>(src);
-    dst[0] = v[0];
-    dst[1] = v[1];
-  } else {
-#pragma unroll
-    for (int i = 0; i < W / 4; ++i) {
-      const u32x4_t v = *reinterpret_cast<const u32x4_t*>(src + 8 * i);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) dst[4 * i + e] = v[e];
-    }
-  }
+// The transposing LDS load of gfx950 (ds_read_b64_tr_b16).  Each lane names 8 bytes (four 16-bit
+// elements); within every 16 lanes, lane 4a + b receives element b of the lanes a, 4 + a, 8 + a and
+// 12 + a, in this order.  With lane 4j + a pointing at four consecutive channels 4a .. 4a + 3 of key
+// row j, lane m = 4a + b ends up with channel m of four key rows: half an MFMA operand of V^T,
+// straight from values that lie in LDS as they lie in the page.
+typedef short short4v_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x2_t lds_transposed(const bf16_t* src) {
+  typedef short4v_t __attribute__((address_space(3))) * lds_ptr_t;
+  return __builtin_bit_cast(u32x2_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)src));
 }
 
 // RP: query heads per kv head, rounded up to a power of two.  WINDOWED: whether queries have a lower
@@ -232,14 +227,15 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
     for (int j = 0; j < kLoadsPerWave; ++j) {
       const int first = (j * kWaves + wave) * kRowsPerLoad;
       const int r = first + lane / kPieces;
-      const int piece = (lane % kPieces) ^ swizzle(r);
+      const int piece_k = (lane % kPieces) ^ swizzle(r);
+      const int piece_v = (lane % kPieces) ^ swizzle_v(r);
       int key = base + r;
       key = key < key_lo ? key_lo : (key > key_hi ? key_hi : key);
       const int blk = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
       const int off = a.page_shift >= 0 ? key & (a.page_size - 1) : key % a.page_size;
-      const size_t at = ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH + 8 * piece;
-      __builtin_amdgcn_global_load_lds(a.k_pages + at, &tiles[(2 * buffer) * kTileElems + first * DH], 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(a.v_pages + at, &tiles[(2 * buffer + 1) * kTileElems + first * DH], 16, 0, 0);
+      const size_t at = ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH;
+      __builtin_amdgcn_global_load_lds(a.k_pages + at + 8 * piece_k, &tiles[(2 * buffer) * kTileElems + first * DH], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(a.v_pages + at + 8 * piece_v, &tiles[(2 * buffer + 1) * kTileElems + first * DH], 16, 0, 0);
     }
   };
 
@@ -341,31 +337,22 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
       for (int t = 0; t < DT; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha[i];
-    // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column], 32 keys at a time.
-    // A block of 16 keys that no column of the wave sees has zero probabilities: its rows are read
-    // all the same (they lie in the tile) and add nothing.
+    // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column], 32 keys at a time, 16
+    // channels an MFMA.  Its A operand (lane (m, g4): channel 16 t + m of the keys 4 g4 .. + 3 and
+    // 16 + 4 g4 .. + 3, the order in which the probabilities lie in pb) comes from two transposing
+    // loads.  A block of 16 keys that no column of the wave sees has zero probabilities: its rows are
+    // read all the same (they lie in the tile) and add nothing.
+    const int tr_row = 4 * g4 + n16 / 4;  // the key row this lane points at, within 16 keys
+    const int tr_ch = 4 * (n16 % 4);      // the first of its four channels, within 16 channels
 #pragma unroll
     for (int g = 0; g < NS / 2; ++g) {
-      uint32_t vrow[8][kVWords];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int key = 32 * g + 16 * (e / 4) + 4 * g4 + (e % 4);  // within the tile
-        // the lane's DT channels start at channel DT * n16: part of one piece, or two whole pieces
-        if constexpr (kVWords <= 4) {
-          lds_words<kVWords>(&v_lds[tile_at(key, DT * n16 / 8) + DT * n16 % 8], vrow[e]);
-        } else {
-          lds_words<4>(&v_lds[tile_at(key, 2 * n16)], vrow[e]);
-          lds_words<4>(&v_lds[tile_at(key, 2 * n16 + 1)], vrow[e] + 4);
-        }
-      }
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
-        const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;  // the odd or the even halves of two words
-        const u32x4_t vw = {__builtin_amdgcn_perm(vrow[1][t / 2], vrow[0][t / 2], sel),
-                            __builtin_amdgcn_perm(vrow[3][t / 2], vrow[2][t / 2], sel),
-                            __builtin_amdgcn_perm(vrow[5][t / 2], vrow[4][t / 2], sel),
-                            __builtin_amdgcn_perm(vrow[7][t / 2], vrow[6][t / 2], sel)};
-        const bf16x8_t va = __builtin_bit_cast(bf16x8_t, vw);
+        const int r0 = 32 * g + tr_row, r1 = r0 + 16;
+        const int ch = 16 * t + tr_ch;
+        const u32x2_t lo = lds_transposed(&v_lds[tile_at_v(r0, ch / 8) + ch % 8]);
+        const u32x2_t hi = lds_transposed(&v_lds[tile_at_v(r1, ch / 8) + ch % 8]);
+        const bf16x8_t va = __builtin_bit_cast(bf16x8_t, u32x4_t{lo[0], lo[1], hi[0], hi[1]});
 #pragma unroll
         for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[i][g], acc[i][t], 0, 0, 0);
       }
@@ -436,23 +423,11 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
     if (!col_ok[i]) continue;
     const float inv = 1.0f / l;
     bf16_t* orow = a.out + (size_t)col_tok[i] * a.out_stride + (size_t)col_head[i] * DH;
-    // acc[i][t][r] is channel DT * (4 g4 + r) + t: for each r the DT output blocks are contiguous
+    // acc[i][t][r] is channel 16 t + 4 g4 + r: four consecutive channels per output block
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      uint32_t w[kVWords];
-#pragma unroll
-      for (int t = 0; t < DT; t += 2) w[t / 2] = pack_bf16x2(acc[i][t][r] * inv, acc[i][t + 1][r] * inv);
-      bf16_t* dst = orow + DT * (4 * g4 + r);
-      if constexpr (kVWords == 1) {
-        *reinterpret_cast<uint32_t*>(dst) = w[0];
-      } else if constexpr (kVWords == 2) {
-        *reinterpret_cast<u32x2_t*>(dst) = u32x2_t{w[0], w[1]};
-      } else {
-#pragma unroll
-        for (int j = 0; j < kVWords / 4; ++j)
-          *reinterpret_cast<u32x4_t*>(dst + 8 * j) = u32x4_t{w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
-      }
-    }
+    for (int t = 0; t < DT; ++t)
+      *reinterpret_cast<u32x2_t*>(orow + 16 * t + 4 * g4) =
+          u32x2_t{pack_bf16x2(acc[i][t][0] * inv, acc[i][t][1] * inv), pack_bf16x2(acc[i][t][2] * inv, acc[i][t][3] * inv)};
   }
 }
 
