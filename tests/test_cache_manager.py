@@ -5,7 +5,6 @@ reference: torchllms/models/test_paged_kv.py:53-136,303-426."""
 import random
 
 import pytest
-import torch
 
 from torchllms_amd.cache import CacheGroupSpec, CacheManager, OutOfPages, OutOfSlots, PagePool, StateSlotSpec, group_layers
 from torchllms_amd.parts import KVNeed, StateNeed

@@ -1,8 +1,6 @@
 """Each part alone on the GPU against its plain counterpart, and a toy mixer with state of its own
 that is registered, built and stepped without a change to the framework's files."""
 
-from dataclasses import dataclass
-from typing import Dict
 
 import pytest
 import torch

@@ -1,7 +1,6 @@
 """The step's host-side plan (CPU).  Vectors marked (ref) restate
 reference: torchllms/models/test_paged_kv.py:144-186."""
 
-import numpy as np
 import pytest
 
 from torchllms_amd.cache import CacheGroupSpec, CacheManager

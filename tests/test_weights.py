@@ -14,7 +14,6 @@ from torchllms_amd.weights import (
     interleaved_to_half_split,
     load_weights,
     random_tensors,
-    write_model_folder,
 )
 
 from .helpers import TINY_A, TINY_B, TINY_C, make_folder, read_folder
