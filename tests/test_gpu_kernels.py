@@ -585,6 +585,7 @@ def _decode(q, k, v, page, window=0, split_size=None, n_pages=None):
         (32, 8, 128, 16, 2000, None), (32, 8, 128, 16, 2000, 64), (32, 8, 128, 16, 2000, 4096), (8, 1, 32, 16, 300, 64),
         (4, 4, 64, 8, 100, None), (6, 2, 64, 4, 77, 64), (16, 1, 128, 32, 513, 128), (8, 1, 256, 16, 200, 64),
         (5, 5, 32, 12, 130, 64), (6, 3, 128, 1, 65, 64), (2, 2, 64, 16, 1, None), (4, 1, 128, 16, 16, None), (4, 1, 128, 16, 17, None),
+        (4, 1, 128, 16, 5000, 64), (2, 1, 64, 16, 4500, 64),  # more than 64 splits: the merge reads statistics past its first wave of lanes
     ],
 )
 def test_attention_decode(hq, hkv, dh, page, S, split):
@@ -867,7 +868,8 @@ def test_gemm_wide_takes_strided_rows_and_says_its_limits():
         _ops().gemm_wide(x, w, torch.float32, 1, 1, 4)
 
 
-@pytest.mark.parametrize("m, n, k, splits", [(64, 4096, 1024, 4), (20, 2048, 512, 8), (33, 72, 384, 2), (17, 8192, 256, 3)])
+@pytest.mark.parametrize("m, n, k, splits", [(64, 4096, 1024, 4), (20, 2048, 512, 8), (33, 72, 384, 2), (17, 8192, 256, 3), (18, 264, 128, 1),
+                                           (19, 520, 1408, 11)])
 @pytest.mark.parametrize("weight_dtype", [torch.bfloat16, torch.float32])
 def test_rmsnorm_adds_up_a_split_product_as_the_reduce_kernel_would(m, n, k, splits, weight_dtype):
     """A product left as the sums of its splits, taken as the delta of the norm: bit for bit what
