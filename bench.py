@@ -2,7 +2,7 @@
 bfloat16 weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
-                    [--shape 8b|1b|70b] [--workload decode|serve]
+                    [--shape 8b|1b|70b] [--workload decode|serve|small-kernels]
 
 A step is one decode step of the whole batch: ``Engine.step`` on one token per request followed by
 the sampling kernel and the copy of the chosen tokens to the host, as generation does it.  The
@@ -15,7 +15,10 @@ step's unavoidable reads (every weight once, the live requests' cache) against H
 ``--shape`` takes the layer sizes of Llama-3.2-1B or Llama-3.1-70B instead (the default is the
 headline's 8B).  ``--workload serve`` runs the scheduler instead of fixed batches: 64 requests at
 once, prompts of 128 to 4,096 random tokens, 512 tokens generated for each at temperature 0.7; its
-line reports generated tokens a second over the whole run, prefill included.
+line reports generated tokens a second over the whole run, prefill included.  ``--workload
+small-kernels`` times what a norm kernel adds to a replayed graph of large products, without a
+profiler (under rocprofv3 no dispatch is shorter than about 4.6 us, an empty kernel included, so a
+kernel trace overstates the small kernels of a step).
 """
 
 from __future__ import annotations
@@ -62,7 +65,7 @@ def parse_args(argv=None):
     p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the headline's)")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve"])
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "small-kernels"])
     p.add_argument("--requests", type=int, default=64, help="serve: requests running at once")
     p.add_argument("--new-tokens", type=int, default=512, help="serve: tokens generated for every request")
     p.add_argument("--no-look-ahead", action="store_true", help="plan every decode step when it runs, not during the step before")
@@ -234,6 +237,56 @@ def serve_run(args, shape) -> int:
     return 0
 
 
+def small_kernels_run(args, shape) -> int:
+    """What a small kernel costs between two large ones of a replayed graph: the time of a graph of
+    32 gate/up products of a decode step (each on a matrix of its own turn, caches flushed before
+    every replay), and of the same graph with 1, 2 and 4 norm kernels behind each product."""
+    import torch
+
+    from torchllms_amd.kernels import ops
+
+    dev = "cuda:0"
+    hidden, inter, rows, n = shape["hidden_size"], shape["intermediate_size"], args.batch, 32
+    weights = [torch.randn(2 * inter, hidden, device=dev, dtype=torch.float32).mul_(0.02).to(torch.bfloat16) for _ in range(4)]
+    x = torch.randn(rows, hidden, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    h, delta = torch.randn_like(x), torch.randn_like(x)
+    gain = torch.ones(hidden, device=dev, dtype=torch.bfloat16)
+    flush = torch.zeros(512 << 18, device=dev)
+
+    def graph_us(norms_behind_each: int) -> float:
+        def run():
+            for i in range(n):
+                ops.gemm_stream_glu(x, weights[i % 4], 4, 8)
+                for _ in range(norms_behind_each):
+                    ops.rmsnorm(h, gain, 1e-5, delta=delta, return_sum=True)
+
+        with torch.inference_mode():
+            run()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                run()
+            best = float("inf")
+            for _ in range(7):
+                flush.sum()
+                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                graph.replay()
+                stop.record()
+                stop.synchronize()
+                best = min(best, start.elapsed_time(stop) * 1e3)
+        return best
+
+    base = graph_us(0)
+    added = {k: (graph_us(k) - base) / n / k for k in (1, 2, 4)}
+    print(json.dumps({
+        "metric": "microseconds a norm kernel adds behind a large kernel of a replayed graph", "unit": "us",
+        "rows": rows, "hidden_size": hidden, "product_us": round(base / n, 2),
+        "norm_us": {f"{k}_behind_each": round(v, 2) for k, v in added.items()},
+    }))
+    return 0
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     if args.gpus != 1:
@@ -242,6 +295,8 @@ def main(argv=None) -> int:
     shape = SHAPES[args.shape]
     if args.workload == "serve":
         return serve_run(args, shape)
+    if args.workload == "small-kernels":
+        return small_kernels_run(args, shape)
     import torch
 
     from torchllms_amd.config import LlamaConfig

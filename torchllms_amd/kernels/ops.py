@@ -517,10 +517,12 @@ def wide_fits(rows: int, strips_per_wave: int, stages: int) -> bool:
 #: ``linear_to_sum``) as a term of the residual sum, where the norm that follows adds up a split
 #: product for nothing
 LINEAR_USES = ("plain", "glu", "qkv", "sum")
-#: microseconds that a small kernel between large ones costs in a replayed decode step (measured);
+#: microseconds that a small kernel between large ones costs in a replayed decode step (measured as
+#: the difference between graphs with and without it: 2.7 to 3.1 for a norm of 1 to 64 rows; a kernel
+#: trace shows 4.6 and more for every dispatch, an empty one included, which is the profiler's own);
 #: ``tune_linear`` charges it to a candidate that leaves the second half of a fused use to a kernel
 #: of its own
-_TAIL_KERNEL_US = 4.5
+_TAIL_KERNEL_US = 2.8
 
 
 def _row_bucket(m: int) -> int:
