@@ -1,15 +1,17 @@
 // Causal attention of prompt portions over paged bfloat16 keys and values (the cached prefix and
 // the portion itself, which the step has already written into the pages): the prefill kernel.
 //
-//   * a block of 4 waves takes a tile of consecutive queries of one request and one kv head, with
-//     all query heads that share it: its 128 MFMA columns are (query, head) pairs, so a key or value
-//     is fetched once for the whole group.
+//   * a block takes a tile of consecutive queries of one request and one kv head, with all query
+//     heads that share it: the 128 MFMA columns of its 4 waves are (query, head) pairs, so a key or
+//     value is fetched once for the whole group.  A launch whose blocks all fit the GPU at once is as
+//     long as its longest block; there a block has a second set of 4 waves for the same columns, each
+//     set takes every second tile of keys, and they add up what they have through LDS at the end.
 //   * keys and values stream through LDS in tiles of 64 keys, both as they lie in the page, and get
 //     there without passing through registers: `global_load_lds_dwordx4` puts a wave's 64 x 16 bytes
 //     at consecutive LDS addresses.  Rows are therefore not padded; instead the 16-byte pieces of a
 //     row are stored in an order that depends on the row (piece ^ f(row)), so that the 16 lanes that
-//     read the same piece of 16 rows still meet 16 different banks.  Two buffers: the next tile lands
-//     while the current one is worked off, with one barrier a tile.
+//     read the same piece of 16 rows still meet 16 different banks.  Two buffers per set of waves:
+//     the next tile lands while the current one is worked off, with one barrier a tile.
 //   * scores are computed transposed, S^T[key][column] = K Q^T, by MFMA 16x16x32 bf16 (a lane's 16
 //     bytes of a key row are one operand); their output layout, taken over two blocks of 16 keys, is
 //     exactly the B-operand layout of P^T in O^T[channel][column] = V^T P^T, so the probabilities
