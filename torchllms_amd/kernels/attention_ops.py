@@ -1,0 +1,302 @@
+"""Attention over the paged cache: the plain kernel (any size, both dtypes), the split-KV decode kernel and
+the tiled prefill kernel (bfloat16, MFMA), with the host-side plans of their launches."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .base import (  # noqa: F401
+    BF16,
+    F32,
+    KernelError,
+    SplitSums,
+    _gpu,
+    _i32,
+    _ptr,
+    _stream,
+    check,
+    core,
+    dtype_code,
+    resolved,
+    variant,
+)
+
+
+def attention_generic(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    token_seq: torch.Tensor,
+    positions: torch.Tensor,
+    block_table: torch.Tensor,
+    window: int,
+    scale: float,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Attention of each token's query heads (the first Hq * dh columns of ``qkv``) over the paged
+    keys and values of its request; returns [n, Hq * dh]."""
+    _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
+    _i32(token_seq, "token_seq")
+    _i32(positions, "positions")
+    n = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention: qkv must be row-major with at least Hq * dh columns")
+    if token_seq.numel() != n or positions.numel() != n:
+        raise KernelError("attention: token_seq and positions need one entry per token")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("attention: block_table must be an int32 matrix")
+    page_size = k_pages.shape[2]
+    for pg in (k_pages, v_pages):
+        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+            raise KernelError("attention: pages must be contiguous [pages, Hkv, page_size, dh] of the query's dtype")
+    if out is None:
+        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    check(
+        core().tl_attention_generic(
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
+            n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), dtype_code(qkv.dtype), _stream(),
+        )
+    )
+    return out
+
+
+# ----------------------------------------------------------------------------- decode attention (bfloat16, MFMA)
+_P, _I, _F = __import__("ctypes").c_void_p, __import__("ctypes").c_int, __import__("ctypes").c_float
+_DECODE_SIGNATURES = {
+    "tl_attn_decode": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P],
+}
+DECODE_HEAD_DIMS = (32, 64, 128, 256)
+_DECODE_BLOCK_KEYS = 64  # keys one block pass covers (4 waves x 16): splits are multiples of it
+
+
+def decode_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: int, head_dim: int) -> bool:
+    """Whether the MFMA decode kernel takes these sizes (else the plain kernel runs)."""
+    if dtype != torch.bfloat16 or head_dim not in DECODE_HEAD_DIMS or n_q_heads % n_kv_heads:
+        return False
+    return n_q_heads // n_kv_heads <= (16 if head_dim <= 128 else 8)
+
+
+_DECODE_MIN_SPLIT = 256  # keys: shorter splits cost more in launch and merge than they gain in spread
+
+
+_DECODE_UNEVEN_SPLIT = 1024  # keys: the longest split when requests differ much in length
+
+
+def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, target_blocks: int = 512, uneven: bool = False):
+    """``(split_size, n_splits)`` for a decode launch whose longest visible key range (counted from
+    its 16-aligned start) is ``longest``: enough splits for about two blocks on each of the 256
+    CUs, none shorter than 256 keys.  Measured from one request of 131,072 tokens to 128 requests
+    of 2,048, 512 blocks were the best or within 2% of it: a block's waves keep enough loads in
+    flight by themselves, and every further split costs its start, its partial results and its
+    share of the merge.  A batch with 512 (request, kv head) pairs or more is not split at all,
+    if the requests are about equally long.  (Alone and on pages in random order, 8 requests of
+    8,192 tokens ran a little faster with four splits of 2,048 keys than with eight of 1,024; inside
+    the decode step it was the other way round, 52.9 against 49.5 us, and the step decides.)
+
+    ``uneven``: the requests differ much in length.  Then all blocks of such a launch would be
+    resident at once and stay where they were put, a CU with long requests' blocks working on
+    when its neighbours have finished; with splits of at most 1,024 keys there are several times
+    more blocks than fit, and those that wait go where others end.  (64 requests of 128 to 4,608
+    tokens: 30% less time than unsplit; 64 equal ones: 10% more, hence the switch.)"""
+    pairs = max(n_tokens * n_kv_heads, 1)
+    want = max(-(-target_blocks // pairs), 1)
+    split = -(-max(longest, 1) // want)
+    if uneven:
+        split = min(split, _DECODE_UNEVEN_SPLIT)
+    split = max(-(-split // _DECODE_BLOCK_KEYS) * _DECODE_BLOCK_KEYS, _DECODE_MIN_SPLIT)
+    # splits of 256 keys only while 512 keys would leave fewer than one block for each CU (measured
+    # with cold caches: 2 requests of 8,192 tokens 23.4 against 25.8 us, 8 of 2,048 21.7 against 23.3,
+    # 2 of 4,096, where 512 keys give 128 blocks, 20.0 against 18.4)
+    if split < 2 * _DECODE_MIN_SPLIT and pairs * -(-max(longest, 1) // (2 * _DECODE_MIN_SPLIT)) >= 256:
+        split = 2 * _DECODE_MIN_SPLIT
+    return split, max(-(-max(longest, 1) // split), 1)
+
+
+def attention_decode(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    token_seq: torch.Tensor,
+    positions: torch.Tensor,
+    block_table: torch.Tensor,
+    window: int,
+    scale: float,
+    longest: int,
+    out: Optional[torch.Tensor] = None,
+    split_size: Optional[int] = None,
+    uneven: bool = False,
+) -> torch.Tensor:
+    """Attention of single-token queries over their requests' pages with the split-KV MFMA kernel.
+    ``longest``: an upper bound of any token's visible key range, counted from its 16-aligned first
+    visible key (position + 1 without a window)."""
+    _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
+    _i32(token_seq, "token_seq")
+    _i32(positions, "positions")
+    if qkv.dtype != torch.bfloat16:
+        raise KernelError("attention_decode takes bfloat16")
+    n = token_seq.numel()
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[0] < n or qkv.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention_decode: qkv must be row-major with a row per token and at least Hq * dh columns")
+    if positions.numel() != n:
+        raise KernelError("attention_decode: one position per token")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("attention_decode: block_table must be an int32 matrix")
+    page_size = k_pages.shape[2]
+    for pg in (k_pages, v_pages):
+        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+            raise KernelError("attention_decode: pages must be contiguous [pages, Hkv, page_size, dh] bfloat16")
+    if out is None:
+        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    if split_size is None:
+        split_size, n_splits = plan_decode_splits(n, n_kv_heads, longest, uneven=uneven)
+    else:
+        n_splits = max(-(-max(longest, 1) // split_size), 1)
+    ws_o = ws_ml = None
+    if n_splits > 1:
+        ws_o = torch.empty((n * n_q_heads * n_splits * head_dim,), dtype=torch.float32, device=qkv.device)
+        ws_ml = torch.empty((n * n_q_heads * n_splits * 2,), dtype=torch.float32, device=qkv.device)
+    lib = variant("attn_decode", head_dim, _DECODE_SIGNATURES)
+    check(
+        lib.tl_attn_decode(
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
+            n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), split_size, n_splits,
+            _ptr(ws_o), _ptr(ws_ml), _stream(),
+        ),
+        lib,
+        "tl_variant_last_error",
+    )
+    return out
+
+
+# ----------------------------------------------------------------------------- prefill attention (bfloat16, MFMA)
+_PREFILL_SIGNATURES = {
+    "tl_attn_prefill": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+}
+PREFILL_HEAD_DIMS = (32, 64, 128, 256)
+
+
+def prefill_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: int, head_dim: int) -> bool:
+    """Whether the MFMA prefill kernel takes these sizes (else the plain kernel runs)."""
+    return dtype == torch.bfloat16 and head_dim in PREFILL_HEAD_DIMS and n_q_heads % n_kv_heads == 0 and n_q_heads // n_kv_heads <= 16
+
+
+def prefill_queries_per_tile(n_q_heads: int, n_kv_heads: int, head_dim: int) -> int:
+    """Queries one block of the prefill kernel covers: its MFMA columns (128, or 64 at head size 256)
+    divided by the group size rounded up to a power of two."""
+    group = n_q_heads // n_kv_heads
+    rp = 1
+    while rp < group:
+        rp *= 2
+    return (128 if head_dim <= 128 else 64) // rp
+
+
+#: blocks of the prefill kernel that the GPU holds at once: 256 CUs, two blocks each
+PREFILL_RESIDENT_BLOCKS = 512
+#: launches of up to this many blocks run with two sets of waves per block (measured at head size
+#: 128: 512 blocks 87 -> 72 us, 1,024 blocks even, 2,048 blocks 800 -> 890 us)
+PREFILL_SPLIT_BLOCKS = 768
+
+
+def prefill_key_groups(n_tiles: int, n_kv_heads: int) -> int:
+    """Sets of waves per block of the prefill kernel.  A launch whose blocks all fit the GPU at once
+    takes as long as its longest block; with two sets of waves, each with every second tile of keys,
+    that block's chain is half as long.  A launch of many more blocks keeps the CUs busy anyway, and
+    there two independent blocks on a CU overlap better than two sets of waves in step."""
+    return 2 if n_tiles * n_kv_heads <= PREFILL_SPLIT_BLOCKS else 1
+
+
+def prefill_tile_count(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int) -> int:
+    return sum(-(-(int(qo_indptr[r + 1]) - int(qo_indptr[r])) // queries_per_tile) for r in range(first_row, n_rows))
+
+
+def prefill_tiles(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int, kv_lens=None, window: int = 0,
+                  n_kv_heads: int = 1, key_groups: int = 1):
+    """Host lists ``(tile_row, tile_q0)`` that cut rows ``first_row .. n_rows-1`` into query tiles.
+
+    With ``kv_lens`` the tiles are put in the order that balances the launch: a tile's cost is the
+    number of keys it sees, and late tiles of a causal prompt see many times more than early ones.
+    Blocks are handed to the CUs in launch order.  When there are far more blocks than fit at once,
+    longest first lets short ones fill the gaps at the end; when about all fit at once, the first
+    half of the launch takes the long tiles in descending order and the second half the short ones in
+    ascending order, so that the blocks that meet on a CU have complementary lengths.  With two sets
+    of waves a block (``key_groups`` = 2) a CU holds one block at a time: longest first."""
+    rows, q0s, costs = [], [], []
+    for r in range(first_row, n_rows):
+        q_len = int(qo_indptr[r + 1]) - int(qo_indptr[r])
+        pos0 = (int(kv_lens[r]) - q_len) if kv_lens is not None else 0
+        for q0 in range(0, q_len, queries_per_tile):
+            rows.append(r)
+            q0s.append(q0)
+            hi = pos0 + min(q0 + queries_per_tile, q_len) - 1
+            lo = max(pos0 + q0 - window + 1, 0) if window > 0 else 0
+            costs.append(hi - lo + 1)
+    if kv_lens is None or len(rows) < 2:
+        return rows, q0s
+    order = sorted(range(len(rows)), key=lambda i: -costs[i])
+    if key_groups == 1 and len(rows) * n_kv_heads <= 2 * PREFILL_RESIDENT_BLOCKS:
+        half = (len(order) + 1) // 2
+        order = order[:half] + order[half:][::-1]
+    return [rows[i] for i in order], [q0s[i] for i in order]
+
+
+def attention_prefill(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    qo_indptr: torch.Tensor,
+    kv_lens: torch.Tensor,
+    block_table: torch.Tensor,
+    tile_row: torch.Tensor,
+    tile_q0: torch.Tensor,
+    window: int,
+    scale: float,
+    out: torch.Tensor,
+    key_groups: int = 1,
+) -> torch.Tensor:
+    """Causal attention of the rows named by the tile lists (see ``prefill_tiles``) with the MFMA
+    prefill kernel.  Token t of ``qkv`` / ``out`` is token t of ``qo_indptr``'s numbering.
+    ``key_groups`` = 2: two sets of waves per block share a tile's keys between them."""
+    _gpu(qkv, k_pages, v_pages, qo_indptr, kv_lens, block_table, tile_row, tile_q0, out)
+    for t, what in ((qo_indptr, "qo_indptr"), (kv_lens, "kv_lens"), (tile_row, "tile_row"), (tile_q0, "tile_q0")):
+        _i32(t, what)
+    if qkv.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise KernelError("attention_prefill takes bfloat16")
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention_prefill: qkv must be row-major with at least Hq * dh columns")
+    if out.dim() != 2 or out.stride(1) != 1 or out.shape[0] != qkv.shape[0] or out.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention_prefill: out must be row-major [tokens, >= Hq * dh]")
+    if tile_row.numel() != tile_q0.numel():
+        raise KernelError("attention_prefill: tile lists differ in length")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("attention_prefill: block_table must be an int32 matrix")
+    if kv_lens.numel() != block_table.shape[0] or qo_indptr.numel() != kv_lens.numel() + 1:
+        raise KernelError("attention_prefill: qo_indptr, kv_lens and block_table disagree about the rows")
+    page_size = k_pages.shape[2]
+    for pg in (k_pages, v_pages):
+        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+            raise KernelError("attention_prefill: pages must be contiguous [pages, Hkv, page_size, dh] bfloat16")
+    lib = variant("attn_prefill", head_dim, _PREFILL_SIGNATURES)
+    check(
+        lib.tl_attn_prefill(
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            qo_indptr.data_ptr(), kv_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+            tile_row.data_ptr(), tile_q0.data_ptr(), tile_row.numel(), n_q_heads, n_kv_heads, head_dim, page_size,
+            window, float(scale), int(key_groups), _stream(),
+        ),
+        lib,
+        "tl_variant_last_error",
+    )
+    return out
