@@ -6,7 +6,7 @@ import pytest
 import torch
 from safetensors.torch import save_file
 
-from torchllms_amd.config import LlamaConfig, get_architecture
+from torchllms_amd.config import LlamaConfig, get_architecture, load_config
 from torchllms_amd.parts import Model
 from torchllms_amd.weights import (
     WeightError,
@@ -176,3 +176,27 @@ def test_sharded_folder_and_missing_files(tmp_path):
     empty.mkdir()
     with pytest.raises(FileNotFoundError, match="no safetensors"):
         _load(empty, TINY_A)
+
+
+def test_random_weights_mode_from_the_command_line(tmp_path):
+    """``python -m torchllms_amd.weights.random_init``: a folder from a config.json and a seed; the
+    same seed gives the same tensors, the loader takes the folder back without complaint."""
+    from safetensors import safe_open
+
+    from torchllms_amd.weights import random_init
+
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(TINY_B))
+    for out in ("a", "b"):
+        assert random_init.main(["--config", str(cfg_path), "--seed", "7", "--out", str(tmp_path / out)]) == 0
+    assert json.loads((tmp_path / "a" / "config.json").read_text())["hidden_size"] == TINY_B["hidden_size"]
+    with safe_open(str(tmp_path / "a" / "model.safetensors"), framework="pt") as fa, \
+            safe_open(str(tmp_path / "b" / "model.safetensors"), framework="pt") as fb:
+        assert sorted(fa.keys()) == sorted(fb.keys()) and "model.embed_tokens.weight" in fa.keys()
+        for name in fa.keys():
+            assert torch.equal(fa.get_tensor(name), fb.get_tensor(name))
+            assert fa.get_tensor(name).dtype == torch.bfloat16
+    arch, config = load_config(tmp_path / "a")
+    expected = Model(arch.model_spec(config)).param_specs()
+    tensors = load_weights(tmp_path / "a", arch.weight_rules(config), expected, torch.bfloat16)
+    assert set(tensors) == set(expected)

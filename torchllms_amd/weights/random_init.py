@@ -89,3 +89,39 @@ def write_model_folder(
     config.save(folder)
     save_file(tensors, str(folder / "model.safetensors"), metadata={"format": "pt"})
     return folder
+
+
+def main(argv=None) -> int:
+    """``python -m torchllms_amd.weights.random_init --config config.json --seed 0 --out DIR``:
+    the random-weights mode from the command line.  The architecture named in the configuration
+    picks the model, as everywhere."""
+    import argparse
+    import json
+
+    p = argparse.ArgumentParser(prog="python -m torchllms_amd.weights.random_init", description=main.__doc__)
+    p.add_argument("--config", required=True, help="a config.json (or a model folder that holds one)")
+    p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--out", required=True, help="folder that receives config.json and model.safetensors")
+    p.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"], help="dtype of the stored tensors")
+    p.add_argument("--norm-jitter", type=float, default=0.0, help="norm weights are 1 + N(0, this) instead of 1")
+    args = p.parse_args(argv)
+    path = Path(args.config)
+    if path.is_dir():
+        path = path / "config.json"
+    with open(path) as f:
+        raw = json.load(f)
+    names = raw.get("architectures") or []
+    if not names:
+        raise SystemExit(f"{path} names no architecture (key \"architectures\")")
+    arch = get_architecture(names[0])
+    config = arch.config_from_dict(raw)
+    dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    folder = write_model_folder(args.out, config, args.seed, dtype=dtype, norm_jitter=args.norm_jitter, arch=arch)
+    print(f"wrote {folder / 'config.json'} and {folder / 'model.safetensors'} (seed {args.seed}, {args.dtype})")
+    return 0
+
+
+if __name__ == "__main__":
+    import sys
+
+    sys.exit(main())
