@@ -15,7 +15,7 @@ def test_decode_splits_cover_the_range_with_about_512_blocks():
                     assert split % 64 == 0 and split >= 256
                     assert n_splits >= 1 and (n_splits - 1) * split < max(longest, 1) <= n_splits * split
                     if uneven:
-                        assert split <= 1024
+                        assert split <= ops._DECODE_UNEVEN_SPLIT == 512
                     elif n_splits > 1:
                         # no more blocks than asked for, unless the shortest split allowed is reached
                         assert split == 256 or n_tokens * n_kv_heads * n_splits <= 512 + n_tokens * n_kv_heads
