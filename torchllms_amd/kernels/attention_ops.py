@@ -203,8 +203,9 @@ def prefill_queries_per_tile(n_q_heads: int, n_kv_heads: int, head_dim: int) -> 
 #: blocks of the prefill kernel that the GPU holds at once: 256 CUs, two blocks each
 PREFILL_RESIDENT_BLOCKS = 512
 #: launches of up to this many blocks run with two sets of waves per block (measured at head size
-#: 128: 512 blocks 87 -> 72 us, 1,024 blocks even, 2,048 blocks 800 -> 890 us)
-PREFILL_SPLIT_BLOCKS = 768
+#: 128 with cold caches: 512 blocks 87 -> 72 us, 1,024 blocks 270 -> 257 us, 1,280 blocks 361 -> 391 us;
+#: at head size 64 the two are even at 768 and 1,024 blocks and one set wins from 1,280 on)
+PREFILL_SPLIT_BLOCKS = 1024
 
 
 def prefill_key_groups(n_tiles: int, n_kv_heads: int) -> int:
