@@ -1,6 +1,7 @@
 // C[M, N] = A[M, K] * W[N, K]^T in true 32-bit: float inputs, float FMA accumulation, no matrix-core
 // reduced-precision mode.  Each output element is accumulated by one thread over k = 0..K-1 in
-// ascending order, so its value does not depend on M or on where the row sits in the batch.
+// ascending order (in groups of 16 that are added up first), so its value does not depend on M or on
+// where the row sits in the batch.
 // Throughput is secondary: this is the matrix product of the 32-bit path.
 #include "common.h"
 
@@ -41,6 +42,15 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
       }
     }
     __syncthreads();
+    // the BK products of this step are added among themselves first and then to the running sum:
+    // the rounding error of a long sum grows with the number of additions to one accumulator, and
+    // this way there are K / BK + BK of them instead of K (at K = 1024 the 32-bit model's distance
+    // from a 64-bit computation halves); the order is still fixed by K alone
+    float part[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) part[i][j] = 0.f;
 #pragma unroll
     for (int k = 0; k < BK; ++k) {
       float a[TM], w[TN];
@@ -51,8 +61,12 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        for (int j = 0; j < TN; ++j) part[i][j] = fmaf(a[i], w[j], part[i][j]);
     }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] += part[i][j];
     __syncthreads();
   }
 #pragma unroll
