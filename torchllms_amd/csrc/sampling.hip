@@ -8,6 +8,9 @@
 // q_i comes from a counter-based generator (Philox 4x32-10) keyed by the row's seed; the counter is
 // (i / 4, step), so a row's draw depends on its own seed and step only, never on the batch.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 namespace {
 
@@ -276,6 +279,18 @@ TL_EXPORT int tl_sample(const float* logits, int row_stride, int n_rows, int voc
   return tl_check_launch("sample");
 }
 
+// Both kernels of the choice in pieces; `candidates` holds n_rows * used entries.
+static int launch_sample_chunks(const float* logits, int row_stride, int n_rows, int vocab, const float* temperature,
+                                const uint64_t* seeds, const uint64_t* steps, int chunk_len, int used, Best* candidates,
+                                int32_t* out, hipStream_t stream) {
+  sample_chunks_kernel<<<dim3(used, n_rows), kThreads, 0, stream>>>(logits, row_stride, vocab, temperature, seeds, steps,
+                                                                   chunk_len, candidates);
+  int rc = tl_check_launch("sample_chunks");
+  if (rc != TL_OK) return rc;
+  sample_pick_kernel<<<n_rows, kWave, 0, stream>>>(candidates, used, out);
+  return tl_check_launch("sample_pick");
+}
+
 // The same choice without top-k, every row cut into `chunks` pieces that blocks of their own work
 // on: for few rows of a large vocabulary, where one block per row leaves most of the GPU idle.
 // candidates: workspace of n_rows * chunks * 8 bytes.  The tokens equal tl_sample's.
@@ -289,12 +304,63 @@ TL_EXPORT int tl_sample_chunks(const float* logits, int row_stride, int n_rows, 
   if (n_rows == 0) return TL_OK;
   const int chunk_len = ((vocab + chunks - 1) / chunks + 3) / 4 * 4;
   const int used = (vocab + chunk_len - 1) / chunk_len;  // no chunk is empty
-  sample_chunks_kernel<<<dim3(used, n_rows), kThreads, 0, stream>>>(logits, row_stride, vocab, temperature, seeds, steps,
-                                                                   chunk_len, (Best*)candidates);
-  int rc = tl_check_launch("sample_chunks");
+  return launch_sample_chunks(logits, row_stride, n_rows, vocab, temperature, seeds, steps, chunk_len, used,
+                              (Best*)candidates, out, stream);
+}
+
+// ----------------------------------------------------------------------------- without a workspace
+// The candidates of tl_sample_chunks_static (see no_alloc.h).  In host code this name is a stand-in,
+// not a device address: the address on each GPU comes from hipGetSymbolAddress, once per device.
+// (No `used` attribute here: with it the compiler keeps the device-side symbol local, and the
+// runtime, which looks the array up by name in the code object, aborts the process.)
+static __device__ __align__(256) unsigned char scratch[TL_STATIC_CANDIDATES * sizeof(Best)];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};  // per device: where that GPU holds its copy of `scratch`
+
+// The current device's copy of `scratch`; looked up at the first call on that device.
+int static_candidates(Best** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "sample_chunks_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return tl_fail(TL_ERR_UNSUPPORTED, "sample_chunks_static: device %d beyond %d", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return tl_fail(TL_ERR_HIP, "sample_chunks_static: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = (Best*)g_scratch_ptr[dev];
+  return TL_OK;
+}
+}  // namespace
+
+// tl_sample_chunks with the candidates in the library's own fixed array: allocates nothing.  The
+// stream must belong to the current device.  Calls that overlap on one GPU race (no_alloc.h).
+TL_EXPORT int tl_sample_chunks_static(const float* logits, int row_stride, int n_rows, int vocab,
+                                      const float* temperature, const uint64_t* seeds, const uint64_t* steps, int chunks,
+                                      int32_t* out, hipStream_t stream) {
+  TL_REQUIRE(n_rows >= 0 && vocab > 0 && row_stride >= vocab, "sample_chunks_static: bad sizes");
+  TL_REQUIRE(logits && temperature && seeds && steps && out, "sample_chunks_static: null argument");
+  TL_REQUIRE(chunks >= 1 && chunks <= 1024 && n_rows <= 65535,
+             "sample_chunks_static: chunks must be 1..1024, rows at most 65535");
+  TL_REQUIRE(row_stride % 4 == 0 && ((uintptr_t)logits % 16) == 0,
+             "sample_chunks_static: rows must start on 16-byte boundaries");
+  if (n_rows == 0) return TL_OK;
+  const int chunk_len = ((vocab + chunks - 1) / chunks + 3) / 4 * 4;
+  const int used = (vocab + chunk_len - 1) / chunk_len;
+  TL_REQUIRE((long long)n_rows * used <= TL_STATIC_CANDIDATES,
+             "sample_chunks_static: %d rows in %d pieces need %lld candidates, the fixed array holds %d", n_rows, used,
+             (long long)n_rows * used, TL_STATIC_CANDIDATES);
+  Best* candidates = nullptr;
+  int rc = static_candidates(&candidates);
   if (rc != TL_OK) return rc;
-  sample_pick_kernel<<<n_rows, kWave, 0, stream>>>((const Best*)candidates, used, out);
-  return tl_check_launch("sample_pick");
+  return launch_sample_chunks(logits, row_stride, n_rows, vocab, temperature, seeds, steps, chunk_len, used, candidates, out,
+                              stream);
 }
 
 // The uniforms the sampler uses for (seed, step), indices 0..n-1; for tests of the sampler.

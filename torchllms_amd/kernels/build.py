@@ -36,7 +36,7 @@ CORE_SOURCES = [
     "gemm_wide.hip",
     "sampling.hip",
 ]
-HEADERS = ["common.h", "qkv_epilogue.h"]
+HEADERS = ["common.h", "qkv_epilogue.h", "no_alloc.h"]
 
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}",

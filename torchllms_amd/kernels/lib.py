@@ -44,6 +44,7 @@ _CORE_SIGNATURES = {
     "tl_gemm_wide_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P],
     "tl_sample": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P],
     "tl_sample_chunks": [_P, _I, _I, _I, _P, _P, _P, _I, _P, _P, _P],
+    "tl_sample_chunks_static": [_P, _I, _I, _I, _P, _P, _P, _I, _P, _P],
     "tl_philox_uniform": [_U64, _U64, _P, _I, _P],
 }
 
