@@ -85,13 +85,12 @@ def weight_bytes(engine) -> int:
             nonlocal total
             total += t.numel() * t.element_size()
 
-    for b in m.blocks:
-        for part in (b.mixer, b.feed_forward, b.mixer_norm, b.ffn_norm):
-            for v in vars(part).values():
-                if hasattr(v, "data_ptr"):
-                    add(v)
-    add(m.final_norm.weight)
-    add(m.head.weight)
+    for part in m.all_parts():
+        if part is m.embedding:
+            continue  # a step reads as many rows of it as it has tokens
+        for v in vars(part).values():
+            if hasattr(v, "data_ptr"):
+                add(v)
     return total
 
 

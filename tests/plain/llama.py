@@ -1,8 +1,8 @@
 """A plain, slow implementation of the Llama 3 dense decoder: whole sequences, no cache, one
 function per part, only ``torch`` tensor arithmetic.  It shares no code with ``torchllms_amd``.
 
-It is written from the formulas of the reference (every function cites file:line under
-``/root/reference``), which was read, not run.  Tests compare the engine against it.
+It is written from the formulas of the reference (every function cites the reference's file:line),
+which was read, not run.  Tests compare the engine against it.
 
 Conventions: one sequence at a time; activations are [S, ...]; ``weights`` is the dict of a
 checkpoint's tensors under the checkpoint's own names (``model.layers.0.self_attn.q_proj.weight``),
@@ -133,7 +133,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional
         scores = torch.matmul(qh, kh.transpose(1, 2)) / math.sqrt(dh)
     else:
         scores = torch.matmul(qh, kh.transpose(1, 2)) * scale
-    scores = scores + causal_mask(sq, sk, q.dtype)
+    scores = scores + causal_mask(sq, sk, q.dtype).to(q.device)
     weights = F.softmax(scores, dim=-1)
     out = torch.matmul(weights, vh)  # [Hq, Sq, dh]
     return out.transpose(0, 1).reshape(sq, hq * dh)
@@ -192,17 +192,19 @@ def block(x: torch.Tensor, lw: Dict[str, torch.Tensor], cfg: dict, positions: to
 
 
 def forward(weights: Dict[str, torch.Tensor], cfg: dict, tokens: List[int], dtype: torch.dtype = torch.float32,
-            start_position: int = 0) -> torch.Tensor:
+            start_position: int = 0, device: str = "cpu") -> torch.Tensor:
     """reference: torchllms/models/networks.py:1017-1047.  Embedding, blocks, final norm, output
     matrix (the embedding matrix when ``tie_word_embeddings``).  Returns logits [S, V] in ``dtype``.
-    ``start_position`` shifts all positions (only distances may matter)."""
-    w = {k: v.to(dtype) for k, v in weights.items()}
+    ``start_position`` shifts all positions (only distances may matter).  ``device``: where torch
+    does the arithmetic (the same tensor operations anywhere)."""
+    w = {k: v.to(device=device, dtype=dtype) for k, v in weights.items()}
     hq = cfg["num_attention_heads"]
     dh = cfg.get("head_dim") or cfg["hidden_size"] // hq
     theta = cfg.get("rope_theta") or 10000.0
     inv_freq = rope_inverse_frequencies(dh, theta, cfg.get("rope_scaling"))
-    ids = torch.tensor(tokens, dtype=torch.long)
-    positions = torch.arange(start_position, start_position + len(tokens))
+    inv_freq = inv_freq.to(device)
+    ids = torch.tensor(tokens, dtype=torch.long, device=device)
+    positions = torch.arange(start_position, start_position + len(tokens), device=device)
     h = w["model.embed_tokens.weight"][ids]
     for i in range(cfg["num_hidden_layers"]):
         h = block(h, layer_weights(w, i, cfg), cfg, positions, inv_freq)

@@ -5,6 +5,7 @@ reference: torchllms/models/test_paged_kv.py:53-136,303-426."""
 import random
 
 import pytest
+import torch
 
 from torchllms_amd.cache import CacheGroupSpec, CacheManager, OutOfPages, OutOfSlots, PagePool, StateSlotSpec, group_layers
 from torchllms_amd.parts import KVNeed, StateNeed
@@ -230,3 +231,82 @@ def test_random_orders_keep_the_invariants(seed):
         c.free(rid)
     c.check_invariants()
     assert c.free_pages() == c.pools[0].num_pages and c.free_slots == 4
+
+
+def test_groups_differ_in_page_size_and_element_type():
+    """Needs that name a page size or an element type of their own form groups of their own, whose
+    tables, pools and tensors follow their own sizes."""
+    needs = [
+        ((0, "mixer"), KVNeed(2, 8, 0)), ((1, "mixer"), KVNeed(2, 8, 0, page_size=8)),
+        ((2, "mixer"), KVNeed(2, 8, 0)), ((3, "mixer"), KVNeed(2, 8, 0, page_size=8, dtype="float32")),
+    ]
+    groups, _ = group_layers(needs)
+    assert [(g.run_ids, g.page_size, g.dtype) for g in groups] == [
+        (((0, "mixer"), (2, "mixer")), 0, None), (((1, "mixer"),), 8, None), (((3, "mixer"),), 8, "float32"),
+    ]
+    pages = CacheManager.pages_for_tokens(groups, 4, 40)
+    assert pages == {"kv0": 10, "kv1": 5, "kv2": 5}
+    assert CacheManager.bytes_per_token(groups, torch.bfloat16) == 2 * 2 * 8 * (2 * 2 + 1 * 2 + 1 * 4)
+    c = CacheManager(groups, [], page_size=4, num_pages=pages, max_seqs=2, dtype=torch.bfloat16, device="cpu")
+    assert c.page_sizes == [4, 8, 8]
+    assert c.k_pages[0].shape == (2, 10, 2, 4, 8) and c.k_pages[1].shape == (1, 5, 2, 8, 8)
+    assert c.k_pages[1].dtype == torch.bfloat16 and c.k_pages[2].dtype == torch.float32
+    assert c.view((1, "mixer")).page_size == 8 and c.view((0, "mixer")).page_size == 4
+    c.admit("a")
+    assert c.new_pages_needed("a", 9) == [3, 2, 2]
+    c.extend("a", 9)
+    c.advance("a", 9)
+    assert [len(c.block_table("a", g)) for g in range(3)] == [3, 2, 2]
+    assert c.new_pages_needed("a", 3) == [0, 0, 0] and c.new_pages_needed("a", 4) == [1, 0, 0]
+    assert c.new_pages_needed("a", 8) == [2, 1, 1]
+    c.truncate("a", 8)
+    assert [len(c.block_table("a", g)) for g in range(3)] == [2, 1, 1]
+    # the small pages end first: 40 tokens fill all three pools, one more fits none
+    c.extend("a", 32)
+    c.advance("a", 32)
+    assert [c.free_pages(g) for g in range(3)] == [0, 0, 0] and not c.can_extend("a", 1)
+    c.check_invariants()
+    c.free("a")
+    assert [c.free_pages(g) for g in range(3)] == [10, 5, 5]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_keep_the_invariants_with_mixed_page_sizes(seed):
+    rng = random.Random(100 + seed)
+    sizes = [rng.choice([2, 4, 8]), rng.choice([3, 16]), rng.choice([4, 5])]
+    windows = [0, rng.choice([0, 7]), 0]
+    groups = [CacheGroupSpec(f"kv{g}", (g,), 1, 4, windows[g], page_size=p) for g, p in enumerate(sizes)]
+    tokens = rng.choice([40, 90])
+    c = CacheManager(groups, [], 4, CacheManager.pages_for_tokens(groups, 4, tokens), max_seqs=3)
+    live = {}
+    next_id = 0
+    for _ in range(500):
+        op = rng.random()
+        if op < 0.2 and c.free_slots:
+            c.admit(next_id)
+            live[next_id] = 0
+            next_id += 1
+        elif op < 0.85 and live:
+            rid = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 2, 3, 7, 16])
+            need = c.new_pages_needed(rid, n)
+            if c.can_extend(rid, n):
+                before = [c.free_pages(g) for g in range(3)]
+                c.extend(rid, n)
+                assert [b - c.free_pages(g) for g, b in enumerate(before)] == need
+                c.advance(rid, n)
+                live[rid] += n
+            else:
+                held = [list(c.block_table(rid, g)) for g in range(3)]
+                with pytest.raises(OutOfPages):
+                    c.extend(rid, n)
+                assert [c.block_table(rid, g) for g in range(3)] == held
+        elif live:
+            rid = rng.choice(list(live))
+            c.free(rid)
+            del live[rid]
+        c.check_invariants()
+    for rid in list(live):
+        c.free(rid)
+    c.check_invariants()
+    assert all(c.free_pages(g) == c.pools[g].num_pages for g in range(3))

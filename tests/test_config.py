@@ -100,11 +100,11 @@ def test_model_spec_is_data():
     cfg = LlamaConfig.from_dict(TINY_B)
     spec = llama_model_spec(cfg)
     assert len(spec.layers) == 3 and [r.layer for r in spec.order] == [0, 1, 2]
-    m = spec.layers[0].mixer
+    m = spec.layers[0].parts["mixer"]
     assert m.kind == "attention" and m.params["num_kv_heads"] == 1 and m.params["head_dim"] == 32
     assert m.params["softmax_scale"] == 32 ** -0.5
     assert m.params["position"].params["scaling"]["factor"] == 8.0
-    assert spec.layers[0].feed_forward.params["intermediate_size"] == 688
+    assert spec.layers[0].parts["ffn"].params["intermediate_size"] == 688
     assert spec.final_norm.params["eps"] == 1e-6
     assert spec.head.params["tied"] is False
 
@@ -120,3 +120,22 @@ def test_order_is_checked():
         bad.validate()
     ok = ModelSpec(**{**spec.__dict__, "order": [LayerRun(0), LayerRun(1), LayerRun(0), LayerRun(1, cache_from=1)]})
     ok.validate()
+
+
+def test_sizes_no_kernel_takes_are_refused_when_the_model_is_checked():
+    """A head size above 256 (no attention kernel takes it) and a width beyond what the norm kernel
+    holds in LDS are refused by the parts themselves, with the limit in the message, before any
+    tensor exists; the engine asks when it is built (tests/test_gpu_engine.py)."""
+    import torch
+
+    from torchllms_amd.parts import Model
+
+    ok = LlamaConfig.from_dict(dict(TINY_B, head_dim=256))
+    for dtype in (torch.float32, torch.bfloat16):
+        Model(llama_model_spec(ok)).check_sizes(dtype)
+    big_head = LlamaConfig.from_dict(dict(TINY_B, head_dim=272))
+    with pytest.raises(ValueError, match="head size 272.*up to 256"):
+        Model(llama_model_spec(big_head)).check_sizes(torch.bfloat16)
+    wide = LlamaConfig.from_dict(dict(TINY_A, hidden_size=40960, num_attention_heads=4, head_dim=16, num_hidden_layers=1))
+    with pytest.raises(ValueError, match="rmsnorm: rows of 40960 elements.*1 to 40704"):
+        Model(llama_model_spec(wide)).check_sizes(torch.float32)

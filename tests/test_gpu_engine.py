@@ -275,7 +275,48 @@ def test_pool_sizes(cases):
         (dict(max_seqs=3, max_model_len=50), lambda n, pp: n == 3 * 7),
     ]:
         eng = Engine.from_folder(folder, dtype="float32", page_size=8, **kw)
-        per_page = CacheManager.bytes_per_page(eng.cache.groups, 8, torch.float32)
+        per_page = 8 * CacheManager.bytes_per_token(eng.cache.groups, torch.float32)
         assert check(eng.cache.pools[0].num_pages, per_page), kw
     with pytest.raises(ValueError, match="kv_memory_fraction"):
         Engine.from_folder(folder, dtype="float32", kv_memory_fraction=1.5)
+
+
+def test_sizes_no_kernel_takes_are_refused_when_the_engine_is_built():
+    """Not at the first step: ``Engine`` asks every part at construction, before it loads anything."""
+    from torchllms_amd.config import LlamaConfig
+    from torchllms_amd.engine import Engine
+
+    cfg = LlamaConfig.from_dict(dict(TINY["B"], head_dim=272, num_hidden_layers=1))
+    for dtype in ("float32", "bfloat16"):
+        with pytest.raises(ValueError, match="head size 272.*up to 256"):
+            Engine.from_random(cfg, seed=0, dtype=dtype, max_seqs=1, max_model_len=64)
+    cfg = LlamaConfig.from_dict(dict(TINY["B"], head_dim=256, num_hidden_layers=1))
+    eng = Engine.from_random(cfg, seed=0, dtype="bfloat16", max_seqs=1, max_model_len=64)
+    with pytest.raises(ValueError, match="page_size"):
+        Engine.from_random(cfg, seed=0, dtype="bfloat16", max_seqs=1, max_model_len=64, page_size=0)
+    del eng
+
+
+def test_a_step_that_fails_leaves_nothing_behind(cases):
+    """A step whose forward pass raises books nothing: the pages it took go back, the request is
+    where it was, and the next step is planned afresh."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    eng = Engine.from_folder(cases["A"].folder, dtype="float32", page_size=8, num_pages=12, max_seqs=2, use_graphs=False)
+    eng.admit("r")
+    first = eng.step([StepEntry("r", [1, 2, 3, 4, 5], [4])]).cpu()
+    free = eng.cache.free_pages()
+    real_forward = eng.model.forward
+    eng.model.forward = lambda ctx, cache: (_ for _ in ()).throw(RuntimeError("kernel failed"))
+    for tokens in ([7], list(range(30))):
+        with pytest.raises(RuntimeError, match="kernel failed"):
+            eng.step([StepEntry("r", tokens, [0])])
+        assert eng.num_tokens("r") == 5 and eng.cache.free_pages() == free and eng._last_decode is None
+        eng.cache.check_invariants()
+    eng.model.forward = real_forward
+    again = eng.step([StepEntry("r", [7], [0])]).cpu()
+    eng.free("r")
+    eng.admit("s")
+    whole = eng.step([StepEntry("s", [1, 2, 3, 4, 5, 7], [4, 5])]).cpu()
+    eng.free("s")
+    assert torch.equal(whole[0], first[0]) and torch.equal(whole[1], again[0])

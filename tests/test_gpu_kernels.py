@@ -20,6 +20,18 @@ def _ops():
     return ops
 
 
+class _Products:
+    """The matrix products' own module (its table of measured choices), imported on first use."""
+
+    def __getattr__(self, name):
+        from torchllms_amd.kernels import products as module
+
+        return getattr(module, name)
+
+
+products = _Products()
+
+
 def _i32(x):
     return torch.tensor(x, dtype=torch.int32, device=DEV)
 
@@ -753,16 +765,16 @@ def test_tune_linear_remembers_a_choice_for_every_row_bucket():
     ops = _ops()
     torch.manual_seed(0)
     weights = [torch.randn(48, 64, device=DEV).bfloat16() for _ in range(2)]
-    for key in [k for k in ops._LINEAR_CHOICE if k[:2] == (48, 64)]:
-        del ops._LINEAR_CHOICE[key]
+    for key in [k for k in products.LINEAR_CHOICE if k[:2] == (48, 64)]:
+        del products.LINEAR_CHOICE[key]
     ops.tune_linear(weights)
     ops.tune_linear(weights, use="glu")
     for bucket in ops.ROW_BUCKETS:
         if bucket <= ops.STREAM_MAX_ROWS:
-            assert ops._LINEAR_CHOICE[(48, 64, bucket, "plain")] in (None,) + tuple(("stream", w) for w in ops.STREAM_WAVE_CHOICES)
-            assert ops._LINEAR_CHOICE[(48, 64, bucket, "glu")] in (None,) + tuple(("stream", w, c) for w in ops.STREAM_WAVE_CHOICES for c in (8, 16))
+            assert products.LINEAR_CHOICE[(48, 64, bucket, "plain")] in (None,) + tuple(("stream", w) for w in ops.STREAM_WAVE_CHOICES)
+            assert products.LINEAR_CHOICE[(48, 64, bucket, "glu")] in (None,) + tuple(("stream", w, c) for w in ops.STREAM_WAVE_CHOICES for c in (8, 16))
         else:
-            assert ops._LINEAR_CHOICE[(48, 64, bucket, "plain")] is None  # K = 64 is no multiple of 128: the library
+            assert products.LINEAR_CHOICE[(48, 64, bucket, "plain")] is None  # K = 64 is no multiple of 128: the library
     x = torch.randn(5, 64, device=DEV).bfloat16()
     got = ops.linear(x, weights[0]).float().cpu()
     torch.testing.assert_close(got, (x.float() @ weights[0].float().T).cpu(), rtol=2 ** -7, atol=0.1)
@@ -914,10 +926,10 @@ def test_linear_to_sum_leaves_a_product_split_only_where_it_was_tuned_to_be_spli
     x = torch.randn(40, 512, device=DEV).bfloat16()
     want = (x.float() @ w.float().T).cpu()
     key = (96, 512, 64, "sum")
-    saved = ops._LINEAR_CHOICE.get(key, "absent")
+    saved = products.LINEAR_CHOICE.get(key, "absent")
     try:
         for choice, split in ((None, False), (("wide", 1, 1, 3), False), (("wide", 1, 4, 3), True), (("wide", 2, 2, 2), True)):
-            ops._LINEAR_CHOICE[key] = choice
+            products.LINEAR_CHOICE[key] = choice
             got = ops.linear_to_sum(x, w)
             assert isinstance(got, ops.SplitSums) == split, choice
             if split:
@@ -929,33 +941,33 @@ def test_linear_to_sum_leaves_a_product_split_only_where_it_was_tuned_to_be_spli
         assert isinstance(f32, torch.Tensor) and f32.dtype == torch.float32
     finally:
         if saved == "absent":
-            ops._LINEAR_CHOICE.pop(key, None)
+            products.LINEAR_CHOICE.pop(key, None)
         else:
-            ops._LINEAR_CHOICE[key] = saved
+            products.LINEAR_CHOICE[key] = saved
 
 
 def test_tune_linear_measures_the_wide_kernel_from_17_rows_on():
     ops = _ops()
     torch.manual_seed(0)
     weights = [(torch.randn(96, 256, device=DEV) * 0.1).bfloat16() for _ in range(2)]
-    for key in [k for k in ops._LINEAR_CHOICE if k[:2] == (96, 256)]:
-        del ops._LINEAR_CHOICE[key]
+    for key in [k for k in products.LINEAR_CHOICE if k[:2] == (96, 256)]:
+        del products.LINEAR_CHOICE[key]
     for use in ops.LINEAR_USES:
         ops.tune_linear(weights, use=use)
     allowed = {None} | {("wide",) + c for c in ops.WIDE_CHOICES if c[1] <= 2}
     for use in ops.LINEAR_USES:
-        assert ops._LINEAR_CHOICE[(96, 256, 32, use)] in allowed and ops._LINEAR_CHOICE[(96, 256, 64, use)] in allowed
+        assert products.LINEAR_CHOICE[(96, 256, 32, use)] in allowed and products.LINEAR_CHOICE[(96, 256, 64, use)] in allowed
     # whatever was chosen, and each of the kernel's launches when it is forced, gives the product
     x = torch.randn(40, 256, device=DEV).bfloat16()
     want = (x.float() @ weights[0].float().T).cpu()
     torch.testing.assert_close(ops.linear(x, weights[0]).float().cpu(), want, rtol=2 ** -7, atol=0.05)
     glu_ref = (torch.nn.functional.silu(x.float() @ weights[0][:48].float().T) * (x.float() @ weights[0][48:].float().T)).cpu()
     for choice in sorted(allowed - {None}) + [("wide", 1, 2, 2)]:
-        ops._LINEAR_CHOICE[(96, 256, 64, "plain")] = ops._LINEAR_CHOICE[(96, 256, 64, "glu")] = choice
+        products.LINEAR_CHOICE[(96, 256, 64, "plain")] = products.LINEAR_CHOICE[(96, 256, 64, "glu")] = choice
         torch.testing.assert_close(ops.linear(x, weights[0]).float().cpu(), want, rtol=2 ** -7, atol=0.05)
         torch.testing.assert_close(ops.linear_glu(x, weights[0]).float().cpu(), glu_ref, rtol=2 ** -6, atol=0.05)
     for use in ops.LINEAR_USES:
-        del ops._LINEAR_CHOICE[(96, 256, 64, use)]
+        del products.LINEAR_CHOICE[(96, 256, 64, use)]
 
 
 # ----------------------------------------------------------------------------- prefill attention (MFMA)

@@ -132,11 +132,13 @@ def test_pre_norm_block_matches_the_plain_block():
     D, S = 48, 17
     pos_spec = PartSpec("rope", dict(head_dim=16, rotary_dim=16, theta=10000.0, scaling=None))
     block = BLOCKS["pre_norm"](
-        mixer=MIXERS.build(PartSpec("attention", dict(hidden_size=D, num_heads=3, num_kv_heads=3, head_dim=16, qkv_bias=False,
-                                                      softmax_scale=0.25, window=0, position=pos_spec))),
-        feed_forward=FEED_FORWARDS.build(PartSpec("swiglu", dict(hidden_size=D, intermediate_size=100))),
-        mixer_norm=NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=1e-5))),
-        ffn_norm=NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=1e-5))),
+        {
+            "mixer": MIXERS.build(PartSpec("attention", dict(hidden_size=D, num_heads=3, num_kv_heads=3, head_dim=16, qkv_bias=False,
+                                                             softmax_scale=0.25, window=0, position=pos_spec))),
+            "ffn": FEED_FORWARDS.build(PartSpec("swiglu", dict(hidden_size=D, intermediate_size=100))),
+            "mixer_norm": NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=1e-5))),
+            "ffn_norm": NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=1e-5))),
+        }
     )
     w = {n: (torch.randn(s.shape) * 0.3 if s.init == "normal" else 1 + 0.1 * torch.randn(s.shape)) for n, s in block.param_specs().items()}
     block.bind({k: v.to(DEV) for k, v in w.items()})
@@ -147,9 +149,9 @@ def test_pre_norm_block_matches_the_plain_block():
     want = plain.block(x, lw, cfg, torch.arange(S), plain.rope_inverse_frequencies(16, 10000.0, None))
     cache = _ctx_and_cache(S, 3, 16, 4, torch.float32)
     ctx = _step(cache, "r", S)
-    h, delta = block.forward(x.to(DEV), None, ctx, cache.kv_view(0))
+    h, delta = block.forward(x.to(DEV), None, ctx, {"mixer": cache.kv_view(0)})
     torch.testing.assert_close((h + delta).cpu(), want, rtol=1e-4, atol=1e-4)
     # a pending delta from the layer before is added first
     cache2 = _ctx_and_cache(S, 3, 16, 4, torch.float32)
-    h2, d2 = block.forward((x * 0.5).to(DEV), (x * 0.5).to(DEV), _step(cache2, "r", S), cache2.kv_view(0))
+    h2, d2 = block.forward((x * 0.5).to(DEV), (x * 0.5).to(DEV), _step(cache2, "r", S), {"mixer": cache2.kv_view(0)})
     torch.testing.assert_close((h2 + d2).cpu(), want, rtol=1e-4, atol=1e-4)

@@ -55,3 +55,160 @@ def test_real_layer_sizes_match_the_plain_model_under_every_schedule(real, dtype
         for name in ("tail", "mixed"):
             for key, row in results[name].items():
                 assert torch.equal(row, results["whole"][key]), f"{name} differs from whole at {key}"
+
+
+# ----------------------------------------------------------------------------- the sizes that are benchmarked
+# One layer of the same sizes: long prompts (a prefill launch of more than 1,024 blocks, portions behind a
+# long prefix), decode steps replayed from graphs across context caps, and many live requests of very
+# unequal lengths.  The 32-bit truth is the plain model on the CPU; the bfloat16 yardstick is the plain
+# model in bfloat16, whose tensor operations torch runs on the GPU here (on the CPU they take minutes).
+ONE_LAYER = dict(REAL, num_hidden_layers=1)
+
+
+def _bf16_tolerance(weights, cfg, tokens, want):
+    yard = plain.forward(weights, cfg, tokens, torch.bfloat16, device="cuda:0").float().cpu()
+    return 2 * (yard - want).abs().amax(dim=-1) + 1e-3  # per position
+
+
+@pytest.fixture(scope="module")
+def one_layer(tmp_path_factory):
+    folder = make_folder(tmp_path_factory.mktemp("long") / "m", ONE_LAYER, seed=5, dtype=torch.bfloat16, norm_jitter=0.1, sharpen=True)
+    cfg, weights = read_folder(folder)
+    return folder, cfg, weights
+
+
+def _cut(rid, tokens, sizes, tail):
+    """A trace of one request: portions of the given sizes, then ``tail`` single tokens, all wanted."""
+    steps, i = [], 0
+    for n in list(sizes) + [1] * tail:
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": tokens[i : i + n], "want": list(range(n))}], "end": []})
+        i += n
+    assert i == len(tokens)
+    steps[-1]["end"] = [rid]
+    return steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_whole_and_in_portions_behind_a_long_prefix(one_layer, dtype):
+    """4,700 tokens in one step (1,176 blocks of the prefill attention kernel: beyond the 1,024 up
+    to which blocks hold two sets of waves), then the same request as 2,100 tokens, portions of 700,
+    2, 1,000, 31 and 827 behind them, and the last 40 tokens one by one."""
+    from torchllms_amd.engine import Engine
+    from torchllms_amd.kernels import ops
+
+    folder, cfg, weights = one_layer
+    n = 4700
+    tokens = random_tokens(n, ONE_LAYER["vocab_size"], 77)
+    want = plain.forward(weights, cfg, tokens, torch.float32)
+    qpt = ops.prefill_queries_per_tile(32, 8, 128)
+    assert -(-n // qpt) * 8 > ops.PREFILL_SPLIT_BLOCKS  # the whole prompt is a launch with one set of waves
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=-(-n // 16) + 1, max_seqs=2, max_model_len=8192)
+    whole = run_trace(eng, _cut("w", tokens, [n], 0))
+    parts = run_trace(eng, _cut("p", tokens, [2100, 700, 2, 1000, 31, 827], 40))
+    tol = _bf16_tolerance(weights, cfg, tokens, want) if dtype == "bfloat16" else None
+    for name, res in (("whole", whole), ("portions", parts)):
+        rid = name[0]
+        got = torch.stack([res[(rid, pos)] for pos in range(n)])
+        err = (got - want).abs().amax(dim=-1)
+        if dtype == "float32":
+            bad = (err >= 10 * FP32_ATOL).nonzero().flatten()
+        else:
+            bad = (err > tol).nonzero().flatten()
+        assert bad.numel() == 0, f"{name}: first wrong position {int(bad[0])} of {bad.numel()}, error {err[bad[0]].item()}"
+    if dtype == "float32":
+        diff = [pos for pos in range(n) if not torch.equal(whole[("w", pos)], parts[("p", pos)])]
+        assert not diff, f"portions differ from the whole prompt at {len(diff)} positions, first {diff[0]}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graphs_across_context_caps(one_layer, dtype):
+    """Two requests decoded side by side from 480 and 30 tokens on, one token a step, until the
+    longer holds 2,070: the recorded decode steps change with the context cap (512, 1,024, 2,048,
+    4,096), each with wider block tables and more splits of the keys."""
+    from torchllms_amd.engine import Engine
+
+    folder, cfg, weights = one_layer
+    long_tokens = random_tokens(2070, ONE_LAYER["vocab_size"], 78)
+    short_tokens = random_tokens(30 + 1590, ONE_LAYER["vocab_size"], 79)
+    want = {"a": plain.forward(weights, cfg, long_tokens, torch.float32), "b": plain.forward(weights, cfg, short_tokens, torch.float32)}
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": long_tokens[:480], "want": list(range(480))},
+                                     {"id": "b", "tokens": short_tokens[:30], "want": list(range(30))}], "end": []}]
+    for i in range(1590):
+        steps.append({"step": len(steps), "entries": [{"id": "a", "tokens": [long_tokens[480 + i]], "want": [0]},
+                                                      {"id": "b", "tokens": [short_tokens[30 + i]], "want": [0]}], "end": []})
+    steps[-1]["end"] = ["a", "b"]
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=2 * 130 + 2, max_seqs=2, max_model_len=4096, use_graphs=True)
+    got = run_trace(eng, steps)
+    caps = sorted(key[2] for key in eng.graphs.graphs)
+    assert set(caps) >= {512, 1024, 2048, 4096}, caps
+    assert sum(g.replays for g in eng.graphs.graphs.values()) > 1500
+    tols = {r: _bf16_tolerance(weights, cfg, t, want[r]) for r, t in (("a", long_tokens), ("b", short_tokens))} if dtype == "bfloat16" else None
+    for rid, toks in (("a", long_tokens), ("b", short_tokens)):
+        rows = torch.stack([got[(rid, pos)] for pos in range(len(toks))])
+        err = (rows - want[rid]).abs().amax(dim=-1)
+        bad = (err >= 10 * FP32_ATOL).nonzero().flatten() if dtype == "float32" else (err > tols[rid]).nonzero().flatten()
+        assert bad.numel() == 0, f"{rid}: first wrong position {int(bad[0])} of {bad.numel()}, error {err[bad[0]].item()}"
+    if dtype == "float32":
+        # the same bits as the whole prompt in one step gives
+        whole = run_trace(eng, _cut("a", long_tokens, [len(long_tokens)], 0))
+        diff = [pos for pos in range(len(long_tokens)) if not torch.equal(whole[("a", pos)], got[("a", pos)])]
+        assert not diff, f"decoded positions differ from the whole prompt at {len(diff)} positions, first {diff[0]}"
+
+
+MANY_LENGTHS = [1900, 23, 700, 64, 1100, 17, 1500] + [10 + (37 * i) % 111 for i in range(57)]  # 64 requests, very unequal
+
+
+@pytest.fixture(scope="module")
+def many(one_layer):
+    folder, cfg, weights = one_layer
+    requests = {f"m{i}": random_tokens(n, ONE_LAYER["vocab_size"], 300 + i) for i, n in enumerate(MANY_LENGTHS)}
+    truth = {rid: plain.forward(weights, cfg, t, torch.float32) for rid, t in requests.items()}
+    return requests, truth
+
+
+@pytest.mark.parametrize("live", [24, 64])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_live_requests_of_unequal_lengths_decode_together(one_layer, many, dtype, live):
+    """24 and 64 live requests of 10 to 1,900 tokens: prompts prefilled eight to a step, then the
+    last 20 tokens of every request decoded together, 24 or 64 rows a step, replayed from graphs
+    whose key says that the lengths differ much (shorter key splits in the decode attention)."""
+    from torchllms_amd.engine import Engine
+
+    folder, cfg, weights = one_layer
+    all_requests, truth = many
+    requests = dict(list(all_requests.items())[:live])
+    tail = 20
+    steps = []
+    rids = list(requests)
+    for lo in range(0, live, 8):
+        group = rids[lo : lo + 8]
+        steps.append({"step": len(steps), "end": [], "entries": [
+            {"id": r, "tokens": requests[r][: len(requests[r]) - tail], "want": [len(requests[r]) - tail - 1]} for r in group if len(requests[r]) > tail]})
+    for i in range(tail):
+        entries = []
+        for r in rids:
+            n = len(requests[r])
+            if n > tail:
+                entries.append({"id": r, "tokens": [requests[r][n - tail + i]], "want": [0]})
+            elif i == 0:
+                entries.append({"id": r, "tokens": requests[r], "want": [n - 1]})  # a short prompt joins whole
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+    steps[-1]["end"] = rids
+    pages = sum(-(-len(t) // 16) for t in requests.values()) + 4
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=pages, max_seqs=live, max_model_len=4096, use_graphs=True)
+    got = run_trace(eng, steps)
+    n_rows = sum(1 for r in rids if len(requests[r]) > tail)
+    assert any(key[0] == n_rows and key[3] for key in eng.graphs.graphs), list(eng.graphs.graphs)  # rows, uneven lengths
+    assert sum(g.replays for g in eng.graphs.graphs.values()) >= tail - 4
+    worst = []
+    for (rid, pos), row in got.items():
+        want = truth[rid][pos]
+        err = (row - want).abs().max().item()
+        if dtype == "float32":
+            assert err < 10 * FP32_ATOL, f"{rid} position {pos}: {err}"
+        else:
+            worst.append((err, rid, pos))
+    if dtype == "bfloat16":
+        tols = {r: _bf16_tolerance(weights, cfg, requests[r], truth[r]) for r in {rid for _, rid, _ in worst}}
+        for err, rid, pos in worst:
+            assert err <= tols[rid][pos].item(), f"{rid} position {pos}: {err} against {tols[rid][pos].item()}"

@@ -18,7 +18,7 @@ from .test_gpu_engine import run_trace
 
 pytestmark = pytest.mark.gpu
 
-HIDDEN, STATE, VOCAB, HEADS, KV, DH, FFN, WINDOW = 40, 24, 97, 4, 2, 16, 56, 6
+HIDDEN, STATE, VOCAB, HEADS, KV, DH, FFN, WINDOW, WINDOW_PAGE = 40, 24, 97, 4, 2, 16, 56, 6, 8
 
 
 @dataclass(frozen=True)
@@ -29,7 +29,7 @@ class ToyConfig:
 
 def _register():
     from torchllms_amd.config import ArchSpec, register_architecture
-    from torchllms_amd.config.spec import LayerRun, LayerSpec, ModelSpec, PartSpec
+    from torchllms_amd.config.spec import LayerRun, ModelSpec, PartSpec, standard_layer
     from torchllms_amd.parts import MIXERS, Mixer, ParamSpec, StateNeed
     from torchllms_amd.weights import NameRule
 
@@ -70,11 +70,13 @@ def _register():
         ffn = PartSpec("swiglu", dict(hidden_size=HIDDEN, intermediate_size=FFN))
 
         def attn(window):
+            # the windowed layer keeps its keys in pages of 8 tokens, whatever the engine's page size
             return PartSpec("attention", dict(hidden_size=HIDDEN, num_heads=HEADS, num_kv_heads=KV, head_dim=DH, qkv_bias=False,
-                                              softmax_scale=DH ** -0.5, window=window, position=rope))
+                                              softmax_scale=DH ** -0.5, window=window, position=rope,
+                                              kv_page_size=WINDOW_PAGE if window else None))
 
         mixers = [attn(0), PartSpec("toy_decay", dict(hidden_size=HIDDEN, state_size=STATE, decay=cfg.decay)), attn(WINDOW)]
-        layers = [LayerSpec(f"layers.{i}", "pre_norm", m, ffn, norm, norm) for i, m in enumerate(mixers)]
+        layers = [standard_layer(f"layers.{i}", "pre_norm", m, ffn, norm, norm) for i, m in enumerate(mixers)]
         order = [LayerRun(0), LayerRun(1), LayerRun(2), LayerRun(1), LayerRun(0, cache_from=0)]
         return ModelSpec("ToyHybridForCausalLM", HIDDEN, VOCAB, 512, PartSpec("embedding", dict(vocab_size=VOCAB, hidden_size=HIDDEN)),
                          layers, order, norm, PartSpec("lm_head", dict(vocab_size=VOCAB, hidden_size=HIDDEN, tied=True)))
@@ -150,9 +152,12 @@ def test_toy_architecture_is_registered_built_and_stepped():
     pool_tokens = max(schedules.max_live_tokens(t) for t in traces.values())
     eng = Engine(arch, cfg, {k: v.to("cuda:0") for k, v in w.items()}, torch.float32, page_size=4,
                  num_pages=-(-pool_tokens // 4), max_seqs=4, max_model_len=512)
-    # groups: full attention (runs 0 and the borrower's source), windowed attention, and state slots for two runs
-    assert sorted((g.window, g.run_ids) for g in eng.cache.groups) == [(0, (0,)), (WINDOW, (2,))]
-    assert [(s.run_ids, s.shape) for s in eng.cache.states] == [((1, 3), (STATE,))]
+    # groups: full attention (runs 0 and the borrower's source), windowed attention in pages of another size,
+    # and state slots for two runs; every group's pool holds the same number of tokens
+    assert sorted((g.window, g.run_ids) for g in eng.cache.groups) == [(0, ((0, "mixer"),)), (WINDOW, ((2, "mixer"),))]
+    assert eng.cache.page_sizes == [4, WINDOW_PAGE] and eng.cache.k_pages[1].shape[3] == WINDOW_PAGE
+    assert eng.cache.pools[0].num_pages == -(-pool_tokens // 4) and eng.cache.pools[1].num_pages == -(-(-(-pool_tokens // 4) * 4) // WINDOW_PAGE)
+    assert [(s.run_ids, s.shape) for s in eng.cache.states] == [(((1, "mixer"), (3, "mixer")), (STATE,))]
     truth = {rid: plain_toy(w, cfg, t) for rid, t in requests.items()}
     for name, steps in traces.items():
         got = run_trace(eng, steps)
@@ -163,5 +168,6 @@ def test_toy_architecture_is_registered_built_and_stepped():
     from torchllms_amd.engine import StepEntry
 
     eng.step([StepEntry("w", random_tokens(30, VOCAB, 9))])
-    assert sum(p >= 0 for p in eng.cache.block_table("w", 1)) <= 3 < sum(p >= 0 for p in eng.cache.block_table("w", 0))
+    assert sum(p >= 0 for p in eng.cache.block_table("w", 1)) <= 2 < sum(p >= 0 for p in eng.cache.block_table("w", 0))
+    assert len(eng.cache.block_table("w", 0)) == 8 and len(eng.cache.block_table("w", 1)) == 4  # 30 tokens in pages of 4 and of 8
     eng.free("w")

@@ -1,8 +1,9 @@
 """More toy parts defined here, in the test, and put together into an architecture of their own:
 a feed-forward that routes every token to one of several experts, a position encoding with
 frequencies of its own that rotates only a part of a head in half-split pairs, a norm that centres
-before it scales, and a block arrangement in which mixer and feed-forward read the same normed
-input.  None of them exists in the framework; they are registered, built from random weights and
+before it scales, a block arrangement in which mixer and feed-forward read the same normed
+input, one with norms before and behind either branch (six parts), and one that has a mixer and a
+norm and nothing else.  None of them exists in the framework; they are registered, built from random weights and
 stepped through the engine in portions and mixed batches, and compared with a plain whole-sequence
 computation written here.  They are toys, not anybody's model."""
 
@@ -20,7 +21,7 @@ from .test_gpu_engine import run_trace
 
 pytestmark = pytest.mark.gpu
 
-HIDDEN, VOCAB, HEADS, KV, DH, ROT, FFN, EXPERTS = 48, 83, 6, 3, 16, 8, 40, 3
+HIDDEN, VOCAB, HEADS, KV, DH, ROT, FFN, EXPERTS, SANDWICH_SCALE, WIDE_PAGE = 48, 83, 6, 3, 16, 8, 40, 3, 0.5, 32
 
 
 @dataclass(frozen=True)
@@ -35,7 +36,7 @@ def toy_frequencies() -> torch.Tensor:
 
 def _register():
     from torchllms_amd.config import ArchSpec, register_architecture
-    from torchllms_amd.config.spec import LayerRun, LayerSpec, ModelSpec, PartSpec
+    from torchllms_amd.config.spec import LayerRun, LayerSpec, ModelSpec, PartSpec, standard_layer
     from torchllms_amd.parts import BLOCKS, FEED_FORWARDS, NORMS, POSITIONS, Block, FeedForward, Norm, ParamSpec, PositionEncoding
     from torchllms_amd.parts.positions import RotaryArgs
     from torchllms_amd.weights import NameRule
@@ -109,12 +110,43 @@ def _register():
         class ParallelBlock(Block):
             """``out = x + mixer(norm(x)) + ffn(norm(x))``: one norm (the mixer's), both branches read it."""
 
+            SLOTS = {"mixer_norm": "norm", "mixer": "mixer", "ffn": "feed_forward"}
+
             def forward(self, h, delta, ctx, cache):
                 from torchllms_amd.kernels import ops
 
                 h, y = self.mixer_norm.forward_add(h, self.mixer_norm.delta(delta))
                 # (a branch may come back as the unadded sums of a split product: see ops.SplitSums)
-                return h, ops.resolved(self.mixer.forward(y, ctx, cache)) + ops.resolved(self.feed_forward.forward(y, ctx))
+                return h, ops.resolved(self.mixer.forward(y, ctx, cache["mixer"])) + ops.resolved(self.ffn.forward(y, ctx))
+
+        @BLOCKS.register("toy_sandwich")
+        class SandwichBlock(Block):
+            """``h = x + scale * post_a(mixer(pre_a(x))); out = h + scale * post_f(ffn(pre_f(h)))``: four
+            norms in a layer, and a constant of the arrangement's own."""
+
+            SLOTS = {"pre_a": "norm", "mixer": "mixer", "post_a": "norm", "pre_f": "norm", "ffn": "feed_forward", "post_f": "norm"}
+
+            def __init__(self, parts, scale):
+                super().__init__(parts)
+                self.scale = scale
+
+            def forward(self, h, delta, ctx, cache):
+                from torchllms_amd.kernels import ops
+
+                h, y = self.pre_a.forward_add(h, self.pre_a.delta(delta))
+                a = self.post_a.forward(ops.resolved(self.mixer.forward(y, ctx, cache["mixer"]))) * self.scale
+                h, y = self.pre_f.forward_add(h, a)
+                return h, self.post_f.forward(ops.resolved(self.ffn.forward(y, ctx))) * self.scale
+
+        @BLOCKS.register("toy_mixer_only")
+        class MixerOnlyBlock(Block):
+            """``out = x + mixer(norm(x))``: a layer without a feed-forward."""
+
+            SLOTS = {"norm": "norm", "mixer": "mixer"}
+
+            def forward(self, h, delta, ctx, cache):
+                h, y = self.norm.forward_add(h, self.norm.delta(delta))
+                return h, self.mixer.forward(y, ctx, cache["mixer"])
 
     def spec(cfg: ToyConfig) -> ModelSpec:
         rope = PartSpec("toy_partial_rotary", dict(rotary_dim=ROT))
@@ -124,19 +156,26 @@ def _register():
         dense = PartSpec("swiglu", dict(hidden_size=HIDDEN, intermediate_size=FFN))
         attn = PartSpec("attention", dict(hidden_size=HIDDEN, num_heads=HEADS, num_kv_heads=KV, head_dim=DH, qkv_bias=False,
                                           softmax_scale=DH ** -0.5, window=0, position=rope))
+        # the last layer's keys and values lie in pages of another size than the engine's
+        attn_wide_pages = PartSpec("attention", dict(attn.params, kv_page_size=WIDE_PAGE))
         layers = [
-            LayerSpec("layers.0", "pre_norm", attn, routed, centred, rms),
-            LayerSpec("layers.1", "toy_parallel", attn, dense, centred, centred),
-            LayerSpec("layers.2", "pre_norm", attn, routed, rms, centred),
+            standard_layer("layers.0", "pre_norm", attn, routed, centred, rms),
+            LayerSpec("layers.1", "toy_parallel", {"mixer_norm": centred, "mixer": attn, "ffn": dense}),
+            standard_layer("layers.2", "pre_norm", attn, routed, rms, centred),
+            LayerSpec("layers.3", "toy_sandwich", {"pre_a": rms, "mixer": attn, "post_a": centred, "pre_f": centred, "ffn": dense,
+                                                   "post_f": rms}, {"scale": SANDWICH_SCALE}),
+            LayerSpec("layers.4", "toy_mixer_only", {"norm": rms, "mixer": attn_wide_pages}),
         ]
         return ModelSpec("ToyRoutedForCausalLM", HIDDEN, VOCAB, 512, PartSpec("embedding", dict(vocab_size=VOCAB, hidden_size=HIDDEN)),
-                         layers, [LayerRun(0), LayerRun(1), LayerRun(2)], centred,
+                         layers, [LayerRun(i) for i in range(5)], centred,
                          PartSpec("lm_head", dict(vocab_size=VOCAB, hidden_size=HIDDEN, tied=False)))
 
     def rules(cfg):
         names = ["embed.weight", "final_norm.weight", "final_norm.bias", "head.weight"]
         per_layer = ["mixer_norm.weight", "mixer_norm.bias", "ffn_norm.weight", "ffn_norm.bias", "ffn.w1.weight", "ffn.w2.weight",
-                     "ffn.w3.weight", "ffn.router.weight", "mixer.wq.weight", "mixer.wk.weight", "mixer.wv.weight", "mixer.wo.weight"]
+                     "ffn.w3.weight", "ffn.router.weight", "mixer.wq.weight", "mixer.wk.weight", "mixer.wv.weight", "mixer.wo.weight",
+                     "norm.weight"]
+        per_layer += [f"{slot}.{t}" for slot in ("pre_a", "post_a", "pre_f", "post_f") for t in ("weight", "bias")]
         per_layer += [f"ffn.experts.{e}.{m}.weight" for e in range(EXPERTS) for m in ("up", "down")]
         return [NameRule(n, n) for n in names] + [NameRule("layers.{}." + n, "layers.{}." + n) for n in per_layer]
 
@@ -189,10 +228,14 @@ def plain_toy(w: Dict[str, torch.Tensor], cfg: ToyConfig, tokens):
     h = h + attn(1, y) + dense(1, y)
     h = h + attn(2, norm(2, "mixer_norm", h))
     h = h + routed(2, norm(2, "ffn_norm", h))
+    h = h + SANDWICH_SCALE * norm(3, "post_a", attn(3, norm(3, "pre_a", h)))
+    h = h + SANDWICH_SCALE * norm(3, "post_f", dense(3, norm(3, "pre_f", h)))
+    h = h + attn(4, norm(4, "norm", h))
     return F.linear(centred(h, "final_norm."), w["head.weight"])
 
 
 def test_toy_parts_are_registered_built_and_stepped():
+    from torchllms_amd.config.spec import LayerRun, LayerSpec, ModelSpec
     from torchllms_amd.engine import Engine
     from torchllms_amd.parts import Model
     from torchllms_amd.weights import random_tensors
@@ -203,6 +246,16 @@ def test_toy_parts_are_registered_built_and_stepped():
     # only what each layer's parts declare: no router in the dense layer, no bias under an RMS norm
     assert "layers.1.ffn.router.weight" not in expected and "layers.0.ffn.router.weight" in expected
     assert "layers.0.ffn_norm.bias" not in expected and "layers.0.mixer_norm.bias" in expected
+    # the arrangement decides which parts a layer has: one norm in the parallel layer, four in the sandwich,
+    # no feed-forward in the last
+    assert not any(n.startswith("layers.1.ffn_norm") for n in expected)
+    assert {n.split(".")[2] for n in expected if n.startswith("layers.3.")} == {"pre_a", "mixer", "post_a", "pre_f", "ffn", "post_f"}
+    assert {n.split(".")[2] for n in expected if n.startswith("layers.4.")} == {"norm", "mixer"}
+    with pytest.raises(ValueError, match="lacks \\['ffn'\\]"):
+        Model(ModelSpec("x", HIDDEN, VOCAB, 8, arch.model_spec(cfg).embedding,
+                        [LayerSpec("layers.0", "toy_parallel", {"mixer_norm": arch.model_spec(cfg).final_norm,
+                                                                "mixer": arch.model_spec(cfg).layers[0].parts["mixer"]})],
+                        [LayerRun(0)], arch.model_spec(cfg).final_norm, arch.model_spec(cfg).head))
     w = random_tensors(expected, seed=11, dtype=torch.float32, norm_jitter=0.2)
     for name in w:
         if name.endswith(("wq.weight", "wk.weight")):
@@ -220,7 +273,10 @@ def test_toy_parts_are_registered_built_and_stepped():
     pool_tokens = max(schedules.max_live_tokens(t) for t in traces.values())
     eng = Engine(arch, cfg, {k: v.to("cuda:0") for k, v in w.items()}, torch.float32, page_size=4,
                  num_pages=-(-pool_tokens // 4), max_seqs=4, max_model_len=512)
-    assert [(g.window, g.run_ids) for g in eng.cache.groups] == [(0, (0, 1, 2))] and not eng.cache.states
+    # two groups of pages: the engine's page size for four layers, the last layer's own; both hold the same tokens
+    assert [(g.page_size, g.run_ids) for g in eng.cache.groups] == [(0, tuple((i, "mixer") for i in range(4))), (WIDE_PAGE, ((4, "mixer"),))]
+    assert eng.cache.page_sizes == [4, WIDE_PAGE] and not eng.cache.states
+    assert eng.cache.pools[1].num_pages == -(-eng.cache.pools[0].num_pages * 4 // WIDE_PAGE)
     assert eng.graphs is None  # no part here says graph_safe: the routed feed-forward's launches depend on the tokens
     for name, steps in traces.items():
         got = run_trace(eng, steps)

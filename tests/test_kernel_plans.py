@@ -3,7 +3,7 @@ a sampled row, and which matrix-product kernel a tuned table sends a product to.
 
 import torch
 
-from torchllms_amd.kernels import ops
+from torchllms_amd.kernels import attention_ops, ops, products
 
 
 def test_decode_splits_cover_the_range_with_about_512_blocks():
@@ -15,7 +15,7 @@ def test_decode_splits_cover_the_range_with_about_512_blocks():
                     assert split % 64 == 0 and split >= 256
                     assert n_splits >= 1 and (n_splits - 1) * split < max(longest, 1) <= n_splits * split
                     if uneven:
-                        assert split <= ops._DECODE_UNEVEN_SPLIT == 512
+                        assert split <= attention_ops.DECODE_UNEVEN_SPLIT == 512
                     elif n_splits > 1:
                         # no more blocks than asked for, unless the shortest split allowed is reached
                         assert split == 256 or n_tokens * n_kv_heads * n_splits <= 512 + n_tokens * n_kv_heads
@@ -31,15 +31,15 @@ def test_the_tuned_table_decides_per_shape_rows_and_use():
     w = torch.zeros(96, 256, dtype=torch.bfloat16)
     x = torch.zeros(40, 256, dtype=torch.bfloat16)
     keys = [(96, 256, b, use) for b in (8, 64, 128) for use in ops.LINEAR_USES]
-    saved = {k: ops._LINEAR_CHOICE[k] for k in keys if k in ops._LINEAR_CHOICE}
+    saved = {k: products.LINEAR_CHOICE[k] for k in keys if k in products.LINEAR_CHOICE}
     try:
         for k in keys:
-            ops._LINEAR_CHOICE.pop(k, None)
+            products.LINEAR_CHOICE.pop(k, None)
         assert ops.linear_choice(x, w) is None  # 40 rows, never measured: the library
         assert ops.linear_choice(x[:8], w) == ("stream", 0)  # 8 rows, never measured: the size rule
-        ops._LINEAR_CHOICE[(96, 256, 64, "plain")] = ("wide", 1, 2, 3)
-        ops._LINEAR_CHOICE[(96, 256, 64, "glu")] = ("wide", 2, 1, 3)
-        ops._LINEAR_CHOICE[(96, 256, 8, "plain")] = None
+        products.LINEAR_CHOICE[(96, 256, 64, "plain")] = ("wide", 1, 2, 3)
+        products.LINEAR_CHOICE[(96, 256, 64, "glu")] = ("wide", 2, 1, 3)
+        products.LINEAR_CHOICE[(96, 256, 8, "plain")] = None
         assert ops.linear_choice(x, w) == ("wide", 1, 2, 3) and ops.linear_choice(x, w, "glu") == ("wide", 2, 1, 3)
         assert ops.linear_choice(x, w, "qkv") is None and ops.linear_choice(x[:8], w) is None
         assert ops.linear_choice(x[:33], w) == ("wide", 1, 2, 3)  # 33 to 64 rows share a bucket
@@ -49,18 +49,39 @@ def test_the_tuned_table_decides_per_shape_rows_and_use():
         assert ops.linear_choice(x.float(), w.float()) is None
     finally:
         for k in keys:
-            ops._LINEAR_CHOICE.pop(k, None)
-        ops._LINEAR_CHOICE.update(saved)
+            products.LINEAR_CHOICE.pop(k, None)
+        products.LINEAR_CHOICE.update(saved)
 
 
 def test_which_candidates_are_charged_a_kernel_of_their_own_for_the_second_half():
     stream, whole, split = ("stream", 4), ("wide", 2, 1, 3), ("wide", 1, 4, 3)
     for choice in (None, stream, whole, split):
-        assert ops._fuses_tail(choice, "plain") and ops._fuses_tail(choice, "sum")
-    assert [ops._fuses_tail(c, "glu") for c in (None, stream, whole, split)] == [False, True, True, False]
-    assert [ops._fuses_tail(c, "qkv") for c in (None, stream, whole, split)] == [False, True, False, True]
+        assert products.fuses_tail(choice, "plain") and products.fuses_tail(choice, "sum")
+    assert [products.fuses_tail(c, "glu") for c in (None, stream, whole, split)] == [False, True, True, False]
+    assert [products.fuses_tail(c, "qkv") for c in (None, stream, whole, split)] == [False, True, False, True]
 
 
 def test_which_launches_of_the_wide_kernel_fit_lds():
     assert ops.wide_fits(64, 2, 3) and ops.wide_fits(128, 1, 3) and ops.wide_fits(128, 2, 2) and not ops.wide_fits(128, 2, 3)
     assert ops.wide_fits(20, 2, 3) and ops.wide_fits(65, 1, 2)
+
+
+def test_the_table_survives_a_file(tmp_path):
+    saved = dict(products.LINEAR_CHOICE)
+    try:
+        products.LINEAR_CHOICE.clear()
+        products.LINEAR_CHOICE.update({(96, 256, 64, "plain"): ("wide", 2, 1, 3), (96, 256, 8, "glu"): ("stream", 4, 8),
+                                       (96, 256, 8, "plain"): None, (512, 128, 1, "qkv"): ("stream", 0)})
+        table = ops.kernel_table()
+        assert table == {"96,256,8,glu": ["stream", 4, 8], "96,256,8,plain": None, "96,256,64,plain": ["wide", 2, 1, 3],
+                         "512,128,1,qkv": ["stream", 0]}
+        assert ops.kernel_table([((96, 256), "plain")]) == {"96,256,8,plain": None, "96,256,64,plain": ["wide", 2, 1, 3]}
+        ops.save_kernel_table(tmp_path / "t.json")
+        before = dict(products.LINEAR_CHOICE)
+        ops.clear_kernel_table()
+        assert products.LINEAR_CHOICE == {}
+        ops.load_kernel_table(tmp_path / "t.json")
+        assert products.LINEAR_CHOICE == before
+    finally:
+        products.LINEAR_CHOICE.clear()
+        products.LINEAR_CHOICE.update(saved)

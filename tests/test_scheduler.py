@@ -19,13 +19,15 @@ VOCAB = 32
 
 
 class FakeEngine:
-    def __init__(self, num_pages=64, page_size=4, max_seqs=4, window=0):
-        self.cache = CacheManager([CacheGroupSpec("kv0", (0,), 1, 4, window)], [], page_size, num_pages, max_seqs)
+    def __init__(self, num_pages=64, page_size=4, max_seqs=4, window=0, groups=None):
+        groups = groups or [CacheGroupSpec("kv0", (0,), 1, 4, window)]
+        self.cache = CacheManager(groups, [], page_size, num_pages, max_seqs)
         self.calls = []  # per step: list of (rid, first position, n tokens)
 
     def step(self, entries):
-        need = sum(self.cache.new_pages_needed(e.rid, len(e.tokens)) for e in entries)
-        assert need <= self.cache.free_pages(), "the scheduler planned a step the pool cannot hold"
+        need = [sum(per_group) for per_group in zip(*(self.cache.new_pages_needed(e.rid, len(e.tokens)) for e in entries))]
+        for g, n in enumerate(need):
+            assert n <= self.cache.free_pages(g), "the scheduler planned a step the pool cannot hold"
         rows, call = [], []
         for e in entries:
             start = self.cache.extend(e.rid, len(e.tokens))
@@ -50,7 +52,7 @@ def generate(prompts, max_new_tokens=None, stop=(), engine=None, max_num_seqs=4,
     loop = GenerationLoop(engine, greedy, max_num_seqs, budget, max_model_len, chunk)
     params = [SamplingParams(max_new_tokens=max_new_tokens, stop_token_ids=stop) for _ in prompts]
     reqs = loop.run(prompts, params)
-    assert engine.cache.live == [] and engine.cache.free_pages() == engine.cache.pools[0].num_pages
+    assert engine.cache.live == [] and all(engine.cache.free_pages(g) == p.num_pages for g, p in enumerate(engine.cache.pools))
     return reqs, engine, loop
 
 
@@ -190,6 +192,54 @@ def test_random_workloads_finish_with_right_tokens(seed):
     eng.cache.check_invariants()
 
 
+def test_prompts_that_advance_side_by_side_cannot_wedge_the_pool():
+    """Portions smaller than the token budget let several prompts advance together; they can use the
+    pool up while all of them are still mid-prompt, when no decoding request is there to preempt
+    anybody.  The youngest then gives way: 10 pages of 16, two prompts of 128 tokens, budget 64,
+    portions of 32 (each request alone fits: 128 + 7 tokens need 9 pages)."""
+    eng = FakeEngine(num_pages=10, page_size=16, max_seqs=4)
+    prompts = [[1] * 128, [1] * 128]
+    reqs, _, loop = generate(prompts, max_new_tokens=8, engine=eng, budget=64, chunk=32)
+    assert [r.output for r in reqs] == [[(128 + k) % VOCAB for k in range(8)]] * 2
+    assert loop.scheduler.stats["preemptions"] >= 1
+    assert reqs[0].preemptions == 0  # the oldest always gets on
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_portions_and_pools_always_finish(seed):
+    """Random portion sizes, token budgets, pools that barely hold the longest request, and two
+    groups of layers with different page sizes: every request finishes with the right tokens, and
+    the books of the cache are right after every step (the fake engine checks them)."""
+    rng = random.Random(1000 + seed)
+    n = rng.randint(2, 9)
+    prompts = [[1] * rng.randint(1, 90) for _ in range(n)]
+    news = [rng.randint(1, 12) for _ in range(n)]
+    longest = max(len(p) + m for p, m in zip(prompts, news))
+    pages = [rng.choice([2, 4, 8, 16]) for _ in range(rng.choice([1, 1, 2]))]
+    groups = [CacheGroupSpec(f"kv{g}", ((g, "mixer"),), 1, 4, 0, page_size=p) for g, p in enumerate(pages)]
+    slack = rng.randint(0, 5)
+    num_pages = {f"kv{g}": -(-longest // p) + slack for g, p in enumerate(pages)}
+    eng = FakeEngine(num_pages=num_pages, page_size=pages[0], max_seqs=rng.randint(1, 4), groups=groups)
+    loop = GenerationLoop(eng, greedy, rng.randint(1, 4), rng.choice([2, 5, 16, 64]), 256, rng.choice([None, 1, 3, 7, 32]))
+    reqs = loop.run(prompts, [SamplingParams(max_new_tokens=m) for m in news])
+    for p, m, r in zip(prompts, news, reqs):
+        assert r.output == [(len(p) + k) % VOCAB for k in range(m)]
+    assert eng.cache.live == []
+    eng.cache.check_invariants()
+
+
+def test_groups_with_different_page_sizes_are_counted_each_for_itself():
+    """A group with pages of 16 and one with pages of 4: the small pages run out first, and the
+    scheduler must see that although the first group has room."""
+    groups = [CacheGroupSpec("kv0", ("a",), 1, 4, 0, page_size=16), CacheGroupSpec("kv1", ("b",), 1, 4, 0, page_size=4)]
+    eng = FakeEngine(num_pages={"kv0": 8, "kv1": 12}, page_size=16, max_seqs=4, groups=groups)  # 128 and 48 tokens
+    reqs, _, loop = generate([[1] * 20, [1] * 20], max_new_tokens=12, engine=eng)
+    assert [r.output for r in reqs] == [[(20 + k) % VOCAB for k in range(12)]] * 2
+    assert loop.scheduler.stats["preemptions"] >= 1  # 2 * 31 tokens do not fit 48 places
+    with pytest.raises(ValueError, match="could never finish"):
+        loop.scheduler.add("big", [1] * 40, SamplingParams(max_new_tokens=12))  # 51 tokens need 13 small pages
+
+
 def test_sampling_counter_survives_preemption():
     """The sampler sees (seed, number of tokens generated so far): recomputation after a preemption
     asks for the same draws again."""
@@ -256,7 +306,7 @@ class AheadEngine(FakeEngine):
     def prepare_decode(self):
         if self._decoded is None:
             return None
-        need = sum(self.cache.new_pages_needed(r, 1) for r in self._decoded)
+        need = sum(self.cache.new_pages_needed(r, 1)[0] for r in self._decoded)
         if need > self.cache.free_pages():
             return None
         for r in self._decoded:

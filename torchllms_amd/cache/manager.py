@@ -1,9 +1,10 @@
 """Cache manager: keys and values in fixed-size pages with a block table per request, and
 slots for per-request state of fixed size.
 
-Layers whose needs are alike (same heads, head size and window) form a *group*.  A group owns a
-pool of pages; one page id addresses the same token range in every layer of the group.  A
-request holds one block table per group (logical block -> page id).  Pages go back to the pool
+Layers whose needs are alike (same heads, head size, window, tokens per page and element type) form
+a *group*.  A group owns a pool of pages; one page id addresses the same token range in every layer
+of the group.  A request holds one block table per group (logical block -> page id); groups may
+differ in page size, so their tables differ in length and their pools in the pages a step takes.  Pages go back to the pool
 when the request ends and, in a group with a window, as soon as the window has passed them.
 
 The bookkeeping is plain host code and runs without a GPU; the page tensors are optional so the
@@ -39,10 +40,12 @@ class CacheGroupSpec:
     """Layers (runs of the execution order) that share one page pool."""
 
     name: str
-    run_ids: Tuple[int, ...]
+    run_ids: Tuple[Hashable, ...]  # keys of the cache entries (one per layer run and mixer) that live in this group
     num_kv_heads: int
     head_dim: int
     window: int = 0  # 0: all keys stay; w > 0: only the last w positions are read
+    page_size: int = 0  # tokens per page; 0: the manager's default
+    dtype: Optional[str] = None  # "float32" / "bfloat16"; None: the manager's default
 
 
 @dataclass(frozen=True)
@@ -50,28 +53,31 @@ class StateSlotSpec:
     """Fixed-size per-request state of some runs: one tensor [runs, max_seqs, *shape]."""
 
     name: str
-    run_ids: Tuple[int, ...]
+    run_ids: Tuple[Hashable, ...]
     shape: Tuple[int, ...]
     dtype: str = "float32"
 
 
-def group_layers(needs: Sequence[Tuple[int, object]]) -> Tuple[List[CacheGroupSpec], List[StateSlotSpec]]:
-    """Group ``(run id, need)`` pairs: KV needs by (heads, head size, window), state needs by
-    (shape, dtype).  ``need`` is a ``parts.base.KVNeed`` / ``StateNeed`` (duck-typed) or None."""
-    kv: Dict[Tuple[int, int, int], List[int]] = {}
-    st: Dict[Tuple[Tuple[int, ...], str], List[int]] = {}
+def group_layers(needs: Sequence[Tuple[Hashable, object]]) -> Tuple[List[CacheGroupSpec], List[StateSlotSpec]]:
+    """Group ``(cache entry key, need)`` pairs: KV needs by (heads, head size, window, page size,
+    dtype), state needs by (shape, dtype).  ``need`` is a ``parts.base.KVNeed`` / ``StateNeed``
+    (duck-typed) or None."""
+    kv: Dict[tuple, List[Hashable]] = {}
+    st: Dict[Tuple[Tuple[int, ...], str], List[Hashable]] = {}
     for run_id, need in needs:
         if need is None:
             continue
         if hasattr(need, "num_kv_heads"):
-            kv.setdefault((need.num_kv_heads, need.head_dim, need.window), []).append(run_id)
+            form = (need.num_kv_heads, need.head_dim, need.window, int(getattr(need, "page_size", None) or 0),
+                    getattr(need, "dtype", None))
+            kv.setdefault(form, []).append(run_id)
         elif hasattr(need, "shape"):
             st.setdefault((tuple(need.shape), need.dtype), []).append(run_id)
         else:
-            raise TypeError(f"run {run_id}: unknown cache need {need!r}")
+            raise TypeError(f"cache entry {run_id}: unknown cache need {need!r}")
     groups = [
-        CacheGroupSpec(name=f"kv{i}", run_ids=tuple(runs), num_kv_heads=h, head_dim=d, window=w)
-        for i, ((h, d, w), runs) in enumerate(kv.items())
+        CacheGroupSpec(name=f"kv{i}", run_ids=tuple(runs), num_kv_heads=h, head_dim=d, window=w, page_size=p, dtype=t)
+        for i, ((h, d, w, p, t), runs) in enumerate(kv.items())
     ]
     states = [
         StateSlotSpec(name=f"state{i}", run_ids=tuple(runs), shape=shape, dtype=dtype)
@@ -164,13 +170,19 @@ class CacheManager:
         dtype: torch.dtype = torch.float32,
         device: Optional[str] = None,
     ):
-        """``num_pages``: an int (every group) or a dict group name -> pages.  ``device`` None:
-        bookkeeping only, no tensors."""
+        """``page_size`` and ``dtype``: what a group has that names none of its own.  ``num_pages``:
+        an int (every group) or a dict group name -> pages.  ``device`` None: bookkeeping only, no
+        tensors."""
         if page_size <= 0 or max_seqs <= 0:
             raise ValueError("page_size and max_seqs must be positive")
         self.groups = list(groups)
         self.states = list(states)
         self.page_size = page_size
+        #: tokens per page of every group
+        self.page_sizes: List[int] = [g.page_size or page_size for g in self.groups]
+        self.dtypes: List[torch.dtype] = [getattr(torch, g.dtype) if g.dtype else dtype for g in self.groups]
+        if any(p <= 0 for p in self.page_sizes):
+            raise ValueError(f"page sizes must be positive, got {self.page_sizes}")
         self.max_seqs = max_seqs
         self.dtype = dtype
         self.device = device
@@ -185,9 +197,9 @@ class CacheManager:
         #: requests, slots and pages at the same epoch only
         self.epoch = 0
         self._free_slots: List[int] = list(range(max_seqs - 1, -1, -1))
-        # run id -> (group index, layer index inside the group) / (state index, layer index)
-        self._run_to_kv: Dict[int, Tuple[int, int]] = {}
-        self._run_to_state: Dict[int, Tuple[int, int]] = {}
+        # cache entry key -> (group index, layer index inside the group) / (state index, layer index)
+        self._run_to_kv: Dict[Hashable, Tuple[int, int]] = {}
+        self._run_to_state: Dict[Hashable, Tuple[int, int]] = {}
         for gi, g in enumerate(self.groups):
             for li, run in enumerate(g.run_ids):
                 self._run_to_kv[run] = (gi, li)
@@ -198,23 +210,34 @@ class CacheManager:
         self.v_pages: List[Optional[torch.Tensor]] = []
         self.state_tensors: List[Optional[torch.Tensor]] = []
         if device is not None:
-            for g, pool in zip(self.groups, self.pools):
-                shape = (len(g.run_ids), pool.num_pages, g.num_kv_heads, page_size, g.head_dim)
-                self.k_pages.append(torch.zeros(shape, dtype=dtype, device=device))
-                self.v_pages.append(torch.zeros(shape, dtype=dtype, device=device))
+            for gi, (g, pool) in enumerate(zip(self.groups, self.pools)):
+                shape = (len(g.run_ids), pool.num_pages, g.num_kv_heads, self.page_sizes[gi], g.head_dim)
+                self.k_pages.append(torch.zeros(shape, dtype=self.dtypes[gi], device=device))
+                self.v_pages.append(torch.zeros(shape, dtype=self.dtypes[gi], device=device))
             for s in self.states:
                 shape = (len(s.run_ids), max_seqs, *s.shape)
                 self.state_tensors.append(torch.zeros(shape, dtype=getattr(torch, s.dtype), device=device))
+        self._views: Dict[Tuple[Hashable, bool], object] = {}
 
     # ------------------------------------------------------------------ sizes
     @staticmethod
-    def bytes_per_page(groups: Sequence[CacheGroupSpec], page_size: int, dtype: torch.dtype) -> int:
-        """Bytes one page id costs summed over all groups (keys and values, every layer)."""
-        elt = torch.empty(0, dtype=dtype).element_size()
-        return sum(2 * len(g.run_ids) * g.num_kv_heads * g.head_dim * page_size * elt for g in groups)
+    def bytes_per_token(groups: Sequence[CacheGroupSpec], dtype: torch.dtype) -> int:
+        """Bytes one cached token costs summed over all groups (keys and values, every layer)."""
+        total = 0
+        for g in groups:
+            elt = torch.empty(0, dtype=getattr(torch, g.dtype) if g.dtype else dtype).element_size()
+            total += 2 * len(g.run_ids) * g.num_kv_heads * g.head_dim * elt
+        return total
 
-    def blocks_for(self, n_tokens: int) -> int:
-        return -(-n_tokens // self.page_size)
+    @staticmethod
+    def pages_for_tokens(groups: Sequence[CacheGroupSpec], page_size: int, n_tokens: int) -> Dict[str, int]:
+        """Pages per group (by name) that hold ``n_tokens`` tokens, at least one each."""
+        return {g.name: max(-(-n_tokens // (g.page_size or page_size)), 1) for g in groups}
+
+    def blocks_for(self, n_tokens: int, group: int = 0) -> int:
+        """Pages of ``group`` that ``n_tokens`` tokens of one request occupy."""
+        page = self.page_sizes[group] if self.page_sizes else self.page_size
+        return -(-n_tokens // page)
 
     # ------------------------------------------------------------------ requests
     def has(self, rid: Hashable) -> bool:
@@ -287,24 +310,26 @@ class CacheManager:
         if w <= 0:
             return 0
         lo = first_query_pos - w + 1
-        return max(lo, 0) // self.page_size
+        return max(lo, 0) // self.page_sizes[group]
 
     def pages_short(self, rid: Hashable, n_new: int) -> Dict[int, int]:
         """Per group, how many pages are missing to take ``n_new`` more tokens (0 if it fits)."""
         e = self.entry(rid)
-        need_blocks = self.blocks_for(e.num_tokens + n_new)
         out = {}
         for gi, pool in enumerate(self.pools):
-            extra = max(need_blocks - len(e.block_tables[gi]), 0)
+            extra = max(self.blocks_for(e.num_tokens + n_new, gi) - len(e.block_tables[gi]), 0)
             out[gi] = max(extra - pool.free_count, 0)
         return out
 
-    def new_pages_needed(self, rid: Hashable, n_new: int) -> int:
-        """Pages per group that taking ``n_new`` more tokens allocates (same for every group)."""
+    def new_pages_needed(self, rid: Hashable, n_new: int) -> List[int]:
+        """Per group, the pages that taking ``n_new`` more tokens allocates."""
         e = self.entry(rid)
-        if not self.groups:
-            return 0
-        return max(self.blocks_for(e.num_tokens + n_new) - len(e.block_tables[0]), 0)
+        total = e.num_tokens + n_new
+        return [max(self.blocks_for(total, gi) - len(e.block_tables[gi]), 0) for gi in range(len(self.groups))]
+
+    def pages_for_new_request(self, n_tokens: int) -> List[int]:
+        """Per group, the pages that the first ``n_tokens`` tokens of a request take."""
+        return [self.blocks_for(n_tokens, gi) for gi in range(len(self.groups))]
 
     def can_extend(self, rid: Hashable, n_new: int) -> bool:
         return all(v == 0 for v in self.pages_short(rid, n_new).values())
@@ -316,7 +341,7 @@ class CacheManager:
             raise ValueError("n_new must be >= 0")
         e = self.entry(rid)
         total = e.num_tokens + n_new
-        if all(total <= len(bt) * self.page_size for bt in e.block_tables):
+        if all(total <= len(bt) * page for bt, page in zip(e.block_tables, self.page_sizes)):
             # the pages it holds have room (most decode steps): nothing to take
             e.reserved_tokens = max(e.reserved_tokens, total)
             return e.num_tokens
@@ -326,20 +351,19 @@ class CacheManager:
                 f"request {rid!r}: {n_new} more tokens after {e.num_tokens} need pages a pool lacks "
                 f"(missing per group: { {self.groups[g].name: s for g, s in short.items() if s} })"
             )
-        need_blocks = self.blocks_for(e.num_tokens + n_new)
         for gi, pool in enumerate(self.pools):
-            extra = need_blocks - len(e.block_tables[gi])
+            extra = self.blocks_for(total, gi) - len(e.block_tables[gi])
             if extra > 0:
                 e.block_tables[gi].extend(pool.take(extra))
                 e.table_arrays[gi] = None
-        e.reserved_tokens = max(e.reserved_tokens, e.num_tokens + n_new)
+        e.reserved_tokens = max(e.reserved_tokens, total)
         return e.num_tokens
 
     def advance(self, rid: Hashable, n_new: int) -> None:
         """``n_new`` tokens were written.  Pages a window has passed go back to their pool."""
         e = self.entry(rid)
-        for bt in e.block_tables:
-            if e.num_tokens + n_new > len(bt) * self.page_size:
+        for bt, page in zip(e.block_tables, self.page_sizes):
+            if e.num_tokens + n_new > len(bt) * page:
                 raise RuntimeError(f"request {rid!r}: advancing past the pages it holds (extend first)")
         e.num_tokens += n_new
         if not self._windowed:
@@ -361,9 +385,9 @@ class CacheManager:
         e = self.entry(rid)
         if not 0 <= num_tokens <= e.num_tokens:
             raise ValueError(f"cannot truncate request {rid!r} from {e.num_tokens} to {num_tokens} tokens")
-        keep = self.blocks_for(num_tokens)
         for gi, pool in enumerate(self.pools):
             bt = e.block_tables[gi]
+            keep = self.blocks_for(num_tokens, gi)
             if keep < e.first_live_block[gi]:
                 raise ValueError("cannot truncate into pages a window has already released")
             tail = [p for p in bt[keep:] if p >= 0]
@@ -385,40 +409,53 @@ class CacheManager:
         self._free_slots.append(e.slot)
 
     # ------------------------------------------------------------------ views for the model
-    def kv_view(self, run_id: int, writes: bool = True) -> KVLayerView:
+    def kv_view(self, run_id: Hashable, writes: bool = True) -> KVLayerView:
         gi, li = self._run_to_kv[run_id]
         return KVLayerView(
             group=gi,
             k_pages=self.k_pages[gi][li],
             v_pages=self.v_pages[gi][li],
-            page_size=self.page_size,
+            page_size=self.page_sizes[gi],
             writes=writes,
         )
 
-    def state_view(self, run_id: int) -> StateView:
+    def state_view(self, run_id: Hashable) -> StateView:
         si, li = self._run_to_state[run_id]
         return StateView(tensor=self.state_tensors[si][li])
 
-    def view_for_run(self, run_id: int, cache_from: Optional[int] = None):
-        src = run_id if cache_from is None else cache_from
-        if src in self._run_to_kv:
-            return self.kv_view(src, writes=cache_from is None)
-        if src in self._run_to_state:
-            return self.state_view(src)
-        return None
+    def view(self, key: Hashable, writes: bool = True):
+        """What is held under the cache entry ``key``: a ``KVLayerView`` (``writes`` False for a run
+        that borrows another run's entry), a ``StateView``, or None when the entry needs nothing.
+        The views are made once and kept: the tensors they point at never move."""
+        try:
+            return self._views[(key, writes)]
+        except KeyError:
+            pass
+        if key in self._run_to_kv:
+            v = self.kv_view(key, writes)
+        elif key in self._run_to_state:
+            v = self.state_view(key)
+        else:
+            v = None
+        self._views[(key, writes)] = v
+        return v
 
-    def gather_kv(self, rid: Hashable, run_id: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    def view_for_run(self, run_id: Hashable, cache_from: Optional[Hashable] = None):
+        return self.view(run_id if cache_from is None else cache_from, writes=cache_from is None)
+
+    def gather_kv(self, rid: Hashable, run_id: Hashable) -> Tuple[torch.Tensor, torch.Tensor]:
         """Keys and values of a request in position order, [n, Hkv, dh] each (debugging, tests).
         Positions whose page a window released come back as zeros."""
         gi, li = self._run_to_kv[run_id]
         e = self.entry(rid)
         g = self.groups[gi]
+        page_size = self.page_sizes[gi]
         n = e.num_tokens
-        k = torch.zeros((n, g.num_kv_heads, g.head_dim), dtype=self.dtype, device=self.device)
+        k = torch.zeros((n, g.num_kv_heads, g.head_dim), dtype=self.dtypes[gi], device=self.device)
         v = torch.zeros_like(k)
         for b, page in enumerate(e.block_tables[gi]):
-            lo = b * self.page_size
-            hi = min(lo + self.page_size, n)
+            lo = b * page_size
+            hi = min(lo + page_size, n)
             if page < 0 or lo >= n:
                 continue
             k[lo:hi] = self.k_pages[gi][li, page, :, : hi - lo].transpose(0, 1)
@@ -435,8 +472,8 @@ class CacheManager:
                 bt = e.block_tables[gi]
                 if e.table_arrays[gi] is not None and e.table_arrays[gi].tolist() != bt:
                     raise AssertionError(f"{rid!r}: the cached array of group {gi}'s block table is stale")
-                need = self.blocks_for(max(e.num_tokens, e.reserved_tokens))
-                if len(bt) < self.blocks_for(e.num_tokens):
+                need = self.blocks_for(max(e.num_tokens, e.reserved_tokens), gi)
+                if len(bt) < self.blocks_for(e.num_tokens, gi):
                     raise AssertionError(f"{rid!r}: {len(bt)} blocks for {e.num_tokens} tokens")
                 if len(bt) > need:
                     raise AssertionError(f"{rid!r}: holds {len(bt)} blocks, needs at most {need}")

@@ -7,7 +7,7 @@ from .registry import (
     load_config,
     register_architecture,
 )
-from .spec import LayerRun, LayerSpec, ModelSpec, PartSpec
+from .spec import LayerRun, LayerSpec, ModelSpec, PartSpec, standard_layer
 
 __all__ = [
     "ARCHITECTURES",
@@ -24,4 +24,5 @@ __all__ = [
     "llama_model_spec",
     "load_config",
     "register_architecture",
+    "standard_layer",
 ]

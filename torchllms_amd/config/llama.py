@@ -14,7 +14,7 @@ from dataclasses import dataclass, field, fields
 from pathlib import Path
 from typing import Any, Dict, List, Optional
 
-from .spec import LayerRun, LayerSpec, ModelSpec, PartSpec
+from .spec import LayerRun, LayerSpec, ModelSpec, PartSpec, standard_layer
 
 _ROPE_SCALING_KEYS = (
     "factor",
@@ -232,14 +232,7 @@ def llama_model_spec(cfg: LlamaConfig) -> ModelSpec:
     )
     ffn = PartSpec("swiglu", dict(hidden_size=cfg.hidden_size, intermediate_size=cfg.intermediate_size))
     layers: List[LayerSpec] = [
-        LayerSpec(
-            name=f"layers.{i}",
-            block="pre_norm",
-            mixer=mixer,
-            feed_forward=ffn,
-            mixer_norm=norm,
-            ffn_norm=norm,
-        )
+        standard_layer(f"layers.{i}", "pre_norm", mixer=mixer, feed_forward=ffn, mixer_norm=norm, ffn_norm=norm)
         for i in range(cfg.num_hidden_layers)
     ]
     spec = ModelSpec(

@@ -22,17 +22,32 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer = an arrangement (``block``) of a mixer, a feed-forward and their norms.
+    """One layer = an arrangement (``block``, a key of the block registry) and the parts it arranges.
 
-    ``name`` is the prefix of the layer's tensors inside the model ("layers.3").
+    ``parts`` maps the arrangement's slot names to parts.  Which slots there are, and which kind of
+    part each takes (mixer, feed-forward, norm), is the arrangement's own business: a pre-norm
+    block has ``mixer_norm``, ``mixer``, ``ffn_norm`` and ``ffn``; one with norms on both sides of
+    every branch has six; one without a feed-forward has two.  ``block_params`` are further keyword
+    arguments of the arrangement (a residual scale, say).
+    ``name`` is the prefix of the layer's tensors inside the model ("layers.3"); a sub-part's
+    tensors follow as ``<name>.<slot>.<tensor>``.
     """
 
     name: str
     block: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    parts: Dict[str, PartSpec]
+    block_params: Dict[str, Any] = field(default_factory=dict)
+
+
+def standard_layer(name: str, block: str, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec,
+                   ffn_norm: PartSpec, **block_params: Any) -> LayerSpec:
+    """A layer of the common four parts under their usual slot names."""
+    return LayerSpec(
+        name=name,
+        block=block,
+        parts={"mixer_norm": mixer_norm, "mixer": mixer, "ffn_norm": ffn_norm, "ffn": feed_forward},
+        block_params=dict(block_params),
+    )
 
 
 @dataclass(frozen=True)

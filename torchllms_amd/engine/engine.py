@@ -72,57 +72,84 @@ class Engine:
         device="cuda:0",
         use_graphs: bool = True,
         tune_kernels: bool = True,
+        kernel_table=None,
     ):
         """``tensors``: the model's tensors under the parts' own names, on ``device``.
-        Pool size: ``num_pages`` pages per group, else what ``kv_memory_gb`` holds, else
-        ``kv_memory_fraction`` of the device memory that is free once the weights are loaded, else
-        room for ``max_seqs`` requests of ``max_model_len`` tokens (reference: networks.py:872-884)."""
+        Pool size: room for ``num_pages`` pages of ``page_size`` tokens, else what ``kv_memory_gb``
+        holds, else ``kv_memory_fraction`` of the device memory that is free once the weights are
+        loaded, else room for ``max_seqs`` requests of ``max_model_len`` tokens (reference:
+        networks.py:872-884); a group of layers with a page size of its own gets as many pages as
+        hold the same number of tokens.
+
+        Which bfloat16 matrix-product kernel serves a decode step is looked up in a table by shape,
+        row count and use.  ``kernel_table`` (a dict as ``kernel_table()`` returns, or the path of a
+        JSON file of one) fills the table first; ``tune_kernels`` then measures what the table does
+        not hold yet.  Kernels differ in rounding, so two processes agree bit for bit in bfloat16
+        only when they run from the same table; with ``tune_kernels=False`` and no table every shape
+        follows a fixed rule of sizes (``ops.linear_choice``)."""
         self.device = require_gpu(device)
         self.arch = arch
         self.config = config
         self.dtype = dtype
         self.spec = arch.model_spec(config)
         self.model = Model(self.spec)
+        # a size that no kernel takes is refused here, not at the first step
+        self.model.check_sizes(dtype)
+        if page_size <= 0:
+            raise ValueError(f"page_size must be positive, got {page_size}")
         self.model.bind(tensors)
         self.vocab_size = self.spec.vocab_size
         self.max_model_len = int(max_model_len or self.spec.max_positions)
         self.page_size = page_size
+        from ..kernels import ops
+
+        if kernel_table is not None:
+            ops.load_kernel_table(kernel_table)
         if dtype == torch.bfloat16 and tune_kernels:
             # which matrix-product kernel serves decode steps best is measured, not guessed; before
             # the pool is sized, so that what the measurement borrows is free again for pages
-            from ..kernels import ops
-
-            for (shape, use), group in self.model.linear_weights().items():
-                ops.tune_linear(group, torch.float32 if group[0] is self.model.head.weight else torch.bfloat16, use)
+            for (shape, use, out_dtype), group in self.model.linear_weights().items():
+                ops.tune_linear(group, out_dtype or torch.bfloat16, use)
             torch.cuda.empty_cache()
         groups, states = group_layers(self.model.cache_needs())
-        if num_pages is None:
-            per_page = CacheManager.bytes_per_page(groups, page_size, dtype)
-            if kv_memory_gb is not None and per_page > 0:
-                num_pages = max(int(kv_memory_gb * (1 << 30)) // per_page, 1)
-            elif kv_memory_fraction is not None and per_page > 0:
-                if not 0.0 < kv_memory_fraction <= 1.0:
-                    raise ValueError(f"kv_memory_fraction must lie in (0, 1], got {kv_memory_fraction}")
-                free_bytes, _ = torch.cuda.mem_get_info(self.device)
-                num_pages = max(int(free_bytes * kv_memory_fraction) // per_page, 1)
+        if isinstance(num_pages, dict):
+            pages = dict(num_pages)
+        else:
+            if num_pages is not None:
+                capacity = int(num_pages) * page_size
             else:
-                num_pages = max_seqs * (-(-self.max_model_len // page_size))
-        self.cache = CacheManager(groups, states, page_size, num_pages, max_seqs, dtype=dtype, device=self.device)
+                per_token = CacheManager.bytes_per_token(groups, dtype)
+                if kv_memory_gb is not None and per_token > 0:
+                    capacity = int(kv_memory_gb * (1 << 30)) // per_token
+                elif kv_memory_fraction is not None and per_token > 0:
+                    if not 0.0 < kv_memory_fraction <= 1.0:
+                        raise ValueError(f"kv_memory_fraction must lie in (0, 1], got {kv_memory_fraction}")
+                    free_bytes, _ = torch.cuda.mem_get_info(self.device)
+                    capacity = int(free_bytes * kv_memory_fraction) // per_token
+                else:
+                    capacity = max_seqs * (-(-self.max_model_len // page_size)) * page_size
+            pages = CacheManager.pages_for_tokens(groups, page_size, max(capacity, 1))
+        self.cache = CacheManager(groups, states, page_size, pages, max_seqs, dtype=dtype, device=self.device)
         self._windowed = any(g.window > 0 for g in groups)
         self.steps_run = 0
         self.tokens_run = 0
         # the last step's plan when every row of it brought one token: (request ids, wanted places,
         # layout); a decode step that follows it with the same requests is planned from it
         self._last_decode = None
-        # decode steps are replayed from HIP graphs when every mixer's launches are fixed by the
+        # decode steps are replayed from HIP graphs when every part's launches are fixed by the
         # step's shape alone
         from .graphs import DecodeGraphs
 
-        parts = [self.model.embedding, self.model.final_norm, self.model.head]
-        for b in self.model.blocks:
-            parts += [b, b.mixer, b.feed_forward, b.mixer_norm, b.ffn_norm]
-        graph_safe = all(getattr(p, "graph_safe", False) for p in parts)
-        self.graphs = DecodeGraphs(self.model, self.cache, self.device, page_size) if (use_graphs and graph_safe) else None
+        graph_safe = all(getattr(p, "graph_safe", False) for p in self.model.all_parts())
+        self.graphs = DecodeGraphs(self.model, self.cache, self.device) if (use_graphs and graph_safe) else None
+
+    def kernel_table(self) -> dict:
+        """The table entries of this model's matrices (JSON-able): hand it to another engine, or
+        save it with ``ops.save_kernel_table``, to run the same kernels in another process."""
+        from ..kernels import ops
+
+        shapes = {(shape, use) for (shape, use, _), group in self.model.linear_weights().items()}
+        return ops.kernel_table(shapes)
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -133,8 +160,10 @@ class Engine:
         dtype = parse_dtype(dtype)
         arch, config = load_config(folder)
         spec = arch.model_spec(config)
-        expected = Model(spec).param_specs()
-        ignore = ["head.weight"] if "head.weight" not in expected else []
+        model = Model(spec)
+        model.check_sizes(dtype)  # before the weights are read: a refusal costs nothing
+        expected = model.param_specs()
+        ignore = model.ignorable_tensors()
         tensors = load_weights(folder, arch.weight_rules(config), expected, dtype, device=device, ignore_when_present=ignore)
         return cls(arch, config, tensors, dtype, device=device, **kw)
 
@@ -146,7 +175,9 @@ class Engine:
         device = require_gpu(device)
         dtype = parse_dtype(dtype)
         arch = get_architecture(config.architectures[0])
-        expected = Model(arch.model_spec(config)).param_specs()
+        model = Model(arch.model_spec(config))
+        model.check_sizes(dtype)
+        expected = model.param_specs()
         if draw_on_device:
             tensors = random_tensors(expected, seed, dtype, norm_jitter, device=device)
         else:
@@ -200,33 +231,39 @@ class Engine:
             return None
         n = len(rids)
         held = prev.kv_lens.tolist()
-        page = self.page_size
         get = cache.get
-        need = 0
         for rid, have in zip(rids, held):
             live = get(rid)
             if live is None or live.num_tokens != have:
                 return None
-            if have % page == 0:  # the new token opens a page
-                need += cache.new_pages_needed(rid, 1)
         if max(held) + 1 > self.max_model_len:
             return None
-        if any(need > pool.free_count for pool in cache.pools):
-            return None
         positions = prev.kv_lens.copy()  # the new token's position = tokens held so far
-        fresh = (positions % page) == 0  # rows whose new token opens a page; the others have room
-        for i in np.nonzero(fresh)[0]:
-            cache.extend(rids[i], 1)
+        # rows whose new token opens a page, per group; the others have room
+        fresh = [(positions % page) == 0 for page in cache.page_sizes]
+        opening = np.zeros(n, dtype=bool)
+        for f in fresh:
+            opening |= f
+        opening = np.nonzero(opening)[0]
+        if opening.size:
+            need = [0] * len(cache.pools)
+            for i in opening:  # (a page taken by an earlier preparation of this very step is not needed again)
+                for g, pages in enumerate(cache.new_pages_needed(rids[i], 1)):
+                    need[g] += pages
+            if any(k > pool.free_count for k, pool in zip(need, cache.pools)):
+                return None
+            for i in opening:
+                cache.extend(rids[i], 1)
         tables, slots = [], []
-        for g in range(len(cache.groups)):
+        for g, page in enumerate(cache.page_sizes):
             bt = prev.block_tables[g]
             sm = prev.slot_mappings[g] + 1
-            if fresh.any():
+            if fresh[g].any():
                 width = max(bt.shape[1], int(positions.max()) // page + 1)
                 wider = np.full((n, width), -1, dtype=np.int32)
                 wider[:, : bt.shape[1]] = bt
                 bt = wider
-                for i in np.nonzero(fresh)[0]:
+                for i in np.nonzero(fresh[g])[0]:
                     blk = int(positions[i]) // page
                     bt[i, blk] = cache.block_table(rids[i], g)[blk]
                     sm[i] = bt[i, blk] * page
@@ -235,8 +272,8 @@ class Engine:
         return StepLayout(
             n_tokens=n, n_seqs=n, n_decode=n, row_of_entry=prev.row_of_entry, tokens=np.zeros(n, dtype=np.int32),
             positions=positions, token_seq=prev.token_seq, qo_indptr=prev.qo_indptr, kv_lens=positions + 1,
-            slot_ids=prev.slot_ids, logit_rows=prev.logit_rows, block_tables=tables, slot_mappings=slots, page_size=page,
-            max_q_len=1, max_kv_len=int(positions.max()) + 1,
+            slot_ids=prev.slot_ids, logit_rows=prev.logit_rows, block_tables=tables, slot_mappings=slots,
+            page_sizes=list(cache.page_sizes), max_q_len=1, max_kv_len=int(positions.max()) + 1,
         )
 
     # ------------------------------------------------------------------ one step ahead
@@ -329,16 +366,19 @@ class Engine:
                     f"request {e.rid!r}: {self.cache.num_tokens(e.rid)} + {n} tokens exceed max_model_len={self.max_model_len}"
                 )
         # all-or-nothing over the whole batch: count the pages the step takes from every pool
-        need = sum(self.cache.new_pages_needed(e.rid, len(e.tokens)) for e in entries)
+        need = [0] * len(self.cache.pools)
+        for e in entries:
+            for gi, pages in enumerate(self.cache.new_pages_needed(e.rid, len(e.tokens))):
+                need[gi] += pages
         for gi, pool in enumerate(self.cache.pools):
-            if need > pool.free_count:
+            if need[gi] > pool.free_count:
                 raise OutOfPages(
-                    f"step needs {need} new pages in group {self.cache.groups[gi].name}, {pool.free_count} are free"
+                    f"step needs {need[gi]} new pages in group {self.cache.groups[gi].name}, {pool.free_count} are free"
                 )
         starts = [self.cache.extend(e.rid, len(e.tokens)) for e in entries]
         slots = [self.cache.slot(e.rid) for e in entries]
         tables = [[self.cache.block_table_array(e.rid, g) for e in entries] for g in range(len(self.cache.groups))]
-        return build_step_layout(entries, starts, slots, tables, self.page_size)
+        return build_step_layout(entries, starts, slots, tables, self.cache.page_sizes)
 
     @torch.inference_mode()
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -347,11 +387,19 @@ class Engine:
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
         layout = self.plan(entries)
-        if self.graphs is not None and layout.n_decode == layout.n_seqs:
-            logits = self.graphs.run(layout)
-        else:
-            ctx = upload(layout, self.device)
-            logits = self.model.forward(ctx, self.cache)
+        try:
+            if self.graphs is not None and layout.n_decode == layout.n_seqs:
+                logits = self.graphs.run(layout)
+            else:
+                ctx = upload(layout, self.device)
+                logits = self.model.forward(ctx, self.cache)
+        except BaseException:
+            # nothing of the step is booked: the pages taken for it go back, and no later step is
+            # planned from this one's plan
+            self._last_decode = None
+            for e in entries:
+                self.cache.truncate(e.rid, self.cache.num_tokens(e.rid))
+            raise
         for e in entries:
             self.cache.advance(e.rid, len(e.tokens))
         self.steps_run += 1

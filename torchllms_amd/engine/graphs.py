@@ -39,15 +39,14 @@ class DecodeGraph:
     owns it: a reference cycle would leave the graph to the cyclic garbage collector, which may
     run, and destroy the graph, in the middle of somebody else's stream capture."""
 
-    def __init__(self, model, cache, device, page_size: int, layout: StepLayout, cap: int, pool=None, uneven: bool = False):
+    def __init__(self, model, cache, device, layout: StepLayout, cap: int, pool=None, uneven: bool = False):
         self.model = model
         self.cache = cache
         self.cap = cap
         self.uneven = uneven
         self.pool = pool
-        width = -(-cap // page_size)
-        n_groups = len(layout.block_tables)
-        self.shapes = section_shapes(layout.n_tokens, layout.n_seqs, layout.logit_rows.size, [width] * n_groups)
+        widths = [-(-cap // page) for page in layout.page_sizes]  # a group's block table up to the context cap
+        self.shapes = section_shapes(layout.n_tokens, layout.n_seqs, layout.logit_rows.size, widths)
         self.offsets, total = section_offsets(self.shapes)
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
         self.host_np = self.host.numpy()
@@ -125,11 +124,10 @@ class DecodeGraphs:
     new shape that never returns).  All recordings share one memory pool: they are replayed one at
     a time and a step's logits are copied out before the next replay."""
 
-    def __init__(self, model, cache, device, page_size: int, max_graphs: int = 128, record_after: int = 2):
+    def __init__(self, model, cache, device, max_graphs: int = 128, record_after: int = 2):
         self.model = model
         self.cache = cache
         self.device = device
-        self.page_size = page_size
         self.max_graphs = max_graphs
         self.record_after = record_after
         self.graphs: Dict[Tuple[int, int, int, bool], DecodeGraph] = {}
@@ -160,6 +158,9 @@ class DecodeGraphs:
             self.graphs.pop(next(iter(self.graphs)))
         if self.pool is None:
             self.pool = torch.cuda.graph_pool_handle()
-        g = DecodeGraph(self.model, self.cache, self.device, self.page_size, layout, cap, self.pool, uneven)
+        g = DecodeGraph(self.model, self.cache, self.device, layout, cap, self.pool, uneven)
+        logits = g.first_run(layout)
+        # kept only once it holds a recording: a step that raised leaves nothing behind that a later
+        # step of the same shape would try to replay
         self.graphs[key] = g
-        return g.first_run(layout)
+        return logits

@@ -44,7 +44,7 @@ class StepLayout:
     logit_rows: np.ndarray  # int32 [n_out]  flat token index of every wanted logit, in entry order
     block_tables: List[np.ndarray] = field(default_factory=list)  # per group int32 [B, max_blocks]
     slot_mappings: List[np.ndarray] = field(default_factory=list)  # per group int32 [T]
-    page_size: int = 0
+    page_sizes: List[int] = field(default_factory=list)  # per group, tokens per page
     max_q_len: int = 0
     max_kv_len: int = 0
 
@@ -60,7 +60,12 @@ class StepLayout:
         lens = self.kv_lens[:n]
         return 2 * n * int(lens.max()) > 3 * int(lens.sum())
 
-    # the reference's names for the same facts, for comparison with its test vectors
+    @property
+    def page_size(self) -> int:
+        """Tokens per page of the first group."""
+        return self.page_sizes[0] if self.page_sizes else 0
+
+    # the reference's names for the same facts (of the first group), for comparison with its test vectors
     @property
     def kv_indptr(self) -> List[int]:
         out = [0]
@@ -78,11 +83,15 @@ def build_step_layout(
     starts: Sequence[int],
     slots: Sequence[int],
     block_tables: Sequence[Sequence[Sequence[int]]],
-    page_size: int,
+    page_size,
     decode_first: bool = True,
 ) -> StepLayout:
     """``starts[i]``: tokens entry i's request already holds; ``slots[i]``: its request slot;
-    ``block_tables[g][i]``: its block table in group g, already long enough for the new tokens."""
+    ``block_tables[g][i]``: its block table in group g, already long enough for the new tokens;
+    ``page_size``: tokens per page, one number for all groups or a list with one per group."""
+    page_sizes = [int(page_size)] * len(block_tables) if isinstance(page_size, int) else [int(p) for p in page_size]
+    if len(page_sizes) != len(block_tables):
+        raise ValueError(f"{len(block_tables)} groups of block tables, {len(page_sizes)} page sizes")
     n_entries = len(entries)
     order = list(range(n_entries))
     if decode_first:
@@ -130,6 +139,7 @@ def build_step_layout(
     bts: List[np.ndarray] = []
     sms: List[np.ndarray] = []
     for g in range(len(block_tables)):
+        page_size = page_sizes[g]
         max_blocks = max((len(block_tables[g][i]) for i in range(n_entries)), default=1)
         max_blocks = max(max_blocks, 1)
         bt = np.full((B, max_blocks), -1, dtype=np.int32)
@@ -166,7 +176,7 @@ def build_step_layout(
         logit_rows=np.asarray(logit_rows, dtype=np.int32),
         block_tables=bts,
         slot_mappings=sms,
-        page_size=page_size,
+        page_sizes=page_sizes,
         max_q_len=max(q_lens) if q_lens else 0,
         max_kv_len=int(kv_lens.max()) if B else 0,
     )

@@ -32,6 +32,10 @@ def build_parser() -> argparse.ArgumentParser:
                    help="most tokens live requests hold at any time (each request rounded up to 64)")
     p.add_argument("--page-size", type=int, default=16, help="tokens per cache page (default 16)")
     p.add_argument("--max-seqs", type=int, default=8, help="request slots (default 8)")
+    p.add_argument("--kernel-table", default=None,
+                   help="JSON file of matrix-product kernel choices (bfloat16): read if it exists, so that this run uses "
+                        "the kernels of the run that wrote it and rounds as that run did; else written after the "
+                        "choices have been measured")
     p.add_argument("--device", default="cuda:0")
     return p
 
@@ -48,15 +52,26 @@ def main(argv=None) -> int:
     from .engine import Engine
     from .layout import StepEntry
 
-    if args.page_size <= 0 or 64 % args.page_size and args.page_size % 64:
-        raise SystemExit("--page-size must divide 64 or be a multiple of it")
+    if args.page_size <= 0:
+        raise SystemExit("--page-size must be positive")
+    # --max-tokens counts every request rounded up to 64 tokens; with pages that neither divide 64
+    # nor are a multiple of it a request's last page may reach beyond that, so each slot gets one more
     num_pages = max(-(-args.max_tokens // args.page_size), 1)
+    if 64 % args.page_size and args.page_size % 64:
+        num_pages += args.max_seqs
     print(f"[trace_run] loading {args.model} as {args.dtype}; pool of {num_pages} pages of {args.page_size} tokens",
           file=sys.stderr, flush=True)
+    table = Path(args.kernel_table) if args.kernel_table else None
     engine = Engine.from_folder(
         args.model, dtype=args.dtype, device=args.device, page_size=args.page_size, num_pages=num_pages,
-        max_seqs=args.max_seqs,
+        max_seqs=args.max_seqs, kernel_table=str(table) if table is not None and table.is_file() else None,
     )
+    if args.dtype == "bfloat16":
+        used = engine.kernel_table()
+        if table is not None and not table.is_file():
+            with open(table, "w") as f:
+                json.dump(used, f, indent=1)
+        print(f"[trace_run] matrix-product kernels: {json.dumps(used)}", file=sys.stderr, flush=True)
     for line in sys.stdin:
         line = line.strip()
         if not line:

@@ -131,10 +131,10 @@ class Scheduler:
             return req
         # the longest it can get: all but the last generated token sit in the cache
         longest = len(prompt) + req.budget - 1
-        for pool in self.cache.pools:
-            if self.cache.blocks_for(longest) > pool.num_pages:
+        for g, pool in enumerate(self.cache.pools):
+            if self.cache.blocks_for(longest, g) > pool.num_pages:
                 raise ValueError(
-                    f"request {rid!r}: {longest} tokens need {self.cache.blocks_for(longest)} pages, "
+                    f"request {rid!r}: {longest} tokens need {self.cache.blocks_for(longest, g)} pages, "
                     f"the pool has {pool.num_pages}; it could never finish"
                 )
         self.waiting.append(req)
@@ -145,10 +145,11 @@ class Scheduler:
         return bool(self.waiting or self.running)
 
     # ------------------------------------------------------------------ planning
-    def _pages_for(self, req: Request, n_new: int) -> int:
+    def _pages_for(self, req: Request, n_new: int) -> List[int]:
+        """Per group, the pages that ``n_new`` more tokens of ``req`` take."""
         if self.cache.has(req.rid):
             return self.cache.new_pages_needed(req.rid, n_new)
-        return self.cache.blocks_for(n_new)
+        return self.cache.pages_for_new_request(n_new)
 
     def _preempt(self, req: Request, plan: StepPlan) -> None:
         self.cache.free(req.rid)
@@ -163,8 +164,8 @@ class Scheduler:
     def schedule(self) -> StepPlan:
         """Decide the next step.  Pages are counted here and taken by ``Engine.step``."""
         # The common step of a running batch: everybody decodes, nobody can join, and even if
-        # every request opened a page the pools would hold them.  The rules of ``_schedule`` give
-        # exactly this plan then, after many more questions.
+        # every request opened a page in every group the pools would hold them.  The rules of
+        # ``_schedule`` give exactly this plan then, after many more questions.
         running = self.running
         if (
             running and len(running) <= self.max_num_batched_tokens
@@ -177,15 +178,33 @@ class Scheduler:
 
     def _schedule(self) -> StepPlan:
         plan = StepPlan()
+        while True:
+            self._plan_stages(plan)
+            if plan.entries or not self.running:
+                break
+            # Nothing fits although requests are running: several prompts advanced side by side
+            # and used the pool up before any of them could decode.  The same rule as for a
+            # decoding request that finds no page: the youngest gives way, so the oldest always
+            # gets on.
+            if len(self.running) == 1:
+                break  # alone and still stuck: the pool cannot hold it (``add`` should have refused it)
+            self._preempt(self.running[-1], plan)
+        if not plan.entries and self.has_work:
+            raise RuntimeError(
+                "scheduler is stuck: work is queued but nothing fits (pool too small for the head of the queue?)"
+            )
+        return plan
+
+    def _plan_stages(self, plan: StepPlan) -> None:
         budget = self.max_num_batched_tokens
         free = [pool.free_count for pool in self.cache.pools]
 
-        def fits(pages: int) -> bool:
-            return all(f >= pages for f in free)
+        def fits(pages: List[int]) -> bool:
+            return all(f >= p for f, p in zip(free, pages))
 
-        def take(pages: int) -> None:
-            for g in range(len(free)):
-                free[g] -= pages
+        def take(pages: List[int]) -> None:
+            for g, p in enumerate(pages):
+                free[g] -= p
 
         # (1) one token for every decoding request, oldest first; make room by preempting the youngest
         decoding = [r for r in self.running if r.remaining == 1]
@@ -203,9 +222,10 @@ class Scheduler:
                     plan.entries.remove(e)
                     budget += len(e.tokens)
                 self._preempt(victim, plan)
-                counted = sum(self._pages_for(e.request, len(e.tokens)) for e in plan.entries)
                 for g in range(len(free)):
-                    free[g] = self.cache.pools[g].free_count - counted
+                    free[g] = self.cache.pools[g].free_count
+                for e in plan.entries:
+                    take(self._pages_for(e.request, len(e.tokens)))
                 if victim is req:
                     break
             if req.state == RUNNING:
@@ -248,18 +268,15 @@ class Scheduler:
             take(self._pages_for(req, n))
             budget -= n
 
-        if not plan.entries and self.has_work:
-            raise RuntimeError(
-                "scheduler is stuck: work is queued but nothing fits (pool too small for the head of the queue?)"
-            )
-        return plan
-
     def _shrink(self, req: Request, n: int, free: List[int]) -> int:
-        """The largest portion below ``n`` that the free pages hold (0: none)."""
-        have = max(min(free), 0) if free else 0
+        """The largest portion below ``n`` that the free pages of every group hold (0: none)."""
         held = self.cache.num_tokens(req.rid) if self.cache.has(req.rid) else 0
-        room = (self.cache.blocks_for(held) + have) * self.cache.page_size - held
-        return max(min(n - 1, room), 0)
+        live = self.cache.get(req.rid)
+        room = n - 1
+        for g, page in enumerate(self.cache.page_sizes):
+            have_blocks = len(live.block_tables[g]) if live is not None else 0
+            room = min(room, (have_blocks + max(free[g], 0)) * page - held)
+        return max(room, 0)
 
     def _add_portion(self, plan: StepPlan, req: Request, n: int) -> None:
         toks = req.token_slice(req.num_computed, req.num_computed + n)

@@ -113,13 +113,16 @@ class LLM:
         tokenizer=None,
         seed: int = 0,
         look_ahead: bool = True,
+        kernel_table=None,
     ):
         """``ckpt_paths``: the model folder (config.json + safetensors), or a list whose first
         entry is that folder or a file in it.  ``precision``: "bfloat16" or "float32"; None takes
         config.json's ``torch_dtype``.  ``max_len`` bounds prompt + generated tokens of a request,
         ``max_bsz`` the requests running at once.  ``model_kwargs`` may override ``max_seq_len``
         (reference: throughput_bench.py:1057-1060).  ``look_ahead``: prepare the next decode step
-        while the GPU runs the current one (the tokens are the same either way)."""
+        while the GPU runs the current one (the tokens are the same either way).  ``kernel_table``:
+        a saved table of matrix-product kernel choices (``Engine.kernel_table``), so that bfloat16
+        results repeat from process to process."""
         from ..engine.engine import Engine
         from ..sampling.sampler import Sampler
 
@@ -143,6 +146,7 @@ class LLM:
         self.engine = Engine.from_folder(
             folder, dtype=precision, device=device, page_size=page_size, num_pages=num_pages,
             kv_memory_gb=kv_memory_gb, kv_memory_fraction=kv_memory_fraction, max_seqs=max_bsz, max_model_len=max_len,
+            kernel_table=kernel_table,
         )
         self.max_len = self.engine.max_model_len
         self.max_bsz = max_bsz

@@ -24,6 +24,11 @@ from .base import (  # noqa: F401
 )
 
 
+#: the largest head size any attention kernel here takes (the plain kernel's; the MFMA kernels take
+#: ``DECODE_HEAD_DIMS`` / ``PREFILL_HEAD_DIMS``, everything else below this runs the plain kernel)
+ATTENTION_MAX_HEAD_DIM = 256
+
+
 def attention_generic(
     qkv: torch.Tensor,
     n_q_heads: int,
@@ -85,7 +90,7 @@ def decode_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: i
 _DECODE_MIN_SPLIT = 256  # keys: shorter splits cost more in launch and merge than they gain in spread
 
 
-_DECODE_UNEVEN_SPLIT = 512  # keys: the longest split when requests differ much in length (measured with 64 requests of 128 to 4,608 tokens: 1 to 1.5% more tokens a second than with 1,024, 12% more than with 2,048)
+DECODE_UNEVEN_SPLIT = 512  # keys: the longest split when requests differ much in length (measured with 64 requests of 128 to 4,608 tokens: 1 to 1.5% more tokens a second than with 1,024, 12% more than with 2,048)
 
 
 def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, target_blocks: int = 512, uneven: bool = False):
@@ -108,7 +113,7 @@ def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, target_bloc
     want = max(-(-target_blocks // pairs), 1)
     split = -(-max(longest, 1) // want)
     if uneven:
-        split = min(split, _DECODE_UNEVEN_SPLIT)
+        split = min(split, DECODE_UNEVEN_SPLIT)
     split = max(-(-split // _DECODE_BLOCK_KEYS) * _DECODE_BLOCK_KEYS, _DECODE_MIN_SPLIT)
     # splits of 256 keys only while 512 keys would leave fewer than one block for each CU (measured
     # with cold caches: 2 requests of 8,192 tokens 23.4 against 25.8 us, 8 of 2,048 21.7 against 23.3,

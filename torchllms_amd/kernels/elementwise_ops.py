@@ -24,6 +24,10 @@ from .base import (  # noqa: F401
 )
 
 
+#: the widest row the norm kernels take: a row is kept in LDS as 32-bit floats (160 KB less 1 KB)
+RMSNORM_MAX_HIDDEN = (160 * 1024 - 1024) // 4
+
+
 def embed(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
     """``table[tokens]``; tokens int32 [n], table [vocab, hidden].  The caller has checked ids < vocab."""
     _gpu(tokens, table)

@@ -2,7 +2,8 @@
 
 Every function checks on the host that shapes, dtypes and devices are what the kernel and its grid
 assume, launches on torch's current HIP stream and raises ``KernelError`` when a launcher refuses.
-Tensors must live on the GPU: there is no CPU path.
+Tensors must live on the GPU: there is no CPU path.  Only what parts and callers use is named here;
+a module's own helpers and tables stay in the module.
 
 ``base``             dtype codes, argument checks, ``SplitSums``
 ``elementwise_ops``  embedding, RMS norm, rotary + cache write, gate, bias
@@ -16,11 +17,6 @@ from .base import (  # noqa: F401
     F32,
     KernelError,
     SplitSums,
-    _DTYPE_CODE,
-    _gpu,
-    _i32,
-    _ptr,
-    _stream,
     check,
     core,
     dtype_code,
@@ -28,7 +24,7 @@ from .base import (  # noqa: F401
     variant,
 )
 from .elementwise_ops import (  # noqa: F401
-    _rmsnorm_split,
+    RMSNORM_MAX_HIDDEN,
     add_bias_,
     embed,
     rmsnorm,
@@ -44,15 +40,10 @@ from .products import (  # noqa: F401
     STREAM_WAVE_CHOICES,
     WIDE_CHOICES,
     WIDE_MAX_ROWS,
-    _LINEAR_CHOICE,
-    _TAIL_KERNEL_US,
-    _TUNE_FLUSH_BYTES,
-    _fuses_tail,
-    _qkv_shapes,
-    _row_bucket,
-    _run_choice,
-    _run_glu,
-    _wide_shapes,
+    clear_kernel_table,
+    kernel_table,
+    load_kernel_table,
+    save_kernel_table,
     gemm_f32,
     gemm_stream,
     gemm_stream_glu,
@@ -71,18 +62,11 @@ from .products import (  # noqa: F401
     wide_supported,
 )
 from .attention_ops import (  # noqa: F401
+    ATTENTION_MAX_HEAD_DIM,
     DECODE_HEAD_DIMS,
     PREFILL_HEAD_DIMS,
     PREFILL_RESIDENT_BLOCKS,
     PREFILL_SPLIT_BLOCKS,
-    _DECODE_BLOCK_KEYS,
-    _DECODE_MIN_SPLIT,
-    _DECODE_SIGNATURES,
-    _DECODE_UNEVEN_SPLIT,
-    _F,
-    _I,
-    _P,
-    _PREFILL_SIGNATURES,
     attention_decode,
     attention_generic,
     attention_prefill,

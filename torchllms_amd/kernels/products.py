@@ -68,7 +68,7 @@ def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
 WIDE_MAX_ROWS = 128
 
 
-def _wide_shapes(x: torch.Tensor, w: torch.Tensor, what: str) -> None:
+def wide_shapes(x: torch.Tensor, w: torch.Tensor, what: str) -> None:
     _gpu(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"{what} takes bfloat16 tensors")
@@ -81,7 +81,7 @@ def gemm_wide(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     """``x @ w.T`` for at most 128 rows of bfloat16 ``x`` (K a multiple of 128) with the kernel whose
     blocks share their slice of ``x`` through LDS; ``k_splits`` > 1 cuts K over several blocks whose
     32-bit partial sums a second kernel adds, or, with ``leave_split``, come back as ``SplitSums``."""
-    _wide_shapes(x, w, "gemm_wide")
+    wide_shapes(x, w, "gemm_wide")
     m, k = x.shape
     n = w.shape[0]
     if leave_split:
@@ -110,7 +110,7 @@ def gemm_wide(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
 def gemm_wide_glu(x: torch.Tensor, w: torch.Tensor, strips_per_wave: int = 1, stages: int = 3) -> torch.Tensor:
     """``silu(x @ gate.T) * (x @ up.T)`` for at most 128 rows of bfloat16 ``x`` and ``w`` [2F, K] =
     gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``."""
-    _wide_shapes(x, w, "gemm_wide_glu")
+    wide_shapes(x, w, "gemm_wide_glu")
     if w.shape[0] % 2:
         raise KernelError("gemm_wide_glu: w must hold gate rows and as many up rows")
     m, k = x.shape
@@ -125,7 +125,7 @@ def gemm_wide_glu(x: torch.Tensor, w: torch.Tensor, strips_per_wave: int = 1, st
     return out
 
 
-def _qkv_shapes(what, x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size) -> int:
+def qkv_shapes(what, x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size) -> int:
     """Checks the arguments that the fused query|key|value products share; returns the output width."""
     _gpu(x, w, cos_sin, k_pages, v_pages, slot_mapping)
     _i32(slot_mapping, "slot_mapping")
@@ -164,7 +164,7 @@ def gemm_wide_qkv(
 ) -> torch.Tensor:
     """As ``gemm_stream_qkv`` for at most 128 rows: the product split along K, and the kernel that
     adds the splits rotates the heads and writes keys and values into their pages."""
-    width = _qkv_shapes("gemm_wide_qkv", x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size)
+    width = qkv_shapes("gemm_wide_qkv", x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size)
     m, k = x.shape
     out = torch.empty((m, width), dtype=torch.bfloat16, device=x.device)
     partial = torch.empty((k_splits, m, width), dtype=torch.float32, device=x.device)
@@ -216,7 +216,7 @@ def gemm_stream_qkv(
     rotation (interleaved pairs, from the ``rope_table`` of the rows' positions) and the cache
     write in the kernel's epilogue.  Returns [n, (Hq + 2 Hkv) * dh] whose query part is rotated;
     the key and value parts are only filled when no pages are given."""
-    width = _qkv_shapes("gemm_stream_qkv", x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size)
+    width = qkv_shapes("gemm_stream_qkv", x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size)
     m, k = x.shape
     out = torch.empty((m, width), dtype=torch.bfloat16, device=x.device)
     check(
@@ -251,8 +251,8 @@ def wide_supported(x: torch.Tensor, w: torch.Tensor) -> bool:
 #:                                                 cols: columns per block of the gated form, 8 or 16)
 #:   ("wide", strips_per_wave, k_splits, stages)   the kernel whose blocks share the activations
 #:   None                                          the library
-#: Shapes never measured follow the size rule below.
-_LINEAR_CHOICE: dict = {}
+#: Shapes never measured follow the size rule of ``linear_choice``.
+LINEAR_CHOICE: dict = {}
 ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128)
 STREAM_WAVE_CHOICES = (0, 4)
 #: (strips per wave, splits of K, buffers) that ``tune_linear`` tries from 17 rows on: whole-K
@@ -276,17 +276,17 @@ LINEAR_USES = ("plain", "glu", "qkv", "sum")
 #: trace shows 4.6 and more for every dispatch, an empty one included, which is the profiler's own);
 #: ``tune_linear`` charges it to a candidate that leaves the second half of a fused use to a kernel
 #: of its own
-_TAIL_KERNEL_US = 2.8
+TAIL_KERNEL_US = 2.8
 
 
-def _row_bucket(m: int) -> int:
+def row_bucket(m: int) -> int:
     for b in ROW_BUCKETS:
         if m <= b:
             return b
     return ROW_BUCKETS[-1]
 
 
-def _fuses_tail(choice, use: str) -> bool:
+def fuses_tail(choice, use: str) -> bool:
     """Whether the kernel of ``choice`` does the second half of ``use`` itself."""
     if use in ("plain", "sum") or choice is None:
         return use in ("plain", "sum")
@@ -296,21 +296,81 @@ def _fuses_tail(choice, use: str) -> bool:
 
 
 def linear_choice(x: torch.Tensor, w: torch.Tensor, use: str = "plain"):
-    """Which bfloat16 kernel runs ``x @ w.T``: a tuple as in the table above, or None for the library."""
+    """Which bfloat16 kernel runs ``x @ w.T``: a tuple as in the table above, or None for the library.
+    What the table holds decides.  A shape it does not hold follows a fixed rule: up to 16 rows the
+    weight-streaming kernel (its own choice of waves) for matrices of at most ``STREAM_MAX_ELEMENTS``
+    elements, the library otherwise."""
     m = x.shape[0]
     if m <= STREAM_MAX_ROWS:
         if not stream_supported(x, w):
             return None
-        key = (w.shape[0], w.shape[1], _row_bucket(m), use)
-        if key in _LINEAR_CHOICE:
-            return _LINEAR_CHOICE[key]
+        key = (w.shape[0], w.shape[1], row_bucket(m), use)
+        if key in LINEAR_CHOICE:
+            return LINEAR_CHOICE[key]
         return ("stream", 0) if w.shape[0] * w.shape[1] <= STREAM_MAX_ELEMENTS else None
     if not wide_supported(x, w):
         return None
-    return _LINEAR_CHOICE.get((w.shape[0], w.shape[1], _row_bucket(m), use))
+    return LINEAR_CHOICE.get((w.shape[0], w.shape[1], row_bucket(m), use))
 
 
-_TUNE_FLUSH_BYTES = 512 << 20  # twice the 256 MB of last-level cache
+# ----------------------------------------------------------------------------- the table, outside the process
+def kernel_table(shapes=None) -> dict:
+    """The table as a JSON-able dict: ``"n,k,rows,use" -> choice`` (a list, or None for the library).
+    ``shapes``: only the entries of these ``((n, k), use)`` pairs."""
+    wanted = None if shapes is None else {(tuple(shape), use) for shape, use in shapes}
+    out = {}
+    for (n, k, bucket, use), choice in sorted(LINEAR_CHOICE.items(), key=lambda kv: (kv[0][0], kv[0][1], kv[0][3], kv[0][2])):
+        if wanted is None or ((n, k), use) in wanted:
+            out[f"{n},{k},{bucket},{use}"] = None if choice is None else list(choice)
+    return out
+
+
+def load_kernel_table(table) -> None:
+    """Put the entries of ``table`` (a dict as ``kernel_table`` returns, or the path of a JSON file
+    holding one) into the table; they replace what was measured for the same keys, and
+    ``tune_linear`` leaves them alone.  Every entry is checked: a table from somewhere else must not
+    be able to ask a kernel for a launch it does not have."""
+    import json
+    import os
+
+    if isinstance(table, (str, os.PathLike)):
+        with open(table) as f:
+            table = json.load(f)
+    entries = {}
+    for key, choice in table.items():
+        try:
+            n, k, bucket, use = key.split(",")
+            n, k, bucket = int(n), int(k), int(bucket)
+        except ValueError:
+            raise ValueError(f'kernel table: key {key!r} is not "n,k,rows,use"') from None
+        if bucket not in ROW_BUCKETS or use not in LINEAR_USES or n <= 0 or k <= 0:
+            raise ValueError(f"kernel table: key {key!r} names no row bucket {ROW_BUCKETS} or use {LINEAR_USES}")
+        if choice is not None:
+            choice = tuple(choice)
+            ok = False
+            if choice and choice[0] == "stream" and bucket <= STREAM_MAX_ROWS:
+                ok = len(choice) in (2, 3) and choice[1] in STREAM_WAVE_CHOICES and (len(choice) == 2 or (use == "glu" and choice[2] in (8, 16)))
+            elif choice and choice[0] == "wide" and bucket > STREAM_MAX_ROWS:
+                ok = len(choice) == 4 and choice[1:] in WIDE_CHOICES and k % 128 == 0 and choice[2] <= k // 128 and wide_fits(bucket, choice[1], choice[3])
+            if not ok:
+                raise ValueError(f"kernel table: entry {key!r} -> {list(choice)!r} names no launch of a kernel here")
+        entries[(n, k, bucket, use)] = choice
+    LINEAR_CHOICE.update(entries)
+
+
+def save_kernel_table(path, shapes=None) -> None:
+    import json
+
+    with open(path, "w") as f:
+        json.dump(kernel_table(shapes), f, indent=1)
+
+
+def clear_kernel_table() -> None:
+    """Forget every measurement (the next ``tune_linear`` measures again)."""
+    LINEAR_CHOICE.clear()
+
+
+TUNE_FLUSH_BYTES = 512 << 20  # twice the 256 MB of last-level cache
 
 
 # In inference mode like the engine's steps: torch keeps the random generator's capture state in
@@ -343,13 +403,13 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         raise ValueError(f"use must be one of {LINEAR_USES}, got {use!r}")
     if use == "glu" and n % 2:
         raise ValueError(f"a gated matrix holds gate rows and as many up rows, got {n} rows")
-    if all((n, k, bucket, use) in _LINEAR_CHOICE for bucket in ROW_BUCKETS):
+    if all((n, k, bucket, use) in LINEAR_CHOICE for bucket in ROW_BUCKETS):
         return
     device = weights[0].device
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     # read, not written, before every replay: written lines would still be on their way to HBM
     # while the products are timed
-    flush = torch.zeros(_TUNE_FLUSH_BYTES // 4, dtype=torch.float32, device=device)  # (summed without a conversion pass)
+    flush = torch.zeros(TUNE_FLUSH_BYTES // 4, dtype=torch.float32, device=device)  # (summed without a conversion pass)
 
     def clock(fn) -> float:
         for i in range(2):  # loads the kernel's code and lets it ask for its LDS before the recording
@@ -377,21 +437,21 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         return best
 
     def cost(bucket, choice, fn) -> float:
-        tail = _TAIL_KERNEL_US * 1e-3 * iters if use == "qkv" and not _fuses_tail(choice, use) else 0.0
+        tail = TAIL_KERNEL_US * 1e-3 * iters if use == "qkv" and not fuses_tail(choice, use) else 0.0
         t = clock(fn) + tail
         if report is not None:
             report(bucket, choice, t / iters * 1e3)
         return t
 
     for bucket in ROW_BUCKETS:
-        if (n, k, bucket, use) in _LINEAR_CHOICE:
+        if (n, k, bucket, use) in LINEAR_CHOICE:
             continue
         x = torch.randn((bucket, k), device=device, dtype=torch.float32).to(torch.bfloat16)
 
         def run(choice):
             if use == "glu":
-                return lambda w: _run_glu(choice, x, w)
-            return lambda w: _run_choice(choice, x, w, out_dtype, leave_split=use == "sum")
+                return lambda w: run_glu(choice, x, w)
+            return lambda w: run_choice(choice, x, w, out_dtype, leave_split=use == "sum")
 
         best, best_time = None, cost(bucket, None, run(None))
         if bucket <= STREAM_MAX_ROWS and use == "glu":
@@ -408,10 +468,10 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
             t = cost(bucket, choice, run(choice))
             if t < best_time:
                 best, best_time = choice, t
-        _LINEAR_CHOICE[(n, k, bucket, use)] = best
+        LINEAR_CHOICE[(n, k, bucket, use)] = best
 
 
-def _run_choice(choice, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, leave_split: bool = False):
+def run_choice(choice, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, leave_split: bool = False):
     if choice is None:
         y = torch.nn.functional.linear(x, w)
         return y if y.dtype == out_dtype else y.to(out_dtype)
@@ -431,7 +491,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         return gemm_f32(x, w)
     _gpu(x, w)
     out_dtype = out_dtype or x.dtype
-    return _run_choice(linear_choice(x, w), x, w, out_dtype)
+    return run_choice(linear_choice(x, w), x, w, out_dtype)
 
 
 def linear_to_sum(x: torch.Tensor, w: torch.Tensor):
@@ -441,7 +501,7 @@ def linear_to_sum(x: torch.Tensor, w: torch.Tensor):
     if x.dtype == torch.float32:
         return gemm_f32(x, w)
     _gpu(x, w)
-    return _run_choice(linear_choice(x, w, "sum"), x, w, x.dtype, leave_split=True)
+    return run_choice(linear_choice(x, w, "sum"), x, w, x.dtype, leave_split=True)
 
 
 def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
@@ -450,15 +510,15 @@ def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     if x.dtype != torch.bfloat16:
         return silu_mul(linear(x, w))
     _gpu(x, w)
-    return _run_glu(linear_choice(x, w, "glu"), x, w)
+    return run_glu(linear_choice(x, w, "glu"), x, w)
 
 
-def _run_glu(choice, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+def run_glu(choice, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     if choice is not None and choice[0] == "stream":
         return gemm_stream_glu(x, w, choice[1], choice[2] if len(choice) > 2 else 16)
     if choice is not None and choice[0] == "wide" and choice[2] == 1:
         return gemm_wide_glu(x, w, choice[1], choice[3])
-    return silu_mul(_run_choice(choice, x, w, x.dtype))
+    return silu_mul(run_choice(choice, x, w, x.dtype))
 
 
 def qkv_rope_store(
@@ -497,7 +557,7 @@ def qkv_rope_store(
                 x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size,
                 choice[1], choice[2], choice[3],
             )
-        qkv = _run_choice(choice, x, w, x.dtype)
+        qkv = run_choice(choice, x, w, x.dtype)
     else:
         qkv = linear(x, w)
     if bias is not None:

@@ -20,7 +20,9 @@ class Attention(Mixer):
 
     Query head h reads key/value head ``h // (num_heads / num_kv_heads)``.  ``window`` w > 0
     limits a query at position p to keys p-w+1..p.  ``shares_kv``: this layer has no k/v
-    projections and reads the cache of the run named by the execution order.
+    projections and reads the cache of the run named by the execution order.  ``kv_page_size``:
+    tokens per page of this layer's keys and values, when not the engine's own (layers that ask for
+    the same form a group of pages of their own).
     """
 
     #: every launch is fixed by the step's shape: a decode step may be recorded in a HIP graph
@@ -37,6 +39,7 @@ class Attention(Mixer):
         window: int,
         position: PartSpec,
         shares_kv: bool = False,
+        kv_page_size: Optional[int] = None,
     ):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
@@ -48,6 +51,7 @@ class Attention(Mixer):
         self.softmax_scale = float(softmax_scale)
         self.window = int(window)
         self.shares_kv = shares_kv
+        self.kv_page_size = kv_page_size
         self.position = POSITIONS.build(position)
         self.wqkv: Optional[torch.Tensor] = None
         self.bqkv: Optional[torch.Tensor] = None
@@ -67,10 +71,20 @@ class Attention(Mixer):
                 specs["wv.bias"] = ParamSpec((kv,), init="zeros")
         return specs
 
+    def check_sizes(self, dtype: torch.dtype) -> None:
+        if not 0 < self.head_dim <= ops.ATTENTION_MAX_HEAD_DIM:
+            raise ValueError(
+                f"attention: head size {self.head_dim}; the attention kernels take head sizes up to "
+                f"{ops.ATTENTION_MAX_HEAD_DIM} (any number of heads and of query heads per kv head)"
+            )
+        rot = self.position.rotary_args()
+        if rot is not None and (rot.rotary_dim % 2 or rot.rotary_dim > self.head_dim):
+            raise ValueError(f"attention: {rot.rotary_dim} rotated channels of a head of {self.head_dim} (even, at most the head size)")
+
     def cache_need(self):
         if self.shares_kv:
             return None
-        return KVNeed(num_kv_heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window)
+        return KVNeed(num_kv_heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window, page_size=self.kv_page_size)
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         names = ["wq"] if self.shares_kv else ["wq", "wk", "wv"]

@@ -47,11 +47,15 @@ class KVNeed:
 
     ``window`` = 0: every past token stays visible.  ``window`` = w > 0: a token at position p
     sees positions p-w+1 .. p only, so pages that lie wholly before that may be given back.
+    ``page_size`` (tokens per page) and ``dtype`` ("float32", "bfloat16") are the engine's own
+    unless the mixer asks for others; layers that ask for the same form one group of pages.
     """
 
     num_kv_heads: int
     head_dim: int
     window: int = 0
+    page_size: Optional[int] = None
+    dtype: Optional[str] = None
 
 
 @dataclass(frozen=True)
@@ -80,9 +84,22 @@ class Part:
 
     def linear_weights(self):
         """The matrices this part multiplies activations with (for kernel selection by measurement):
-        tensors, or pairs ``(tensor, use)`` where ``use`` names the fused form of the product that
-        the part calls ("glu": ``ops.linear_glu``, "qkv": ``ops.qkv_rope_store``)."""
+        tensors, pairs ``(tensor, use)`` where ``use`` names the fused form of the product that
+        the part calls ("glu": ``ops.linear_glu``, "qkv": ``ops.qkv_rope_store``, "sum":
+        ``ops.linear_to_sum``), or triples ``(tensor, use, out_dtype)`` when the product's result
+        has another dtype than its inputs (32-bit logits)."""
         return []
+
+    def ignorable_params(self):
+        """Local names of tensors that a checkpoint may hold for this part although the part, as
+        configured, has no use for them (an output matrix beside tied embeddings): the loader drops
+        them with a warning instead of calling them unexpected."""
+        return []
+
+    def check_sizes(self, dtype: torch.dtype) -> None:
+        """Raise (``ValueError`` or a subclass) if no kernel takes this part's sizes in ``dtype``;
+        called once when an engine is built, so that a size is refused there and not at the first
+        step."""
 
 
 class Norm(Part):
@@ -145,26 +162,35 @@ class Mixer(Part):
 
 
 class Block(Part):
-    """Arrangement of one layer.  ``forward`` takes the residual stream ``h`` and a pending
-    ``delta`` that has not been added to it yet (None for the first layer) and returns the
-    same pair, so the sum can be fused into whatever reads it next."""
+    """Arrangement of one layer's parts.  ``SLOTS`` names the sub-parts the arrangement has and the
+    kind of each ("mixer", "feed_forward" or "norm"), in the order their tensors are listed; the
+    model builds them from the layer's ``LayerSpec.parts`` and hands them over as a dict, and each
+    is reachable as an attribute of its slot's name.
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ffn_norm: Norm):
-        self.mixer = mixer
-        self.feed_forward = feed_forward
-        self.mixer_norm = mixer_norm
-        self.ffn_norm = ffn_norm
+    ``forward`` takes the residual stream ``h`` and a pending ``delta`` that has not been added to
+    it yet (None for the first layer) and returns the same pair, so the sum can be fused into
+    whatever reads it next.  ``cache`` maps the slot of every mixer to what the cache manager holds
+    for it in this run (a ``KVLayerView``, a ``StateView`` or None)."""
 
-    #: names under which the four sub-parts' tensors appear inside a layer
-    SLOTS = ("mixer_norm", "mixer", "ffn_norm", "ffn")
+    SLOTS: Dict[str, str] = {}
+
+    def __init__(self, parts: Dict[str, Part]):
+        missing = [s for s in self.SLOTS if s not in parts]
+        extra = [s for s in parts if s not in self.SLOTS]
+        if missing or extra:
+            raise ValueError(
+                f"{type(self).__name__} arranges the parts {list(self.SLOTS)}; missing {missing}, not its own {extra}"
+            )
+        self.parts: Dict[str, Part] = {slot: parts[slot] for slot in self.SLOTS}
+        for slot, part in self.parts.items():
+            setattr(self, slot, part)
 
     def sub_parts(self) -> Dict[str, Part]:
-        return {
-            "mixer_norm": self.mixer_norm,
-            "mixer": self.mixer,
-            "ffn_norm": self.ffn_norm,
-            "ffn": self.feed_forward,
-        }
+        return self.parts
+
+    def mixers(self) -> Dict[str, "Mixer"]:
+        """slot -> mixer, for every sub-part that may keep something in the cache."""
+        return {slot: part for slot, part in self.parts.items() if isinstance(part, Mixer)}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         out = {}
@@ -217,6 +243,8 @@ class Head(Part):
 MIXERS = Registry("mixer")
 FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
+#: the kinds a block's ``SLOTS`` may name, and where parts of each kind are registered
+SLOT_KINDS = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
 POSITIONS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
 EMBEDDINGS = Registry("embedding")

@@ -12,10 +12,11 @@ class PreNormBlock(Block):
     norm that reads it; the last one is handed on as ``delta``."""
 
     graph_safe = True
+    SLOTS = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "feed_forward"}
 
     def forward(self, h, delta, ctx, cache):
         h, y = self.mixer_norm.forward_add(h, self.mixer_norm.delta(delta))
-        a = self.mixer.forward(y, ctx, cache)
+        a = self.mixer.forward(y, ctx, cache["mixer"])
         h, y = self.ffn_norm.forward_add(h, self.ffn_norm.delta(a))
-        f = self.feed_forward.forward(y, ctx)
+        f = self.ffn.forward(y, ctx)
         return h, f

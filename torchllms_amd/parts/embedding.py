@@ -57,7 +57,11 @@ class LMHead(Head):
         self.weight = embedding.weight
 
     def linear_weights(self):
-        return [self.weight]
+        return [(self.weight, "plain", torch.float32)]
+
+    def ignorable_params(self):
+        # checkpoints of tied models sometimes carry the output matrix all the same
+        return ["weight"] if self.tied else []
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.linear(x, self.weight, out_dtype=torch.float32)
