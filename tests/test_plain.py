@@ -117,15 +117,68 @@ def test_rope_llama3_bands():
         plain.rope_inverse_frequencies(32, 1e4, {"rope_type": "yarn"})
 
 
-def test_rope_llama3_band_edges_are_continuous():
-    # at wavelength = original/high the blend weight is 1 (unchanged); at original/low it is 0 (/factor)
+def _both_frequency_functions():
+    from torchllms_amd.parts.positions import rotary_inverse_frequencies
+
+    return [("plain", plain.rope_inverse_frequencies), ("engine", rotary_inverse_frequencies)]
+
+
+@pytest.mark.parametrize("factor, low, high, old", [(8.0, 1.0, 4.0, 8192), (32.0, 1.0, 4.0, 8192), (4.0, 2.0, 3.0, 640)])
+def test_rope_llama3_blend_is_continuous_linear_and_ends_where_the_bands_say(factor, low, high, old):
+    """What fixes the middle band beside the reference's text: on a dense grid of frequencies
+    (2,048 of them, from sixty to hundreds inside the band) the ratio scaled / unscaled is 1 for wavelengths below
+    old/high, 1/factor above old/low, and in between it moves from the one to the other without a
+    jump, rising with x = old / wavelength, with one slope everywhere (linear in x).  Swapped blend
+    weights, or low and high exchanged, put the values of the two outer bands at the wrong edges:
+    a jump of (1 - 1/factor) at each (reference: networks.py:259-277).  Both the plain function and
+    the engine's own are asked."""
+    sc = {"rope_type": "llama3", "factor": factor, "low_freq_factor": low, "high_freq_factor": high,
+          "original_max_position_embeddings": old}
+    dim, theta = 4096, 500000.0
+    for name, fn in _both_frequency_functions():
+        base = fn(dim, theta, None).double()
+        got = fn(dim, theta, sc).double()
+        x = old * base / (2 * math.pi)  # old / wavelength, falling along the grid
+        ratio = got / base
+        short, long = x > high, x < low
+        band = ~short & ~long
+        assert band.sum() > 50 and short.sum() > 100 and long.sum() > 100, name
+        assert torch.allclose(ratio[short], torch.ones_like(ratio[short]), rtol=1e-6), name
+        assert torch.allclose(ratio[long], torch.full_like(ratio[long], 1 / factor), rtol=1e-6), name
+        # no jump anywhere: neighbours on the grid differ by at most what the slope allows
+        slope = (1 - 1 / factor) / (high - low)
+        steps = (x[:-1] - x[1:]).abs()
+        jumps = (ratio[:-1] - ratio[1:]).abs()
+        assert (jumps <= slope * steps * 1.01 + 1e-6).all(), f"{name}: a jump of {jumps.max().item()} at x = {x[jumps.argmax()].item()}"
+        # rising with x inside the band, with the same slope between any two neighbours
+        xb, rb = x[band], ratio[band]
+        local = (rb[:-1] - rb[1:]) / (xb[:-1] - xb[1:])
+        assert torch.allclose(local, torch.full_like(local, slope), rtol=2e-3), f"{name}: slopes {local.min().item()}..{local.max().item()}, expected {slope}"
+        # and anchored: the value at the band's middle is the mean of the two outer values
+        mid = (xb - (low + high) / 2).abs().argmin()
+        assert rb[mid].item() == pytest.approx((1 + 1 / factor) / 2 + slope * (xb[mid].item() - (low + high) / 2), rel=1e-5), name
+
+
+def test_rope_llama3_middle_band_numbers_worked_out_by_hand():
+    """Llama 3.1's own constants (theta 500000, head size 128, factor 8, low 1, high 4, old 8192), pair
+    i has theta_i = 500000^(-2i/128) and wavelength 2 pi / theta_i.  From the reference's lines
+    (networks.py:259-277), with a pocket calculator:
+      i = 28: wavelength 1956.5 < 2048               -> untouched
+      i = 29: wavelength 2401.7, smooth = (8192/2401.7 - 1)/3 = 0.80362 -> ratio (1-s)/8 + s = 0.828168
+      i = 31: wavelength 3619.2, smooth = 0.42115                        -> ratio 0.493507
+      i = 34: wavelength 6695.1, smooth = 0.074527                       -> ratio 0.190211
+      i = 35: wavelength 8218.7 > 8192               -> divided by 8
+    """
     sc = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
-          "original_max_position_embeddings": 64}
-    for wl, want_ratio in [(16.0, 1.0), (64.0, 1 / 8)]:
-        f = 2 * math.pi / wl
-        smooth = (64 / wl - 1.0) / (4.0 - 1.0)
-        blended = (1 - smooth) * f / 8 + smooth * f
-        assert blended / f == pytest.approx(want_ratio, rel=1e-6)
+          "original_max_position_embeddings": 8192}
+    want = {28: 0.003211446, 29: 0.0026160993 * 0.828168412, 31: 0.0017360467 * 0.493507123, 34: 0.00093847387 * 0.190210744,
+            35: 0.00076449699 / 8}
+    assert want[29] == pytest.approx(0.00216657076, rel=1e-7) and want[34] == pytest.approx(0.000178507813, rel=1e-7)
+    for name, fn in _both_frequency_functions():
+        got = fn(128, 500000.0, sc)
+        assert got.dtype == torch.float32
+        for i, value in want.items():
+            assert got[i].item() == pytest.approx(value, rel=2e-6), f"{name}: pair {i}"
 
 
 def test_row_permutation_matches_the_other_pairing():
