@@ -114,6 +114,7 @@ class LLM:
         seed: int = 0,
         look_ahead: bool = True,
         kernel_table=None,
+        random_weights: bool = False,
     ):
         """``ckpt_paths``: the model folder (config.json + safetensors), or a list whose first
         entry is that folder or a file in it.  ``precision``: "bfloat16" or "float32"; None takes
@@ -122,7 +123,9 @@ class LLM:
         (reference: throughput_bench.py:1057-1060).  ``look_ahead``: prepare the next decode step
         while the GPU runs the current one (the tokens are the same either way).  ``kernel_table``:
         a saved table of matrix-product kernel choices (``Engine.kernel_table``), so that bfloat16
-        results repeat from process to process."""
+        results repeat from process to process.  ``random_weights``: the folder needs a config.json
+        only (and a tokenizer.json for text); the weights are drawn from ``seed`` as
+        ``weights.write_model_folder`` would write them."""
         from ..engine.engine import Engine
         from ..sampling.sampler import Sampler
 
@@ -143,11 +146,17 @@ class LLM:
             max_len = min(max_len, int(model_kwargs.pop("max_seq_len")))
         if model_kwargs:
             raise ValueError(f"unknown model_kwargs {sorted(model_kwargs)}")
-        self.engine = Engine.from_folder(
-            folder, dtype=precision, device=device, page_size=page_size, num_pages=num_pages,
-            kv_memory_gb=kv_memory_gb, kv_memory_fraction=kv_memory_fraction, max_seqs=max_bsz, max_model_len=max_len,
-            kernel_table=kernel_table,
+        engine_kw = dict(
+            dtype=precision, device=device, page_size=page_size, num_pages=num_pages, kv_memory_gb=kv_memory_gb,
+            kv_memory_fraction=kv_memory_fraction, max_seqs=max_bsz, max_model_len=max_len, kernel_table=kernel_table,
         )
+        if random_weights:
+            from ..config.registry import load_config
+
+            _, config = load_config(folder)
+            self.engine = Engine.from_random(config, seed=seed, **engine_kw)
+        else:
+            self.engine = Engine.from_folder(folder, **engine_kw)
         self.max_len = self.engine.max_model_len
         self.max_bsz = max_bsz
         self.batched = batched
