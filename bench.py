@@ -2,23 +2,32 @@
 bfloat16 weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
-                    [--shape 8b|1b|70b] [--workload decode|serve|small-kernels]
+                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels]
 
-A step is one decode step of the whole batch: ``Engine.step`` on one token per request followed by
-the sampling kernel and the copy of the chosen tokens to the host, as generation does it.  The
-requests' earlier context is not computed: their pages are filled with random keys and values,
-which costs a decode step the same reads.  One JSON line is printed: ``value`` is decoded tokens a
-second at the default batch; ``prefill`` times one 2,048-token prompt; ``roofline`` sets the decode
-step's unavoidable reads (every weight once, the live requests' cache) against HBM's 8 TB/s;
-``points`` holds decode at batch 1 and 64.
+Everything runs through the generation loop: the scheduler admits the requests, cuts their prompts
+into portions under its token budget, and plans every decode step; the step function runs it; the
+sampling kernel picks the tokens (greedy), and they travel to the host, as in serving.  Nothing of
+the context is faked: prompts of random token ids are prefilled for real.
+
+One JSON line is printed.  ``value``: decoded tokens a second of ``--batch`` requests whose context
+ends at ``--context``: the prompts are ``context`` less the generated tokens long, and K decode
+steps are timed after W warm-up steps (a step is one decode step of the whole batch).  ``points``:
+the same at batch 1 and 64.  ``prefill``: one prompt of 2,048 tokens in one step.  ``roofline``: the
+bytes a decode step has to read (every weight once, the live requests' cache) over its time, against
+HBM's published 8 TB/s and against what a plain read kernel reaches on this GPU.  ``workload``: the
+reference's own decode benchmark (reference: torchllms/inference/throughput_bench.py:498-563):
+prompts of 2,048 tokens, 256 generated, batch 1, 8 and 64, tokens a second = B * (new - 1) /
+seconds from the end of the prefill to the last token, with the bytes per step at the mean context
+of 2,176 and their share of 8 TB/s.
 
 ``--shape`` takes the layer sizes of Llama-3.2-1B or Llama-3.1-70B instead (the default is the
-headline's 8B).  ``--workload serve`` runs the scheduler instead of fixed batches: 64 requests at
-once, prompts of 128 to 4,096 random tokens, 512 tokens generated for each at temperature 0.7; its
-line reports generated tokens a second over the whole run, prefill included.  ``--workload
-small-kernels`` times what a norm kernel adds to a replayed graph of large products, without a
-profiler (under rocprofv3 no dispatch is shorter than about 4.6 us, an empty kernel included, so a
-kernel trace overstates the small kernels of a step).
+headline's 8B).  ``--workload serve`` runs 64 requests at once with prompts of 128 to 4,096 random
+tokens and 512 tokens generated for each at temperature 0.7; its line reports generated tokens a
+second over the whole run, prefill included.  ``--workload peaks`` measures what this GPU reaches:
+a read of 4 GiB with 16-byte loads, a device copy, a loop of MFMA instructions on registers, and the
+library's large matrix product.  ``--workload small-kernels`` times what a norm kernel adds to a
+replayed graph of large products, without a profiler (under rocprofv3 no dispatch is shorter than
+about 4.6 us, an empty kernel included, so a kernel trace overstates the small kernels of a step).
 """
 
 from __future__ import annotations
@@ -28,7 +37,11 @@ import json
 import sys
 import time
 
+from ctypes import c_int, c_size_t, c_void_p
+
 HBM_GBS = 8000.0  # MI355X HBM3E, published
+PEAK_SIGNATURES = {"tl_peak_stream_read": [c_void_p, c_size_t, c_int, c_void_p, c_void_p],
+                   "tl_peak_mfma_bf16": [c_int, c_int, c_void_p, c_void_p]}
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # dense MFMA, published
 
 # the model of the headline benchmark: Llama-3.1-8B layer sizes, random weights
@@ -65,7 +78,10 @@ def parse_args(argv=None):
     p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the headline's)")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve", "small-kernels"])
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels"])
+    p.add_argument("--token-budget", type=int, default=8192, help="tokens a step may hold (the scheduler cuts prompts to it)")
+    p.add_argument("--no-reference-workload", action="store_true",
+                   help="leave out the reference's benchmark (2,048-token prompts, 256 new tokens at batch 1, 8, 64)")
     p.add_argument("--requests", type=int, default=64, help="serve: requests running at once")
     p.add_argument("--new-tokens", type=int, default=512, help="serve: tokens generated for every request")
     p.add_argument("--no-look-ahead", action="store_true", help="plan every decode step when it runs, not during the step before")
@@ -94,65 +110,102 @@ def weight_bytes(engine) -> int:
     return total
 
 
-def fill_context(engine, rids, n_tokens, seed=0):
-    """Give every request ``n_tokens`` cached tokens without computing them: pages are claimed and
-    filled with random keys and values."""
+def generation_run(engine, sampler, batch, prompt_len, new_tokens, vocab, budget, look_ahead=True, timed_steps=None, warmup=0,
+                   seed=0):
+    """``batch`` random prompts of ``prompt_len`` tokens through the generation loop, ``new_tokens``
+    greedy tokens each.  The scheduler decodes first: a request whose prompt is in the cache decodes
+    while the others' prompts are still being prefilled, so the decode phase of the whole batch
+    begins when the last prompt is in, and lasts until the first request ends.  Returns the seconds
+    from the end of the prefill to the end of the run (``decode_s``; with a token budget that holds
+    all prompts in one step every request decodes in lock step all the way, as in the reference's
+    benchmark) and, with ``timed_steps`` = K, the seconds of exactly K decode steps of the whole
+    batch after ``warmup`` + 3 further ones (the steps in which the decode shape is met for the first
+    times and recorded as a HIP graph), bracketed by synchronisations."""
+    import random
+
     import torch
 
-    for rid in rids:
-        engine.admit(rid)
-        engine.cache.extend(rid, n_tokens)
-        engine.cache.advance(rid, n_tokens)
-    g = torch.Generator(device=engine.device).manual_seed(seed)
-    for pages in list(engine.cache.k_pages) + list(engine.cache.v_pages):
-        flat = pages.view(-1)
-        chunk = 1 << 28
-        for lo in range(0, flat.numel(), chunk):
-            flat[lo : lo + chunk].normal_(0.0, 1.0, generator=g)
-
-
-def decode_run(engine, sampler, batch, context, steps, warmup, vocab, look_ahead=True):
-    """Time ``steps`` decode steps of ``batch`` requests whose context ends at ``context`` tokens.
-    A step is what the generation loop does for one: run the batch, sample, read the tokens; with
-    ``look_ahead`` the next step's plan is made while the GPU runs this one, as the loop does."""
-    import torch
-
-    from torchllms_amd.engine import StepEntry
+    from torchllms_amd.inference.llm import GenerationLoop
     from torchllms_amd.sampling import SamplingParams
 
-    rids = [f"d{i}" for i in range(batch)]
-    # a decode shape is recorded as a HIP graph once it has come back a few times: these steps are
-    # part of setting the engine up, before the warm-up steps that the caller asked for
-    prime = 3
-    start = context - (steps + warmup + prime) - 1
-    fill_context(engine, rids, start)
-    params = [SamplingParams(temperature=0.0, seed=i) for i in range(batch)]
-    tokens = [(7 * i + 3) % vocab for i in range(batch)]
+    rng = random.Random(seed)
+    prompts = [[rng.randrange(vocab) for _ in range(prompt_len)] for _ in range(batch)]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=new_tokens, stop_token_ids=(), seed=i) for i in range(batch)]
+    loop = GenerationLoop(engine, sampler, max_num_seqs=batch, max_num_batched_tokens=budget,
+                          max_model_len=prompt_len + new_tokens, look_ahead=look_ahead)
+    skip = 3 + warmup
+    state = {"decode_steps": 0, "kv_tokens": 0, "t0": None, "t1": None, "t_start": None, "prefill_done": None}
 
-    prepared = None
+    def on_step(plan):
+        # (called when the step's tokens are booked) a decode step of the whole batch fed every request a
+        # token that it had generated; while prompts are still being prefilled, or once a request has
+        # ended, a step is not one
+        if len(plan.entries) != batch or not all(len(e.tokens) == 1 and len(e.request.output) >= 2 for e in plan.entries):
+            return
+        state["decode_steps"] += 1
+        if timed_steps is not None:
+            if skip < state["decode_steps"] <= skip + timed_steps:
+                state["kv_tokens"] += sum(e.request.num_computed for e in plan.entries)  # keys each row read
+            if state["decode_steps"] == skip:
+                torch.cuda.synchronize()
+                state["t0"] = time.perf_counter()
+            elif state["decode_steps"] == skip + timed_steps:
+                torch.cuda.synchronize()
+                state["t1"] = time.perf_counter()
 
-    def one_step(k):
-        nonlocal tokens, prepared
-        entries = [StepEntry(r, [t], [0]) for r, t in zip(rids, tokens)]
-        logits = engine.step_prepared(prepared, entries) if prepared is not None else None
-        if logits is None:
-            logits = engine.step(entries)
-        pending = sampler.launch(logits, params, [k] * batch)
-        prepared = engine.prepare_decode() if look_ahead else None
-        tokens = pending.tolist()
+    # the end of the prefill: the scheduler's own books say when every prompt is in the cache
+    sched = loop.scheduler
+    update = sched.update
 
-    for k in range(prime + warmup):
-        one_step(k)
+    def update_and_watch(plan, sampled):
+        done = update(plan, sampled)
+        if state["prefill_done"] is None and not sched.waiting and all(r.output for r in sched.running):
+            torch.cuda.synchronize()
+            state["prefill_done"] = time.perf_counter()
+        return done
+
+    sched.update = update_and_watch
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(steps):
-        one_step(prime + warmup + k)
+    state["t_start"] = time.perf_counter()
+    requests = loop.run(prompts, params, on_step)
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    mean_ctx = start + prime + warmup + (steps + 1) / 2
-    for r in rids:
-        engine.free(r)
-    return dt / steps, mean_ctx
+    t_end = time.perf_counter()
+    assert all(len(r.output) == new_tokens for r in requests)
+    engine.cache.check_invariants()
+    out = {
+        "prefill_s": state["prefill_done"] - state["t_start"],
+        "decode_s": t_end - state["prefill_done"],
+        "decode_steps": state["decode_steps"],
+        "prepared_steps": loop.stats["prepared_steps"],
+    }
+    if timed_steps is not None:
+        if state["t1"] is None:
+            raise RuntimeError(f"only {state['decode_steps']} decode steps ran, {skip + timed_steps} were needed")
+        out["timed_s"] = state["t1"] - state["t0"]
+        out["mean_kv_tokens"] = state["kv_tokens"] / timed_steps  # keys all rows of a timed step read, on average
+    return out
+
+
+def measured_read_gbs(device, gib: int = 4) -> float:
+    """What a plain read kernel (16-byte loads, four in flight per thread, 2,048 blocks) reaches on
+    this GPU, in GB/s: the best of five passes over ``gib`` GiB."""
+    import torch
+
+    from torchllms_amd.kernels import lib
+
+    peaks = lib.variant("peaks", 1, PEAK_SIGNATURES)
+    buf = torch.empty(gib << 30, dtype=torch.uint8, device=device)
+    buf.view(torch.int32).fill_(1)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = float("inf")
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(6):
+        start.record()
+        lib.check(peaks.tl_peak_stream_read(buf.data_ptr(), buf.numel(), 2048, None, stream), peaks, "tl_variant_last_error")
+        stop.record()
+        stop.synchronize()
+        best = min(best, start.elapsed_time(stop))
+    return buf.numel() / (best * 1e-3) / 1e9
 
 
 def prefill_run(engine, n_tokens, vocab, repeats=3):
@@ -236,6 +289,52 @@ def serve_run(args, shape) -> int:
     return 0
 
 
+def peaks_run(args) -> int:
+    """What this GPU reaches at its clocks of today, beside the published figures: a read of 4 GiB by a
+    kernel of 16-byte loads, a device-to-device copy (its bytes counted once read, once written), MFMA
+    bfloat16 16x16x32 instructions issued from registers alone, and the library's product of two
+    8,192 x 8,192 bfloat16 matrices."""
+    import torch
+
+    from torchllms_amd.kernels import lib
+
+    dev = "cuda:0"
+    peaks = lib.variant("peaks", 1, PEAK_SIGNATURES)
+    stream = torch.cuda.current_stream().cuda_stream
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def best_ms(fn, repeats=6):
+        best = float("inf")
+        for _ in range(repeats):
+            start.record()
+            fn()
+            stop.record()
+            stop.synchronize()
+            best = min(best, start.elapsed_time(stop))
+        return best
+
+    read_gbs = measured_read_gbs(dev)
+    src = torch.empty(2 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    src.view(torch.int32).fill_(3)
+    copy_ms = best_ms(lambda: dst.copy_(src))
+    iters, blocks = 20000, 256 * 8
+    mfma_ms = best_ms(lambda: lib.check(peaks.tl_peak_mfma_bf16(iters, blocks, None, stream), peaks, "tl_variant_last_error"))
+    mfma_tflops = blocks * 4 * iters * 8 * (2 * 16 * 16 * 32) / (mfma_ms * 1e-3) / 1e12
+    a = torch.randn(8192, 8192, device=dev).to(torch.bfloat16)
+    b = torch.randn(8192, 8192, device=dev).to(torch.bfloat16)
+    mm_ms = best_ms(lambda: torch.matmul(a, b))
+    print(json.dumps({
+        "metric": "measured peaks of this GPU", "unit": "GB/s and TFLOP/s",
+        "hbm_read_gbs": round(read_gbs, 1), "hbm_read_frac_of_published": round(read_gbs / HBM_GBS, 4),
+        "hbm_copy_gbs_read_plus_write": round(2 * src.numel() / (copy_ms * 1e-3) / 1e9, 1),
+        "mfma_bf16_tflops": round(mfma_tflops, 1), "mfma_bf16_frac_of_published": round(mfma_tflops / PEAK_TFLOPS["bfloat16"], 4),
+        "library_matmul_bf16_tflops": round(2 * 8192 ** 3 / (mm_ms * 1e-3) / 1e12, 1),
+        "published": {"hbm_gbs": HBM_GBS, "mfma_bf16_tflops": PEAK_TFLOPS["bfloat16"], "fp32_tflops": PEAK_TFLOPS["float32"]},
+    }))
+    return 0
+
+
 def small_kernels_run(args, shape) -> int:
     """What a small kernel costs between two large ones of a replayed graph: the time of a graph of
     32 gate/up products of a decode step (each on a matrix of its own turn, caches flushed before
@@ -296,6 +395,8 @@ def main(argv=None) -> int:
         return serve_run(args, shape)
     if args.workload == "small-kernels":
         return small_kernels_run(args, shape)
+    if args.workload == "peaks":
+        return peaks_run(args)
     import torch
 
     from torchllms_amd.config import LlamaConfig
@@ -307,6 +408,18 @@ def main(argv=None) -> int:
     cfg = LlamaConfig.from_dict(dict(shape, num_hidden_layers=n_layers))
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
     max_batch = max(batches)
+    def tokens_to_generate(b, steps):
+        """Enough for ``steps`` timed decode steps of the whole batch: the first token comes from the
+        prefill, the first request decodes alone while the other prompts are prefilled (at most so many
+        steps), 3 + W steps record and warm up, and the last token is never fed back."""
+        prefill_steps = -(-b * args.context // max(args.token_budget - b, 1)) + 1
+        return 1 + prefill_steps + 3 + args.warmup + steps + 1
+
+    new_tokens = tokens_to_generate(args.batch, args.steps)
+    prompt_len = args.context - new_tokens
+    if prompt_len < 1:
+        print(f"--context {args.context} is too short for {new_tokens} generated tokens")
+        return 2
     pages_per_req = -(-args.context // args.page_size) + 1
     engine = Engine.from_random(
         cfg, seed=0, dtype=args.dtype, draw_on_device=True, page_size=args.page_size,
@@ -316,17 +429,45 @@ def main(argv=None) -> int:
     elt = 2 if args.dtype == "bfloat16" else 4
     wbytes = weight_bytes(engine)
     kv_per_token = 2 * n_layers * cfg.num_key_value_heads * cfg.head_dim * elt
+    look_ahead = not args.no_look_ahead
+
+    def step_bytes(b, mean_ctx):
+        return wbytes + b * cfg.hidden_size * elt + b * mean_ctx * kv_per_token
 
     results = {}
     for b in batches:
         steps = args.steps if b == args.batch else max(args.steps // 2, 4)
-        sec, mean_ctx = decode_run(engine, sampler, b, args.context, steps, args.warmup, cfg.vocab_size, not args.no_look_ahead)
-        step_bytes = wbytes + b * cfg.hidden_size * elt + b * mean_ctx * kv_per_token
-        results[b] = dict(sec=sec, tps=b / sec, bytes=step_bytes)
+        new_b = tokens_to_generate(b, steps)
+        run = generation_run(engine, sampler, b, args.context - new_b, new_b, cfg.vocab_size, args.token_budget, look_ahead,
+                             timed_steps=steps, warmup=args.warmup)
+        sec = run["timed_s"] / steps
+        nbytes = wbytes + b * cfg.hidden_size * elt + run["mean_kv_tokens"] * kv_per_token
+        results[b] = dict(sec=sec, tps=b / sec, bytes=nbytes, steps=steps, mean_ctx=run["mean_kv_tokens"] / b)
 
     pre_sec = prefill_run(engine, args.prefill_tokens, cfg.vocab_size)
     flops = prefill_flops(cfg, n_layers, args.prefill_tokens)
 
+    # the reference's own decode benchmark: 2,048-token prompts, 256 new tokens
+    workload = {}
+    if not args.no_reference_workload:
+        ref_prompt, ref_new = 2048, 256
+        if ref_prompt + ref_new <= args.context:
+            for b in sorted(set([1, 8, 64]) & set(range(1, max_batch + 1))):
+                # the whole batch's prompts in one step, as the reference's benchmark prefills them in one forward pass:
+                # every request then decodes in lock step from the first token to the last
+                one_step = b * ref_prompt
+                generation_run(engine, sampler, b, ref_prompt, 8, cfg.vocab_size, one_step, look_ahead, seed=1)  # records the shape
+                run = generation_run(engine, sampler, b, ref_prompt, ref_new, cfg.vocab_size, one_step, look_ahead, seed=2)
+                assert run["decode_steps"] == ref_new - 1, run
+                sec = run["decode_s"] / (ref_new - 1)
+                nbytes = step_bytes(b, ref_prompt + ref_new / 2)
+                workload[f"b{b}"] = {
+                    "decode_tps": round(b * (ref_new - 1) / run["decode_s"], 1), "ms_per_step": round(sec * 1e3, 4),
+                    "gb_per_step": round(nbytes / 1e9, 3), "frac": round(nbytes / sec / 1e9 / HBM_GBS, 4),
+                    "prefill_tps": round(b * ref_prompt / run["prefill_s"], 1),
+                }
+
+    read_gbs = measured_read_gbs(engine.device)
     main_r = results[args.batch]
     achieved = main_r["bytes"] / main_r["sec"] / 1e9
     line = {
@@ -342,7 +483,7 @@ def main(argv=None) -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-        "data": "synthetic: random-init weights, random token ids, cache of earlier context filled with random values",
+        "data": "synthetic: random-init weights, prompts of random token ids prefilled through the scheduler, greedy decoding",
         "config": {
             "model": SHAPE_NAMES[args.shape],
             "global_batch": args.batch,
@@ -357,7 +498,10 @@ def main(argv=None) -> int:
             "intermediate_size": cfg.intermediate_size,
             "vocab_size": cfg.vocab_size,
             "page_size": args.page_size,
+            "prompt_tokens": prompt_len,
+            "new_tokens": new_tokens,
             "prefill_tokens": args.prefill_tokens,
+            "token_budget": args.token_budget,
             "rope": f"llama3 factor {shape['rope_scaling']['factor']:g} theta 5e5",
         },
         "prefill": {
@@ -372,8 +516,13 @@ def main(argv=None) -> int:
             "peak": HBM_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_GBS, 4),
+            "measured_read_peak": round(read_gbs, 1),
+            "frac_of_measured": round(achieved / read_gbs, 4),
         },
         "points": {f"decode_b{b}": round(r["tps"], 2) for b, r in results.items() if b != args.batch},
+        "points_frac": {f"decode_b{b}": round(r["bytes"] / r["sec"] / 1e9 / HBM_GBS, 4) for b, r in results.items() if b != args.batch},
+        "mean_context": {f"b{b}": round(r["mean_ctx"], 1) for b, r in results.items()},
+        "workload": dict(workload, prompt_tokens=2048, new_tokens=256, mean_context=2176) if workload else None,
     }
     print(json.dumps(line))
     return 0

@@ -191,9 +191,11 @@ def build_variant(kind: str, value: int, force: bool = False) -> Path:
 
 register_variant("attn_decode", "attention_decode.hip", "TL_HEAD_DIM")
 register_variant("attn_prefill", "attention_prefill.hip", "TL_HEAD_DIM")
+# the roofline micro-benchmarks of bench.py (one library; the macro only names its version)
+register_variant("peaks", "peaks.hip", "TL_PEAKS")
 
 #: sizes compiled ahead of time by ``build_all`` (tests, the smoke run and the benchmark use these)
-PREBUILT_VARIANTS: Dict[str, Iterable[int]] = {"attn_decode": (32, 64, 128, 256), "attn_prefill": (32, 64, 128, 256)}
+PREBUILT_VARIANTS: Dict[str, Iterable[int]] = {"attn_decode": (32, 64, 128, 256), "attn_prefill": (32, 64, 128, 256), "peaks": (1,)}
 
 
 def build_all(force: bool = False) -> List[Path]:
