@@ -310,6 +310,28 @@ def test_gemm_f32_is_true_32_bit(m, n, k):
     assert torch.equal(alone[0], got[0])
 
 
+@pytest.mark.parametrize("n, k", [(64, 4096), (50, 1030), (4099, 100), (16, 14336), (33, 16), (7, 5)])
+def test_gemm_f32_with_few_rows_gives_the_bits_of_the_kernel_for_many(n, k):
+    """Up to 16 rows (decode steps) take a kernel that spreads an element's groups of 16 products over
+    the lanes of a wave and adds their sums in the groups' order: the same arithmetic per element as the
+    tiled kernel for more rows, so the same bits, whatever the number of rows, also where K is no
+    multiple of 16 or of a round of 1,024, N no multiple of 16, and rows are strided."""
+    torch.manual_seed(n + k)
+    x = torch.randn(40, k + 3)[:, :k].to(DEV)  # rows with a stride that is no multiple of 4
+    w = torch.randn(n, k).to(DEV)
+    many = _ops().gemm_f32(x, w)  # 40 rows: the tiled kernel
+    want = x.double() @ w.double().T
+    assert (many.double() - want).abs().max().item() < 2e-6 * math.sqrt(k) * 4
+    for rows in (1, 2, 3, 4, 7, 8, 13, 16):
+        few = _ops().gemm_f32(x[:rows], w)
+        assert torch.equal(few, many[:rows]), f"{rows} rows differ from the tiled kernel"
+    shifted = _ops().gemm_f32(x[5:8], w)
+    assert torch.equal(shifted, many[5:8])
+    if k % 4 == 0:
+        aligned = _ops().gemm_f32(x[:2].contiguous(), w)
+        assert torch.equal(aligned, many[:2])
+
+
 # ----------------------------------------------------------------------------- attention
 def _paged(k, v, page, n_pages, seed=0, dtype=torch.float32):
     """Scatter dense per-request keys/values [S, Hkv, dh] into shuffled pages; returns pages and
@@ -373,6 +395,35 @@ def test_attention_generic(dtype, hq, hkv, dh, page, S, sq):
         torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
     else:
         torch.testing.assert_close(got, want, rtol=2 ** -7, atol=2 ** -7)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize(
+    "hq, hkv, dh, page, S, sq, window",
+    [(4, 2, 16, 8, 37, 3, 0), (6, 3, 48, 4, 150, 9, 0), (8, 1, 128, 16, 700, 2, 0), (3, 3, 6, 32, 270, 5, 0), (2, 1, 256, 16, 65, 2, 0),
+     (4, 4, 64, 1, 200, 4, 70), (5, 5, 32, 16, 1000, 3, 64), (2, 2, 80, 8, 129, 1, 0)],
+)
+def test_attention_generic_in_blocks_of_their_own_gives_the_same_bits(dtype, hq, hkv, dh, page, S, sq, window):
+    """The plain kernel computes every block of 64 keys by itself and lets the blocks join in ascending
+    order; for decode steps the blocks are computed by waves of their own and joined by a second
+    kernel.  Same blocks, same operations, same order: the same bits, with a window and without, with
+    head sizes that are no multiple of 4, and whatever the bound on the context says."""
+    torch.manual_seed(5)
+    q = torch.randn(sq, hq, dh) * 2
+    k = torch.randn(S, hkv, dh)
+    v = torch.randn(S, hkv, dh)
+    one_wave = _attend(_ops().attention_generic, q, k, v, page, window=window, dtype=dtype)
+    want = _windowed_plain(q, k, v, window)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -6, atol=2 ** -6)
+    if dtype == torch.bfloat16:
+        want = _windowed_plain(q.bfloat16().float(), k.bfloat16().float(), v.bfloat16().float(), window)
+    torch.testing.assert_close(one_wave, want, **tol)
+    for longest in (S, S + 200, min(window, S) if window else S):
+        def split(*a):
+            return _ops().attention_generic_split(*a, longest=longest)
+
+        many = _attend(split, q, k, v, page, window=window, dtype=dtype)
+        assert torch.equal(many, one_wave), f"bound {longest}"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

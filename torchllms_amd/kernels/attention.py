@@ -11,6 +11,9 @@ import torch
 
 from . import ops
 
+#: contexts beyond this many keys give every block of 64 keys a wave of its own in the plain kernel
+GENERIC_SPLIT_FROM = 128
+
 
 def paged_attention(
     qkv: torch.Tensor,
@@ -31,19 +34,15 @@ def paged_attention(
     fast_decode = n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
     # the MFMA prefill kernel takes positive softmax scales only; anything else runs the plain kernel
     fast_prefill = n_dec < n and scale > 0 and ops.prefill_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
-    if not fast_decode and not fast_prefill:
-        return ops.attention_generic(
-            qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq, ctx.positions,
-            ctx.block_tables[group], window, scale,
-        )
     out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
-    # rows with a single new token come first in the batch: they take the split-KV decode kernel
+    # rows with a single new token come first in the batch
     if n_dec > 0:
+        if ctx.decode_longest is not None:
+            longest = ctx.decode_longest
+        else:
+            longest = int(ctx.host.positions[:n_dec].max()) + 1
         if fast_decode:
-            if ctx.decode_longest is not None:
-                longest = ctx.decode_longest
-            else:
-                longest = int(ctx.host.positions[:n_dec].max()) + 1
+            # the split-KV MFMA kernel
             if window > 0:
                 longest = min(longest, window + 15)
             uneven = ctx.decode_uneven if ctx.decode_uneven is not None else ctx.host.decode_uneven
@@ -53,9 +52,15 @@ def paged_attention(
                 uneven=uneven,
             )
         else:
-            ops.attention_generic(
+            # the plain kernel: one wave a (token, head) would walk the whole context alone, so the
+            # blocks of 64 keys get waves of their own (the same bits either way)
+            if window > 0:
+                longest = min(longest, window)
+            plain = ops.attention_generic_split if longest > GENERIC_SPLIT_FROM else ops.attention_generic
+            extra = dict(longest=longest) if longest > GENERIC_SPLIT_FROM else {}
+            plain(
                 qkv[:n_dec], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[:n_dec],
-                ctx.positions[:n_dec], ctx.block_tables[group], window, scale, out=out[:n_dec],
+                ctx.positions[:n_dec], ctx.block_tables[group], window, scale, out=out[:n_dec], **extra,
             )
     # rows that bring a portion of a prompt take the tiled MFMA kernel
     if n_dec < n:

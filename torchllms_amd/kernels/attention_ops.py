@@ -73,6 +73,55 @@ def attention_generic(
 
 # ----------------------------------------------------------------------------- decode attention (bfloat16, MFMA)
 _P, _I, _F = __import__("ctypes").c_void_p, __import__("ctypes").c_int, __import__("ctypes").c_float
+def attention_generic_split(
+    qkv: torch.Tensor,
+    n_q_heads: int,
+    n_kv_heads: int,
+    head_dim: int,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    token_seq: torch.Tensor,
+    positions: torch.Tensor,
+    block_table: torch.Tensor,
+    window: int,
+    scale: float,
+    longest: int,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """``attention_generic`` for steps with few tokens and long contexts (decode): every block of 64
+    keys is computed by a wave of its own and a second kernel joins the blocks in order.  The same
+    blocks, operations and order as the one-wave form: the same bits.  ``longest``: an upper bound of
+    the keys any token sees (its position + 1, or the window)."""
+    _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
+    _i32(token_seq, "token_seq")
+    _i32(positions, "positions")
+    n = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention: qkv must be row-major with at least Hq * dh columns")
+    if token_seq.numel() != n or positions.numel() != n:
+        raise KernelError("attention: token_seq and positions need one entry per token")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("attention: block_table must be an int32 matrix")
+    page_size = k_pages.shape[2]
+    for pg in (k_pages, v_pages):
+        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+            raise KernelError("attention: pages must be contiguous [pages, Hkv, page_size, dh] of the query's dtype")
+    if out is None:
+        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    # blocks are aligned to absolute positions: a range of `longest` keys touches at most this many
+    max_blocks = max(int(longest), 1) // 64 + 2
+    partials = torch.empty((n, n_q_heads, max_blocks, head_dim + 2), dtype=torch.float32, device=qkv.device)
+    check(
+        core().tl_attention_generic_split(
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
+            n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), dtype_code(qkv.dtype), max_blocks,
+            partials.data_ptr(), _stream(),
+        )
+    )
+    return out
+
+
 _DECODE_SIGNATURES = {
     "tl_attn_decode": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P],
 }

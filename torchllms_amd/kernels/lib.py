@@ -33,6 +33,7 @@ _CORE_SIGNATURES = {
     "tl_silu_mul": [_P, _P, _I, _I, _I, _P],
     "tl_add_bias": [_P, _P, _I, _I, _I, _I, _P],
     "tl_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "tl_attention_generic_split": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
     "tl_gemm_f32": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],

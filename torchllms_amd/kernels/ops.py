@@ -69,6 +69,7 @@ from .attention_ops import (  # noqa: F401
     PREFILL_SPLIT_BLOCKS,
     attention_decode,
     attention_generic,
+    attention_generic_split,
     attention_prefill,
     decode_attention_supported,
     plan_decode_splits,
