@@ -1066,7 +1066,8 @@ def _prefill(rows, hq, hkv, dh, page, window=0, seed=0, key_groups=1):
         (6, 2, 64, 4, [(90, 31), (40, 40)]),
         (16, 1, 128, 32, [(129, 129)]),
         (4, 1, 256, 16, [(100, 100), (70, 5)]),
-        (5, 5, 32, 12, [(61, 61)]),
+        (5, 5, 32, 2, [(61, 61)]),
+        (5, 5, 32, 128, [(261, 261), (140, 3)]),
         (2, 2, 64, 16, [(1, 1), (2, 2), (17, 16)]),
     ],
 )
@@ -1076,6 +1077,15 @@ def test_attention_prefill(hq, hkv, dh, page, rows, key_groups):
     up at the end; a row of fewer keys than two tiles leaves the second set without any."""
     got, want = _prefill(rows, hq, hkv, dh, page, key_groups=key_groups)
     torch.testing.assert_close(got, want, rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_attention_prefill_takes_pages_of_a_power_of_two_only():
+    """Pages of 12 tokens are refused by the MFMA kernel with a clear error (and sent to the plain
+    kernel by the dispatcher: tests/test_gpu_random_configs.py runs such page sizes end to end)."""
+    ops = _ops()
+    assert ops.prefill_attention_supported(torch.bfloat16, 4, 2, 64, 16) and not ops.prefill_attention_supported(torch.bfloat16, 4, 2, 64, 12)
+    with pytest.raises(ops.KernelError, match="page_size 12 is no power of two"):
+        _prefill([(61, 61)], 5, 5, 32, 12)
 
 
 @pytest.mark.parametrize("key_groups", [1, 2])

@@ -91,7 +91,7 @@ struct PrefillArgs {
   int n_kv_heads;
   int group;
   int page_size;
-  int page_shift;
+  int page_shift;  // log2(page_size)
   int window;
   float scale_log2e;
 };
@@ -122,9 +122,14 @@ __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_ex
 // The block's LDS: [group][buffer][keys | values][kTileElems].  It is declared here and not in the
 // kernel: a __shared__ array whose size depends on a template parameter of the kernel itself keeps
 // this compiler from emitting the kernel's host stub.
+// With two groups the second one hands its results over through the same memory at the end: per
+// lane and column block a maximum, a sum and the output's 4 * DT sums, as 32-bit floats.
+constexpr int kExchangeBytes = NC * (2 + 4 * DT) * kWaves * kWave * 4;
 template <int GROUPS>
 __device__ __forceinline__ bf16_t* tile_memory() {
-  __shared__ __attribute__((aligned(16))) bf16_t tiles[GROUPS * 2 * 2 * kTileElems];
+  constexpr int kTileBytes = GROUPS * 2 * 2 * kTileElems * 2;
+  constexpr int kBytes = GROUPS == 2 && kExchangeBytes > kTileBytes ? kExchangeBytes : kTileBytes;
+  __shared__ __attribute__((aligned(16))) bf16_t tiles[kBytes / 2];
   return tiles;
 }
 
@@ -195,77 +200,70 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
       if (!col_ok[i]) qreg[i][u].u = u32x4_t{0u, 0u, 0u, 0u};
     }
   }
-  // range of keys this wave's columns can see at all (tiles outside it are skipped)
-  int wave_hi = -1, wave_lo = 0x3fffffff;
-#pragma unroll
-  for (int i = 0; i < NC; ++i) {
-    const int p_ok = col_ok[i] ? col_pos[i] : -1;
-    const int l_ok = col_ok[i] ? col_lo[i] : 0x3fffffff;
-    wave_hi = max(wave_hi, p_ok);
-    wave_lo = min(wave_lo, l_ok);
-  }
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    wave_hi = max(wave_hi, __shfl_xor(wave_hi, off, kWave));
-    wave_lo = min(wave_lo, __shfl_xor(wave_lo, off, kWave));
-  }
-
-  float m_run[NC], l_part[NC];
+  float m_run[NC];
   float4_t acc[NC][DT];
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
     m_run[i] = -INFINITY;
-    l_part[i] = 0.f;
 #pragma unroll
     for (int t = 0; t < DT; ++t) acc[i][t] = float4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // global -> LDS for one tile of keys and values, asynchronously.  Wave load j of wave w covers rows
+  // global -> LDS for one tile of keys or of values, asynchronously.  Wave load j of wave w covers rows
   // (j * kWaves + w) * kRowsPerLoad ... of the tile: lane -> (row, slot), and fetches the piece that
   // belongs in that slot.  Keys outside the visible range are clamped into it (their scores are
   // masked), so no load touches a page the request does not hold.
-  auto dma = [&](int base, int buffer) {
+  // The pages of a tile's rows are looked up one pass before the loads that need them are issued
+  // (`lookup`, then `dma` with what it found), so that no pass begins by waiting for its block table.
+  // Rows outside the visible range (before a window's edge, behind the last key) are fetched from the
+  // nearest page the request holds, at their own offset in the page: any row of a held page is memory
+  // that may be read, and their scores are masked.  Addresses are a page's offset (one 64-bit
+  // multiply-add per load) plus what does not depend on the page.
+  const int blk_lo = key_lo >> a.page_shift, blk_hi = key_hi >> a.page_shift;
+  const unsigned page_bytes = (unsigned)a.n_kv_heads * (unsigned)a.page_size * DH * 2;  // all kv heads of a page
+  const char* const k_head = reinterpret_cast<const char*>(a.k_pages) + (size_t)kvh * head_elems * 2;  // this kv head's rows in page 0
+  const char* const v_head = reinterpret_cast<const char*>(a.v_pages) + (size_t)kvh * head_elems * 2;
+  const int my_row = lane / kPieces + wave * kRowsPerLoad;  // this lane's row within a wave load's turn
+  struct Rows {
+    int page[kLoadsPerWave];
+  };
+  auto lookup = [&](int base, Rows& rows) {
+#pragma unroll
+    for (int j = 0; j < kLoadsPerWave; ++j) {
+      int blk = (base + j * kWaves * kRowsPerLoad + my_row) >> a.page_shift;
+      blk = blk < blk_lo ? blk_lo : (blk > blk_hi ? blk_hi : blk);
+      rows.page[j] = bt[blk];
+    }
+  };
+  auto dma = [&](int base, const Rows& rows, int buffer, bool values) {
 #pragma unroll
     for (int j = 0; j < kLoadsPerWave; ++j) {
       const int first = (j * kWaves + wave) * kRowsPerLoad;
       const int r = first + lane / kPieces;
-      const int piece_k = (lane % kPieces) ^ swizzle(r);
-      const int piece_v = (lane % kPieces) ^ swizzle_v(r);
-      int key = base + r;
-      key = key < key_lo ? key_lo : (key > key_hi ? key_hi : key);
-      const int blk = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
-      const int off = a.page_shift >= 0 ? key & (a.page_size - 1) : key % a.page_size;
-      const size_t at = ((size_t)bt[blk] * a.n_kv_heads + kvh) * head_elems + (size_t)off * DH;
-      __builtin_amdgcn_global_load_lds(a.k_pages + at + 8 * piece_k, &tiles[(2 * buffer) * kTileElems + first * DH], 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(a.v_pages + at + 8 * piece_v, &tiles[(2 * buffer + 1) * kTileElems + first * DH], 16, 0, 0);
+      const int piece = (lane % kPieces) ^ (values ? swizzle_v(r) : swizzle(r));
+      const unsigned in_page = (unsigned)((base + r) & (a.page_size - 1)) * (DH * 2) + 16 * piece;
+      const char* src = (values ? v_head : k_head) + ((size_t)(unsigned)rows.page[j] * page_bytes + in_page);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const bf16_t*>(src),
+                                       &tiles[(2 * buffer + (values ? 1 : 0)) * kTileElems + first * DH], 16, 0, 0);
     }
   };
 
-  dma(tile_begin + grp * KT, 0);
-  int buffer = 0;
-  // One tile of keys: wait for it, start the next one's loads, work it off.  `masked`: whether some
-  // column may not see some key of the tile; where every column sees every key the tests are
-  // compiled out.
-  auto work_tile = [&](int base, auto masked) {
-    // this wave's loads of the tile have landed; after the barrier everybody's have, and everybody
-    // has finished with the tile before, whose buffer the next tile's loads may now overwrite
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    dma(base + GROUPS * KT, buffer ^ 1);  // unconditional (keys are clamped): no wait has to cover a path without it
-    const bf16_t* k_lds = tiles + (2 * buffer) * kTileElems;
-    const bf16_t* v_lds = tiles + (2 * buffer + 1) * kTileElems;
+  constexpr int NS = KT / 16;  // blocks of 16 keys in a tile
+  // The tiles of keys are worked off in a pipeline of three stages, so that the matrix cores and the
+  // vector units have independent work at the same time within one wave:
+  //   scores of tile t+1 (MFMA)  |  softmax of tile t (vector)  |  output of tile t-1 (MFMA)
+  // One pass of the loop does the softmax of tile t beside the output product of tile t-1, then the
+  // rescaling of the sums beside the scores of tile t+1.  Keys are fetched two tiles ahead and values
+  // as their tile's scores are computed; each lands one pass before it is read.
+  float4_t c[NC][NS];                  // scores S^T of the current tile
+  bf16x8_t pb_prev[NC][NS / 2];        // probabilities of the tile before, as the B operand of the output product
+  float4_t acc_l[NC];                  // sums of probabilities: the output product with a row of ones as its values
+#pragma unroll
+  for (int i = 0; i < NC; ++i) acc_l[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+  const bf16x8_t ones = __builtin_bit_cast(bf16x8_t, u32x4_t{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
 
-    if (base > wave_hi || base + KT - 1 < wave_lo) return;  // nothing here for this wave's columns
-
-    // the whole tile at once: scores, softmax bookkeeping (one running maximum and one rescaling of
-    // the sums per tile), then P.V in groups of 32 keys
-    constexpr int NS = KT / 16;  // blocks of 16 keys
-    {
-    // phase 1: scores S^T[key][column], one MFMA chain per (16 keys, column block).  No branch from
-    // here to the end of the tile, so that the compiler can interleave the chains and the column
-    // blocks' softmax arithmetic; a block of 16 keys that the wave does not see at all is computed
-    // and masked like any other.
-    float4_t c[NC][NS];
+  // scores S^T[key][column] of one tile, one MFMA chain per (16 keys, column block)
+  auto scores = [&](const bf16_t* k_lds) {
 #pragma unroll
     for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
@@ -282,72 +280,20 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
         for (int i = 0; i < NC; ++i)
           c[i][sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[sub].op(), qreg[i][u].op(), c[i][sub], 0, 0, 0);
     }
-    // softmax bookkeeping once per tile and column: mask, maximum, rescale, probabilities.
-    // Scores stay unscaled; the scale enters through one fused multiply-add per element:
-    // exp2(s * scale - m), with m the running maximum of s * scale.
-    bf16x8_t pb[NC][NS / 2];  // per 32 keys; slot e < 4: key 4 g4 + e of the first 16 keys; e >= 4: of the second 16
-    float alpha[NC];
-#pragma unroll
-    for (int i = 0; i < NC; ++i) {
-      float tmax = -INFINITY;
-#pragma unroll
-      for (int sub = 0; sub < NS; ++sub)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          // plain bit operations, no short-circuit: a branch here, right behind the MFMAs, is what
-          // this compiler has been seen to get wrong (the masked value overwrote live scores)
-          float sc = c[i][sub][r];
-          if constexpr (decltype(masked)::value) {
-            const int key = base + 16 * sub + 4 * g4 + r;
-            const bool valid = WINDOWED ? (key >= col_lo[i]) & (key <= col_pos[i]) : key <= col_pos[i];
-            sc = valid ? sc : -INFINITY;
-            c[i][sub][r] = sc;
-          }
-          tmax = fmaxf(tmax, sc);
-        }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-      const float m_new = fmaxf(m_run[i], tmax * a.scale_log2e);  // the scale is positive
-      // a column may not have met a visible key yet: then nothing is rescaled and nothing added
-      const bool none = m_new == -INFINITY;
-      alpha[i] = none ? 1.f : __builtin_amdgcn_exp2f(m_run[i] - m_new);
-      const float neg_m = none ? 0.f : -m_new;
-      float psum = 0.f;
-      uint32_t pw[2 * NS];
-#pragma unroll
-      for (int sub = 0; sub < NS; ++sub) {
-        float pr[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          pr[r] = __builtin_amdgcn_exp2f(fmaf(c[i][sub][r], a.scale_log2e, neg_m));  // exp2(-inf) = 0
-          psum += pr[r];
-        }
-        pw[2 * sub] = pack_bf16x2(pr[0], pr[1]);
-        pw[2 * sub + 1] = pack_bf16x2(pr[2], pr[3]);
-      }
-#pragma unroll
-      for (int g = 0; g < NS / 2; ++g)
-        pb[i][g] = __builtin_bit_cast(bf16x8_t, u32x4_t{pw[4 * g], pw[4 * g + 1], pw[4 * g + 2], pw[4 * g + 3]});
-      l_part[i] = l_part[i] * alpha[i] + psum;
-      m_run[i] = m_new;
-    }
-    // the sums so far follow the maxima (no test whether any moved: a branch here keeps the compiler
-    // from overlapping this arithmetic with the MFMAs around it, which costs more than it saves)
-#pragma unroll
-    for (int i = 0; i < NC; ++i)
-#pragma unroll
-      for (int t = 0; t < DT; ++t)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha[i];
-    // phase 2: O^T[channel][column] += V^T[channel][key] P^T[key][column], 32 keys at a time, 16
-    // channels an MFMA.  Its A operand (lane (m, g4): channel 16 t + m of the keys 4 g4 .. + 3 and
-    // 16 + 4 g4 .. + 3, the order in which the probabilities lie in pb) comes from two transposing
-    // loads.  A block of 16 keys that no column of the wave sees has zero probabilities: its rows are
-    // read all the same (they lie in the tile) and add nothing.
-    const int tr_row = 4 * g4 + n16 / 4;  // the key row this lane points at, within 16 keys
-    const int tr_ch = 4 * (n16 % 4);      // the first of its four channels, within 16 channels
+  };
+
+  // O^T[channel][column] += V^T[channel][key] P^T[key][column], 32 keys at a time, 16 channels an MFMA.
+  // Its A operand (lane (m, g4): channel 16 t + m of the keys 4 g4 .. + 3 and 16 + 4 g4 .. + 3, the
+  // order in which the probabilities lie in pb) comes from two transposing loads.  The sum of the
+  // probabilities is the same product with ones for values: a few MFMAs instead of an addition per
+  // score, and exactly the sum of what the output was weighted with.
+  const int tr_row = 4 * g4 + n16 / 4;  // the key row this lane points at, within 16 keys
+  const int tr_ch = 4 * (n16 % 4);      // the first of its four channels, within 16 channels
+  auto output = [&](const bf16_t* v_lds, const bf16x8_t (&pb)[NC][NS / 2]) {
 #pragma unroll
     for (int g = 0; g < NS / 2; ++g) {
+#pragma unroll
+      for (int i = 0; i < NC; ++i) acc_l[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pb[i][g], acc_l[i], 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
         const int r0 = 32 * g + tr_row, r1 = r0 + 16;
@@ -359,30 +305,150 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
         for (int i = 0; i < NC; ++i) acc[i][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb[i][g], acc[i][t], 0, 0, 0);
       }
     }
+  };
+
+  // Softmax bookkeeping of the tile whose scores are in c, once per tile and column: mask, maximum,
+  // probabilities (into pb), and alpha, the factor by which everything summed so far shrinks.
+  // Scores stay unscaled; the scale enters through one fused multiply-add per element:
+  // exp2(s * scale - m), with m the running maximum of s * scale.  `masked`: whether some column may
+  // not see some key of the tile; where every column sees every key the tests are compiled out.
+  constexpr float kSlack = 8.f;
+  // scores of keys that a column does not see become -inf (plain selects, no short-circuit)
+  auto mask = [&](int base) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+#pragma unroll
+      for (int sub = 0; sub < NS; ++sub)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int key = base + 16 * sub + 4 * g4 + r;
+          const bool valid = WINDOWED ? (key >= col_lo[i]) & (key <= col_pos[i]) : key <= col_pos[i];
+          c[i][sub][r] = valid ? c[i][sub][r] : -INFINITY;
+        }
+  };
+  auto softmax = [&](bf16x8_t (&pb)[NC][NS / 2], float (&alpha)[NC], bool& moved) {
+    moved = false;
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int sub = 0; sub < NS; ++sub)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, c[i][sub][r]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      // The reference maximum of a column only moves when a score exceeds it by more than kSlack
+      // powers of two.  Until then the tile's probabilities may exceed 1, by at most 2^kSlack, which
+      // costs nothing (32-bit sums, and bfloat16 keeps its relative precision), and everything summed
+      // so far keeps its scale: most tiles need no rescaling at all.
+      const float t_max = tmax * a.scale_log2e;  // the scale is positive
+      const bool move = t_max > m_run[i] + kSlack;  // also the first visible key of a column (from -inf)
+      moved |= move;
+      const float m_new = move ? t_max : m_run[i];
+      alpha[i] = move ? __builtin_amdgcn_exp2f(m_run[i] - m_new) : 1.f;
+      // a column may not have met a visible key yet: then its scores are all -inf and nothing is added
+      const float neg_m = m_new == -INFINITY ? 0.f : -m_new;
+      uint32_t pw[2 * NS];
+#pragma unroll
+      for (int sub = 0; sub < NS; ++sub) {
+        float pr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pr[r] = __builtin_amdgcn_exp2f(fmaf(c[i][sub][r], a.scale_log2e, neg_m));  // exp2(-inf) = 0
+        pw[2 * sub] = pack_bf16x2(pr[0], pr[1]);
+        pw[2 * sub + 1] = pack_bf16x2(pr[2], pr[3]);
+      }
+#pragma unroll
+      for (int g = 0; g < NS / 2; ++g)
+        pb[i][g] = __builtin_bit_cast(bf16x8_t, u32x4_t{pw[4 * g], pw[4 * g + 1], pw[4 * g + 2], pw[4 * g + 3]});
+      m_run[i] = m_new;
     }
   };
-  // Tiles that lie wholly before the tile's first query (and after no window's edge) are seen by all
-  // columns of the block: they run in a loop of their own, without masks.  The two loops are code
-  // one after the other, not two arms of a branch inside one loop, which is what keeps the register
-  // count where it was.
+
+  // everything summed so far follows the maxima that moved
+  auto rescale = [&](const float (&alpha)[NC]) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc_l[i][r] *= alpha[i];
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[i][t][r] *= alpha[i];
+    }
+  };
+
   // Every wave of the block passes the same number of barriers: with two groups both make as many
-  // steps, and the second one's last tile may lie past the last key (then it only waits and loads).
+  // steps, and the second one's last tile may lie past the last key (its keys are clamped and masked).
   const int n_steps = ((key_hi - tile_begin) / KT + GROUPS) / GROUPS;
-  int base = tile_begin + grp * KT;
-  int step = 0;
-  if (!WINDOWED) {
-    for (; step < n_steps && base + KT - 1 <= pos0 + q0; ++step, base += GROUPS * KT, buffer ^= 1)
-      work_tile(base, std::false_type{});
-  }
-  for (; step < n_steps; ++step, base += GROUPS * KT, buffer ^= 1) work_tile(base, std::true_type{});
+  auto base_of = [&](int step) { return tile_begin + (step * GROUPS + grp) * KT; };
+  auto k_tile = [&](int step) { return tiles + (2 * (step & 1)) * kTileElems; };
+  auto v_tile = [&](int step) { return tiles + (2 * (step & 1) + 1) * kTileElems; };
+
+  Rows rows_k, rows_v;  // the rows of the next pass's loads: keys of tile step + 2, values of tile step
+  lookup(base_of(0), rows_v);
+  lookup(base_of(1), rows_k);
+  dma(base_of(0), rows_v, 0, false);  // (tile 0's keys lie where its values do)
+  dma(base_of(1), rows_k, 1, false);
+  lookup(base_of(2), rows_k);
+  // the first pass has no tile before it: its output product runs all the same (no branch in a pass),
+  // on probabilities of zero and values of zero
+#pragma unroll
+  for (int i = 0; i < NC; ++i)
+#pragma unroll
+    for (int g = 0; g < NS / 2; ++g) pb_prev[i][g] = __builtin_bit_cast(bf16x8_t, u32x4_t{0u, 0u, 0u, 0u});
+  for (int e = (wave * kWave + lane) * 8; e < kTileElems; e += kWaves * kWave * 8)
+    *reinterpret_cast<u32x4_t*>(&tiles[3 * kTileElems + e]) = u32x4_t{0u, 0u, 0u, 0u};  // the values' second buffer
+  wait_for_loads();
+  __syncthreads();
+  scores(k_tile(0));
+
+  // one pass: tile `step`'s softmax beside tile `step - 1`'s output, then the rescaling beside tile
+  // `step + 1`'s scores
+  auto pass = [&](int step) {
+    // this wave's loads of the pass before have landed (keys of tile step + 1, values of tile step - 1);
+    // after the barrier everybody's have, and everybody has finished with the buffers that this
+    // pass's loads overwrite (keys of tile step, values of tile step - 2)
+    wait_for_loads();
+    __syncthreads();
+    dma(base_of(step + 2), rows_k, step & 1, false);  // unconditional (pages are clamped): no wait has to cover a path without it
+    dma(base_of(step), rows_v, step & 1, true);
+    lookup(base_of(step + 3), rows_k);  // for the next pass
+    lookup(base_of(step + 1), rows_v);
+    bf16x8_t pb[NC][NS / 2];
+    float alpha[NC];
+    bool moved;
+    // a tile that lies wholly before the block's first query (and behind every window's edge) is seen
+    // whole by every column: no masks (the same decision for all waves of the block)
+    const int base = base_of(step);
+    if (base + KT - 1 > pos0 + q0 || (WINDOWED && base < window_lo(pos0 + q_last))) mask(base);
+    softmax(pb, alpha, moved);
+    output(v_tile(step - 1), pb_prev);
+    if (__any(moved)) rescale(alpha);  // (the same for the whole wave)
+    scores(k_tile(step + 1));
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+#pragma unroll
+      for (int g = 0; g < NS / 2; ++g) pb_prev[i][g] = pb[i][g];
+  };
+  // (One loop for all tiles.  Two loops, the first without masks for the tiles that every column sees
+  // whole, cost this compiler more registers than it has: everything the pipeline carries from pass to
+  // pass is then alive across both.)
+  for (int step = 0; step < n_steps; ++step) pass(step);
+  // the last tile's output
+  wait_for_loads();
+  __syncthreads();
+  output(v_tile(n_steps - 1), pb_prev);
+  // the sum of the probabilities of this lane's columns (every channel row of acc_l holds it)
+  float l_part[NC];
+#pragma unroll
+  for (int i = 0; i < NC; ++i) l_part[i] = acc_l[i][0];
 
   if constexpr (GROUPS == 2) {
     // The second group hands its maxima, sums and outputs to the first through the memory of the
     // tiles (nobody reads a tile any more, and the last, unused load has landed).  Value i of thread
     // t lies at i * 256 + t: consecutive lanes, consecutive words.
     constexpr int kPerLane = NC * (2 + 4 * DT);
-    static_assert(kPerLane * kWaves * kWave * sizeof(float) <= GROUPS * 4 * kTileElems * sizeof(bf16_t),
-                  "the tiles' memory is too small for the exchange");
+    static_assert(kPerLane * kWaves * kWave * sizeof(float) == kExchangeBytes, "the exchange is as large as tile_memory says");
     float* xch = reinterpret_cast<float*>(tile_memory<GROUPS>()) + (wave * kWave + lane);
     constexpr int kStride = kWaves * kWave;
     wait_for_loads();
@@ -419,9 +485,7 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
 
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
-    float l = l_part[i];
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
+    const float l = l_part[i];
     if (!col_ok[i]) continue;
     const float inv = 1.0f / l;
     bf16_t* orow = a.out + (size_t)col_tok[i] * a.out_stride + (size_t)col_head[i] * DH;
@@ -468,9 +532,10 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   a.qo_indptr = qo_indptr; a.kv_lens = kv_lens; a.block_table = block_table; a.bt_stride = bt_stride;
   a.tile_row = tile_row; a.tile_q0 = tile_q0;
   a.n_kv_heads = n_kv_heads; a.group = R; a.page_size = page_size; a.window = window;
-  a.page_shift = -1;
-  for (int sh = 0; sh < 31; ++sh)
-    if ((1 << sh) == page_size) a.page_shift = sh;
+  a.page_shift = 0;
+  while ((1 << a.page_shift) < page_size) ++a.page_shift;
+  if ((1 << a.page_shift) != page_size)
+    return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: page_size %d is no power of two", page_size);
   a.scale_log2e = scale * 1.4426950408889634f;
   dim3 grid(n_kv_heads, n_tiles);  // consecutive blocks share a query tile: their loads of q overlap
   const bool windowed = window > 0;

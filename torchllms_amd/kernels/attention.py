@@ -33,7 +33,7 @@ def paged_attention(
     n_dec = ctx.host.n_decode
     fast_decode = n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
     # the MFMA prefill kernel takes positive softmax scales only; anything else runs the plain kernel
-    fast_prefill = n_dec < n and scale > 0 and ops.prefill_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
+    fast_prefill = n_dec < n and scale > 0 and ops.prefill_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim, k_pages.shape[2])
     out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
     # rows with a single new token come first in the batch
     if n_dec > 0:
