@@ -171,3 +171,106 @@ def test_toy_architecture_is_registered_built_and_stepped():
     assert sum(p >= 0 for p in eng.cache.block_table("w", 1)) <= 2 < sum(p >= 0 for p in eng.cache.block_table("w", 0))
     assert len(eng.cache.block_table("w", 0)) == 8 and len(eng.cache.block_table("w", 1)) == 4  # 30 tokens in pages of 4 and of 8
     eng.free("w")
+
+
+def _register_windowed():
+    """Two attention layers from the framework's own parts, the second with a window of 20 keys in pages of
+    8: every part is fit for a recorded graph, so decode steps of this model are replayed and prepared ahead."""
+    from torchllms_amd.config import ArchSpec, register_architecture
+    from torchllms_amd.config.spec import LayerRun, ModelSpec, PartSpec, standard_layer
+    from torchllms_amd.weights import NameRule
+
+    window = 20
+
+    def spec(cfg: ToyConfig) -> ModelSpec:
+        rope = PartSpec("rope", dict(head_dim=DH, rotary_dim=DH, theta=100.0, scaling=None))
+        norm = PartSpec("rmsnorm", dict(size=HIDDEN, eps=1e-5))
+        ffn = PartSpec("swiglu", dict(hidden_size=HIDDEN, intermediate_size=FFN))
+
+        def attn(w):
+            return PartSpec("attention", dict(hidden_size=HIDDEN, num_heads=HEADS, num_kv_heads=KV, head_dim=DH, qkv_bias=False,
+                                              softmax_scale=DH ** -0.5, window=w, position=rope, kv_page_size=WINDOW_PAGE if w else None))
+
+        layers = [standard_layer(f"layers.{i}", "pre_norm", attn(w), ffn, norm, norm) for i, w in enumerate([0, window])]
+        return ModelSpec("ToyWindowedForCausalLM", HIDDEN, VOCAB, 512, PartSpec("embedding", dict(vocab_size=VOCAB, hidden_size=HIDDEN)),
+                         layers, [LayerRun(0), LayerRun(1)], norm, PartSpec("lm_head", dict(vocab_size=VOCAB, hidden_size=HIDDEN, tied=True)))
+
+    def rules(cfg):
+        per_layer = ["mixer_norm.weight", "ffn_norm.weight", "ffn.w1.weight", "ffn.w2.weight", "ffn.w3.weight",
+                     "mixer.wq.weight", "mixer.wk.weight", "mixer.wv.weight", "mixer.wo.weight"]
+        return [NameRule(n, n) for n in ("embed.weight", "final_norm.weight")] + [NameRule("layers.{}." + n, "layers.{}." + n) for n in per_layer]
+
+    arch = register_architecture(ArchSpec("ToyWindowedForCausalLM", lambda d: ToyConfig(**d), spec, rules))
+    return arch, window
+
+
+def test_windowed_layers_decode_through_graphs_and_prepared_steps():
+    """Decode steps of a model with a window are planned from the step before, replayed from a graph and
+    prepared a step ahead like any other: the pages that the window gives back leave the plan's block tables
+    as they leave the requests'.  Same bits as an engine that plans and launches every step by itself."""
+    from torchllms_amd.engine import Engine, StepEntry
+    from torchllms_amd.parts import Model
+    from torchllms_amd.weights import random_tensors
+
+    arch, window = _register_windowed()
+    cfg = ToyConfig(architectures=("ToyWindowedForCausalLM",))
+    w = random_tensors(Model(arch.model_spec(cfg)).param_specs(), seed=5, dtype=torch.float32, norm_jitter=0.1)
+    for name in w:
+        if name.endswith(("wq.weight", "wk.weight")):
+            w[name] = w[name] * 15
+    w = {k: v.to("cuda:0") for k, v in w.items()}
+    make = lambda graphs: Engine(arch, cfg, w, torch.float32, page_size=4, num_pages=120, max_seqs=4, max_model_len=512, use_graphs=graphs)
+    plain, ahead = make(False), make(True)
+    toks = {r: random_tokens(200, VOCAB, 70 + i) for i, r in enumerate("abc")}
+    start = {"a": 61, "b": 3, "c": 17}
+    for eng in (plain, ahead):
+        for r in toks:
+            eng.admit(r)
+        eng.step([StepEntry(r, toks[r][: start[r]], []) for r in toks])
+    used, prepared = 0, None
+    for step in range(90):
+        entries = [StepEntry(r, [toks[r][start[r] + step]], [0]) for r in toks]
+        plain._last_decode = None  # this engine plans every step from the requests' tables alone
+        want = plain.step(entries)
+        got = ahead.step_prepared(prepared, entries) if prepared is not None else None
+        used += got is not None
+        if got is None:
+            got = ahead.step(entries)
+        assert torch.equal(want, got), step
+        prepared = ahead.prepare_decode()
+        if prepared is not None:
+            # the next step's plan names exactly the pages that the requests hold now
+            for g in range(2):
+                for row, r in enumerate("abc"):
+                    table = ahead.cache.block_table(r, g)
+                    assert prepared.layout.block_tables[g][row, : len(table)].tolist() == table, (step, g, r)
+        ahead.cache.check_invariants()
+    assert used >= 75  # all but the first steps of a shape, which run eagerly before they are recorded
+    # the window gave pages back on the way: request a holds 151 tokens, of them the last 20 in the windowed group
+    assert sum(p >= 0 for p in ahead.cache.block_table("a", 1)) <= -(-window // WINDOW_PAGE) + 1
+    assert sum(p >= 0 for p in ahead.cache.block_table("a", 0)) == -(-151 // 4)
+    got = ahead.step([StepEntry("a", [toks["a"][151]], [0]), StepEntry("b", [toks["b"][93]], []), StepEntry("c", [toks["c"][107]], [])])
+    want = plain_windowed(w, toks["a"][:152], window)[-1]
+    assert (got[0].cpu() - want).abs().max().item() < 5e-5
+
+
+def plain_windowed(w, tokens, window):
+    """The two-layer windowed model over a whole sequence, no cache, no engine."""
+    w = {k: v.cpu() for k, v in w.items()}
+    S = len(tokens)
+    pos = torch.arange(S)
+    f = plain.rope_inverse_frequencies(DH, 100.0, None)
+    h = w["embed.weight"][torch.tensor(tokens)]
+    for layer, win in enumerate([0, window]):
+        p = f"layers.{layer}."
+        x = plain.rms_norm(h, w[p + "mixer_norm.weight"], 1e-5)
+        q = plain.rope_rotate_interleaved(F.linear(x, w[p + "mixer.wq.weight"]).view(S, HEADS, DH), pos, f)
+        k = plain.rope_rotate_interleaved(F.linear(x, w[p + "mixer.wk.weight"]).view(S, KV, DH), pos, f)
+        v = F.linear(x, w[p + "mixer.wv.weight"]).view(S, KV, DH)
+        rows = []
+        for i in range(S):
+            lo = max(i - win + 1, 0) if win else 0
+            rows.append(plain.attention(q[i : i + 1], k[lo : i + 1], v[lo : i + 1]))
+        h = h + F.linear(torch.cat(rows), w[p + "mixer.wo.weight"])
+        h = h + plain.swiglu(plain.rms_norm(h, w[p + "ffn_norm.weight"], 1e-5), w[p + "ffn.w1.weight"], w[p + "ffn.w3.weight"], w[p + "ffn.w2.weight"])
+    return F.linear(plain.rms_norm(h, w["final_norm.weight"], 1e-5), w["embed.weight"])

@@ -159,6 +159,26 @@ def test_a_lone_request_that_outgrows_the_pool_is_caught_at_add():
     assert eng.cache.live == []
 
 
+def test_a_window_bounds_what_a_request_must_hold():
+    # every group has a window of 6 keys: a request holds the pages those keys touch and no more, so a
+    # pool of five pages takes a request of 60 tokens (fifteen pages if none came back), cut into the
+    # portions the free pages hold, and generates what an ample pool generates
+    prompt = list(range(1, 41))
+    tight_engine = FakeEngine(num_pages=5, page_size=4, window=6)
+    (tight,), _, _ = generate([prompt], max_new_tokens=20, engine=tight_engine)
+    (ample,), _, _ = generate([prompt], max_new_tokens=20, engine=FakeEngine(num_pages=64, page_size=4, window=6))
+    assert tight.output == ample.output and len(tight.output) == 20 and tight.preemptions == 0
+    assert max(n for call in tight_engine.calls for _, _, n in call) <= 20  # no portion beyond the pool
+    # beside a group that keeps every key the request is still refused: that group needs all fifteen
+    groups = [CacheGroupSpec("full", ("a",), 1, 4, 0), CacheGroupSpec("windowed", ("b",), 1, 4, 6)]
+    loop = GenerationLoop(FakeEngine(num_pages=5, page_size=4, groups=groups), greedy, 4, 64, 256)
+    with pytest.raises(ValueError, match="60 tokens need 15 pages"):
+        loop.run([prompt], [SamplingParams(max_new_tokens=21)])
+    # and a window wider than the pool is refused too
+    with pytest.raises(ValueError, match="could never finish"):
+        GenerationLoop(FakeEngine(num_pages=2, page_size=4, window=9), greedy, 4, 64, 256).run([prompt], [SamplingParams(max_new_tokens=4)])
+
+
 def test_failure_gives_everything_back():
     eng = FakeEngine()
 

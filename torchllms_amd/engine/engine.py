@@ -130,7 +130,6 @@ class Engine:
                     capacity = max_seqs * (-(-self.max_model_len // page_size)) * page_size
             pages = CacheManager.pages_for_tokens(groups, page_size, max(capacity, 1))
         self.cache = CacheManager(groups, states, page_size, pages, max_seqs, dtype=dtype, device=self.device)
-        self._windowed = any(g.window > 0 for g in groups)
         self.steps_run = 0
         self.tokens_run = 0
         # the last step's plan when every row of it brought one token: (request ids, wanted places,
@@ -267,6 +266,14 @@ class Engine:
                     blk = int(positions[i]) // page
                     bt[i, blk] = cache.block_table(rids[i], g)[blk]
                     sm[i] = bt[i, blk] * page
+            window = cache.groups[g].window
+            if window > 0:
+                # the last step's advance gave back the pages that the window has passed: their
+                # blocks are -1 in the requests' tables, and so they are here
+                first_live = np.maximum(positions - window + 1, 0) // page
+                released = np.arange(bt.shape[1], dtype=np.int64)[None, :] < first_live[:, None]
+                if (released & (bt >= 0)).any():
+                    bt = np.where(released, np.int32(-1), bt)
             tables.append(bt)
             slots.append(sm)
         return StepLayout(
@@ -282,10 +289,9 @@ class Engine:
         decode step of the same requests (one token each, the same wanted places) that does not
         depend on the tokens is done now, the plan made, its pages taken, the upload buffer filled.
         ``step_prepared`` then only needs the tokens.  None when there is nothing to prepare: the
-        last step was no decode step, pages are short, a window releases pages, the step's shape has
-        no recorded graph yet.  A preparation that is never used costs nothing but the pages it took
+        last step was no decode step, pages are short, the step's shape has no recorded graph yet.  A preparation that is never used costs nothing but the pages it took
         early, which their requests keep, and would have taken with the step anyway."""
-        if self.graphs is None or self._windowed or self._last_decode is None:
+        if self.graphs is None or self._last_decode is None:
             return None
         rids, wants, prev, epoch = self._last_decode
         if epoch != self.cache.epoch:
@@ -329,11 +335,10 @@ class Engine:
     def plan(self, entries: Sequence[StepEntry]) -> StepLayout:
         """Reserve pages for the step's tokens (all or nothing) and lay the step out."""
         # decode steps follow one another with the same requests: such a step is planned from the
-        # last one's plan.  Pages that a window releases change block tables behind the planner's
-        # back, so models with windows always take the general path.
+        # last one's plan
         if self._last_decode is not None:
             last = self._last_decode
-            layout = self._plan_next_decode(entries) if not self._windowed else None
+            layout = self._plan_next_decode(entries)
             self._last_decode = None
             if layout is not None:
                 self._last_decode = (last[0], last[1], layout, self.cache.epoch)

@@ -132,9 +132,10 @@ class Scheduler:
         # the longest it can get: all but the last generated token sit in the cache
         longest = len(prompt) + req.budget - 1
         for g, pool in enumerate(self.cache.pools):
-            if self.cache.blocks_for(longest, g) > pool.num_pages:
+            need = self._most_pages_held(g, longest)
+            if need > pool.num_pages:
                 raise ValueError(
-                    f"request {rid!r}: {longest} tokens need {self.cache.blocks_for(longest, g)} pages, "
+                    f"request {rid!r}: {longest} tokens need {need} pages, "
                     f"the pool has {pool.num_pages}; it could never finish"
                 )
         self.waiting.append(req)
@@ -143,6 +144,17 @@ class Scheduler:
     @property
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
+
+    def _most_pages_held(self, group: int, n_tokens: int) -> int:
+        """The pages of ``group`` that a request of ``n_tokens`` cannot do without.  A group that
+        keeps every key needs them all; a group with a window gives pages back as the window passes
+        them, and a portion can be cut down to one token, so what it must hold at once are the
+        pages that ``window`` keys touch (one more when they straddle a page's edge)."""
+        whole = self.cache.blocks_for(n_tokens, group)
+        window = self.cache.groups[group].window
+        if window <= 0:
+            return whole
+        return min(whole, self.cache.blocks_for(window, group) + 1)
 
     # ------------------------------------------------------------------ planning
     def _pages_for(self, req: Request, n_new: int) -> List[int]:
