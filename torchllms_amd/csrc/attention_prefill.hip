@@ -10,8 +10,13 @@
 //     there without passing through registers: `global_load_lds_dwordx4` puts a wave's 64 x 16 bytes
 //     at consecutive LDS addresses.  Rows are therefore not padded; instead the 16-byte pieces of a
 //     row are stored in an order that depends on the row (piece ^ f(row)), so that the 16 lanes that
-//     read the same piece of 16 rows still meet 16 different banks.  Two buffers per set of waves:
-//     the next tile lands while the current one is worked off, with one barrier a tile.
+//     read the same piece of 16 rows still meet 16 different banks.  Two buffers of keys and two of
+//     values per set of waves, one barrier a tile: a tile lands one pass before it is read.
+//   * within a wave the tiles run through a pipeline of three stages (scores of the next tile, softmax
+//     of this one, output product of the last), so matrix cores and vector units have independent work
+//     at the same time; sums of probabilities are one more MFMA row, a column's reference maximum
+//     moves only when a score passes it by a margin, and masks are applied only on tiles that hold a
+//     causal limit, a window's edge or the end of the keys.  Page sizes are powers of two.
 //   * scores are computed transposed, S^T[key][column] = K Q^T, by MFMA 16x16x32 bf16 (a lane's 16
 //     bytes of a key row are one operand); their output layout, taken over two blocks of 16 keys, is
 //     exactly the B-operand layout of P^T in O^T[channel][column] = V^T P^T, so the probabilities
