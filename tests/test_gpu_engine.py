@@ -115,8 +115,10 @@ def test_float32_does_not_depend_on_the_schedule(cases, name, schedule):
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_bfloat16_is_as_close_as_plain_bfloat16(cases, name, schedule):
     """The yardstick for bfloat16 is the plain model run in bfloat16: the engine's distance from
-    the 32-bit truth may not exceed twice the plain bfloat16 model's own, in the maximum and in
-    the mean."""
+    the 32-bit truth may not exceed twice the plain bfloat16 model's own, in the maximum, in the
+    mean, and position by position (there against the plain model's error at that very position,
+    or its mean over all positions where that is larger: a fault confined to one position, a page's
+    edge say, does not hide below the largest error found anywhere)."""
     case = cases[name]
     got = case.result("bfloat16", schedule)
     ref_max = max((case.plain16[r] - case.plain32[r]).abs().max().item() for r in case.requests)
@@ -125,6 +127,13 @@ def test_bfloat16_is_as_close_as_plain_bfloat16(cases, name, schedule):
     mean = torch.stack([(row - case.plain32[rid][pos]).abs().mean() for (rid, pos), row in got.items()]).mean().item()
     assert err <= 2 * ref_max, f"{name}/{schedule}: {where} max abs error {err} vs plain bfloat16 {ref_max}"
     assert mean <= 2 * ref_mean, f"{name}/{schedule}: mean abs error {mean} vs plain bfloat16 {ref_mean}"
+    floor = torch.cat([(case.plain16[r] - case.plain32[r]).abs().amax(dim=1) for r in case.requests]).mean().item()
+    for (rid, pos), row in got.items():
+        here = (row - case.plain32[rid][pos]).abs().max().item()
+        plain_here = (case.plain16[rid][pos] - case.plain32[rid][pos]).abs().max().item()
+        assert here <= 2 * max(plain_here, floor), (
+            f"{name}/{schedule}: {rid} position {pos}: error {here}, plain bfloat16 there {plain_here}, on average {floor}"
+        )
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])
