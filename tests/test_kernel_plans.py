@@ -85,3 +85,12 @@ def test_the_table_survives_a_file(tmp_path):
     finally:
         products.LINEAR_CHOICE.clear()
         products.LINEAR_CHOICE.update(saved)
+
+
+def test_libraries_built_in_the_tree_match_their_sources():
+    """A library built before its source was last edited is compiled again at its next use, on the GPU
+    box, where the time counts: build again after every change (``__graft_entry__.build()``).  A
+    tree without built libraries (a fresh checkout) has nothing to compare."""
+    from torchllms_amd.kernels import build
+
+    assert build.stale_libraries() == []

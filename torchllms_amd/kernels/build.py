@@ -198,6 +198,24 @@ register_variant("peaks", "peaks.hip", "TL_PEAKS")
 PREBUILT_VARIANTS: Dict[str, Iterable[int]] = {"attn_decode": (32, 64, 128, 256), "attn_prefill": (32, 64, 128, 256), "peaks": (1,)}
 
 
+def stale_libraries() -> List[str]:
+    """Names of libraries that were built earlier and whose sources or flags have changed since:
+    their next use compiles them again.  Libraries that were never built are not named."""
+    wanted = [(CORE_NAME, CORE_SOURCES, [])]
+    for kind, values in PREBUILT_VARIANTS.items():
+        v = VARIANTS[kind]
+        wanted += [(variant_name(kind, value), [v["source"]], [f"-D{v['macro']}={value}"]) for value in values]
+    stale = []
+    for lib_name, sources, defines in wanted:
+        have = _existing_library(lib_name)
+        if have is None:
+            continue
+        stamp = have.with_suffix(".stamp")
+        if not stamp.is_file() or stamp.read_text().strip() != _hash(sources, defines):
+            stale.append(lib_name)
+    return stale
+
+
 def build_all(force: bool = False) -> List[Path]:
     """Everything the tests, the smoke run and the benchmark load."""
     out = [build_core(force=force)]
