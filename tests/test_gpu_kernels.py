@@ -298,7 +298,7 @@ def test_add_bias(dtype):
 
 
 # ----------------------------------------------------------------------------- 32-bit matrix product
-@pytest.mark.parametrize("m, n, k", [(1, 100, 50), (7, 257, 1000), (130, 64, 64), (65, 129, 17)])
+@pytest.mark.parametrize("m, n, k", [(1, 100, 50), (7, 257, 1000), (130, 64, 64), (65, 129, 17), (300, 391, 70), (97, 130, 1029)])
 def test_gemm_f32_is_true_32_bit(m, n, k):
     torch.manual_seed(0)
     x, w = torch.randn(m, k), torch.randn(n, k)
@@ -327,6 +327,11 @@ def test_gemm_f32_with_few_rows_gives_the_bits_of_the_kernel_for_many(n, k):
         assert torch.equal(few, many[:rows]), f"{rows} rows differ from the tiled kernel"
     shifted = _ops().gemm_f32(x[5:8], w)
     assert torch.equal(shifted, many[5:8])
+    # prompts take a larger tile with more of the result per thread: the same sums again
+    torch.manual_seed(n + k + 1)
+    tall = torch.cat([x, torch.randn(131, k + 3, device=DEV)[:, :k]])
+    assert torch.equal(_ops().gemm_f32(tall, w)[:40], many)
+    assert torch.equal(_ops().gemm_f32(tall[37:], w)[:3], many[37:])
     if k % 4 == 0:
         aligned = _ops().gemm_f32(x[:2].contiguous(), w)
         assert torch.equal(aligned, many[:2])

@@ -3,23 +3,43 @@
 // ascending order (in groups of 16 that are added up first), so its value does not depend on M or on
 // where the row sits in the batch.
 // Throughput is secondary: this is the matrix product of the 32-bit path.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
 
-constexpr int BM = 64, BN = 64, BK = 16, TM = 4, TN = 4;
-constexpr int kThreads = (BM / TM) * (BN / TN);  // 256
+constexpr int BK = 16;  // products that are added among themselves before they join the running sum
 
-__global__ void __launch_bounds__(kThreads)
+// A block computes a BM x BN tile of C with (BM / TM) x (BN / TN) = 256 threads, each a TM x TN piece of it
+// (its rows and columns in runs of four, so that operands come from LDS sixteen bytes at a time).  Tiles of A
+// and W, BK wide, pass through LDS transposed (k-major); the next tiles travel from memory into registers
+// while the current ones are multiplied, and two sets of LDS tiles leave one barrier a step.
+// Two shapes: 64 x 64 with 4 x 4 a thread for steps of a few dozen rows, 128 x 128 with 8 x 8 a thread for
+// prompts (twice the arithmetic per byte read from LDS).  The arithmetic of an output element is the same in
+// both, and in the kernel for few rows below: the BK products of a step chained by fused multiply-adds from k
+// ascending, starting from zero, then added to the running sum.
+template <int BM, int BN, int TM, int TN>
+__global__ void __launch_bounds__((BM / TM) * (BN / TN))
 gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
                 float* __restrict__ C, int ldc, int M, int N, int K) {
-  __shared__ float As[BK][BM + 4];
-  __shared__ float Ws[BK][BN + 4];
+  constexpr int kThreads = (BM / TM) * (BN / TN);
+  static_assert(kThreads == 256 && TM % 4 == 0 && TN % 4 == 0, "256 threads, pieces in runs of four");
+  constexpr int kPerA = BM * BK / kThreads;  // elements of a tile that one thread moves: a run along k
+  constexpr int kPerW = BN * BK / kThreads;
+  static_assert(kPerA % 4 == 0 && kPerW % 4 == 0 && BK % kPerA == 0 && BK % kPerW == 0, "runs of whole float4s");
+  constexpr int kPitchA = BM + 4, kPitchW = BN + 4;
+  constexpr int kAhead = TM * TN >= 64 ? 2 : 4;  // steps of k whose operands are in registers together
+  __shared__ __attribute__((aligned(16))) float As[2][BK][kPitchA];
+  __shared__ __attribute__((aligned(16))) float Ws[2][BK][kPitchW];
   const int tid = threadIdx.x;
   const int tx = tid % (BN / TN);  // column group
   const int ty = tid / (BN / TN);  // row group
-  const int m0 = blockIdx.y * BM;
-  const int n0 = blockIdx.x * BN;
+  // consecutive blocks share their columns: the tile of W is read from memory once for all of them
+  const int m0 = blockIdx.x * BM;
+  const int n0 = blockIdx.y * BN;
+  // run r of the thread's rows is rows (BM / (TM / 4)) * r + 4 * ty ... + 3 of the tile; columns likewise
+  constexpr int kRowRun = BM / (TM / 4), kColRun = BN / (TN / 4);
 
   float acc[TM][TN];
 #pragma unroll
@@ -27,21 +47,46 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = 0.f;
 
-  for (int k0 = 0; k0 < K; k0 += BK) {
-    // each thread loads 4 elements of each tile: tile row = tid / 4, k offsets (tid % 4) * 4 .. +3
-    {
-      const int r = tid / 4;
-      const int kk = (tid % 4) * 4;
+  // what this thread moves: row (of A or of W) and the run of k within the step
+  const int ar = tid / (BK / kPerA), ak = (tid % (BK / kPerA)) * kPerA;
+  const int wr = tid / (BK / kPerW), wk = (tid % (BK / kPerW)) * kPerW;
+  const bool a_vec = (lda % 4) == 0 && ((uintptr_t)A % 16) == 0;
+  const bool w_vec = (ldw % 4) == 0 && ((uintptr_t)W % 16) == 0;
+  const float* a_row = A + (size_t)min(m0 + ar, M - 1) * lda;
+  const float* w_row = W + (size_t)min(n0 + wr, N - 1) * ldw;
+  const bool a_in = m0 + ar < M, w_in = n0 + wr < N;
+  float ra[kPerA], rw[kPerW];
+  auto fetch_run = [&](const float* row, bool inside, bool vec, int k, float* dst, auto per) {
+    constexpr int kPer = decltype(per)::value;
+    if (inside && vec && k + kPer <= K) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int k = k0 + kk + u;
-        const int m = m0 + r;
-        As[kk + u][r] = (m < M && k < K) ? A[(size_t)m * lda + k] : 0.f;
-        const int n = n0 + r;
-        Ws[kk + u][r] = (n < N && k < K) ? W[(size_t)n * ldw + k] : 0.f;
+      for (int u = 0; u < kPer; u += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(row + k + u);
+        dst[u] = v.x; dst[u + 1] = v.y; dst[u + 2] = v.z; dst[u + 3] = v.w;
       }
+    } else {
+#pragma unroll
+      for (int u = 0; u < kPer; ++u) dst[u] = (inside && k + u < K) ? row[k + u] : 0.f;
     }
-    __syncthreads();
+  };
+  auto fetch = [&](int k0) {
+    fetch_run(a_row, a_in, a_vec, k0 + ak, ra, std::integral_constant<int, kPerA>{});
+    fetch_run(w_row, w_in, w_vec, k0 + wk, rw, std::integral_constant<int, kPerW>{});
+  };
+  auto store = [&](int buffer) {
+#pragma unroll
+    for (int u = 0; u < kPerA; ++u) As[buffer][ak + u][ar] = ra[u];
+#pragma unroll
+    for (int u = 0; u < kPerW; ++u) Ws[buffer][wk + u][wr] = rw[u];
+  };
+
+  fetch(0);
+  store(0);
+  __syncthreads();
+  int buffer = 0;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    const bool more = k0 + BK < K;
+    if (more) fetch(k0 + BK);
     // the BK products of this step are added among themselves first and then to the running sum:
     // the rounding error of a long sum grows with the number of additions to one accumulator, and
     // this way there are K / BK + BK of them instead of K (at K = 1024 the 32-bit model's distance
@@ -51,13 +96,21 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j) part[i][j] = 0.f;
-#pragma unroll
+    // (unrolled by kAhead only: unrolled whole, the compiler asks for all sixteen steps' operands at once
+    // and the large tile takes 405 registers)
+#pragma unroll kAhead
     for (int k = 0; k < BK; ++k) {
       float a[TM], w[TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a[i] = As[k][ty * TM + i];
+      for (int r = 0; r < TM / 4; ++r) {
+        const float4 v = *reinterpret_cast<const float4*>(&As[buffer][k][kRowRun * r + 4 * ty]);
+        a[4 * r] = v.x; a[4 * r + 1] = v.y; a[4 * r + 2] = v.z; a[4 * r + 3] = v.w;
+      }
 #pragma unroll
-      for (int j = 0; j < TN; ++j) w[j] = Ws[k][tx * TN + j];
+      for (int r = 0; r < TN / 4; ++r) {
+        const float4 v = *reinterpret_cast<const float4*>(&Ws[buffer][k][kColRun * r + 4 * tx]);
+        w[4 * r] = v.x; w[4 * r + 1] = v.y; w[4 * r + 2] = v.z; w[4 * r + 3] = v.w;
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -67,15 +120,17 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j) acc[i][j] += part[i][j];
+    if (more) store(buffer ^ 1);
     __syncthreads();
+    buffer ^= 1;
   }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int m = m0 + ty * TM + i;
+    const int m = m0 + kRowRun * (i / 4) + 4 * ty + i % 4;
     if (m >= M) continue;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int n = n0 + tx * TN + j;
+      const int n = n0 + kColRun * (j / 4) + 4 * tx + j % 4;
       if (n < N) C[(size_t)m * ldc + n] = acc[i][j];
     }
   }
@@ -200,9 +255,15 @@ TL_EXPORT int tl_gemm_f32(const float* A, int lda, const float* W, int ldw, floa
 #undef TL_ROWS_LAUNCH
     return tl_check_launch("gemm_f32_rows");
   }
-  const unsigned gy = (M + BM - 1) / BM;
-  TL_REQUIRE(gy <= 65535, "gemm_f32: M=%d exceeds the grid limit of one launch", M);
-  dim3 grid((N + BN - 1) / BN, gy);
-  gemm_f32_kernel<<<grid, kThreads, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  // prompts take the large tile, if that still makes a block for every CU (both give the same sums)
+  if (M > 96 && (size_t)((M + 127) / 128) * ((N + 127) / 128) >= 256) {
+    const unsigned gy = (N + 127) / 128;
+    TL_REQUIRE(gy <= 65535, "gemm_f32: N=%d exceeds the grid limit of one launch", N);
+    gemm_f32_kernel<128, 128, 8, 8><<<dim3((M + 127) / 128, gy), 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  } else {
+    const unsigned gy = (N + 63) / 64;
+    TL_REQUIRE(gy <= 65535, "gemm_f32: N=%d exceeds the grid limit of one launch", N);
+    gemm_f32_kernel<64, 64, 4, 4><<<dim3((M + 63) / 64, gy), 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  }
   return tl_check_launch("gemm_f32");
 }
