@@ -85,3 +85,31 @@ def test_random_configuration(tmp_path, seed):
             else:
                 diff = [k for k in first if not torch.equal(first[k], got[k])]
                 assert not diff, f"{name}: {len(diff)} positions differ from whole, first {sorted(diff)[0]}"
+
+
+@pytest.mark.parametrize("head_dim, heads, kv_heads, hidden, page", [(10, 4, 2, 64, 16), (36, 3, 1, 100, 5), (66, 4, 2, 136, 7), (250, 2, 1, 128, 16), (2, 3, 3, 30, 3)])
+def test_head_sizes_that_are_no_multiple_of_16(tmp_path, head_dim, heads, kv_heads, hidden, page):
+    """The configuration allows any even head size and the engine any page size: sizes that the MFMA kernels
+    and the 16-byte loads do not fit (head sizes 2, 10, 36, 66, 250; pages of 3, 5 and 7 tokens) run through
+    the plain kernels, right in both dtypes, not refused and not wrong."""
+    from torchllms_amd.engine import Engine
+
+    cfg = {"architectures": ["LlamaForCausalLM"], "hidden_size": hidden, "num_hidden_layers": 2, "num_attention_heads": heads,
+           "num_key_value_heads": kv_heads, "head_dim": head_dim, "intermediate_size": 130, "vocab_size": 301,
+           "max_position_embeddings": 512, "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "tie_word_embeddings": False,
+           "attention_bias": True}
+    folder = make_folder(tmp_path / "m", cfg, seed=head_dim, dtype=torch.bfloat16, norm_jitter=0.1, sharpen=True)
+    cfg, weights = read_folder(folder)
+    requests = {f"r{i}": random_tokens(n, 301, 7 * head_dim + i) for i, n in enumerate([33, 70, 47, 129])}
+    plain32 = {rid: plain.forward(weights, cfg, t, torch.float32) for rid, t in requests.items()}
+    plain16 = {rid: plain.forward(weights, cfg, t, torch.bfloat16).float() for rid, t in requests.items()}
+    largest = max(v.abs().max().item() for v in plain32.values())
+    bf16_err = max((plain16[r] - plain32[r]).abs().max().item() for r in requests)
+    traces = {name: getattr(schedules, name)(requests) for name in ("whole", "mixed")}
+    pool = max(schedules.max_live_tokens(t) for t in traces.values())
+    for dtype in ("float32", "bfloat16"):
+        engine = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=-(-pool // page) + 4, max_seqs=4)
+        for name, trace in traces.items():
+            err, where = _max_err(run_trace(engine, trace), plain32)
+            bound = 2 * bf16_err if dtype == "bfloat16" else 5e-5 * max(1.0, largest)
+            assert err <= bound, f"{dtype}/{name}: {where} max abs error {err}, bound {bound}"
