@@ -146,7 +146,9 @@ def build_library(lib_name: str, sources: Sequence[str], defines: Sequence[str] 
         objs = []
 
         def compile_one(src: str) -> Path:
-            obj = out_dir / f"{lib_name}.{Path(src).stem}.o"
+            # the process id keeps two processes that build the same library at once (two first calls from
+            # one checkout) out of each other's files; the library itself is moved into place whole
+            obj = out_dir / f"{lib_name}.{Path(src).stem}.{os.getpid()}.o"
             _run([hipcc, *HIPCC_FLAGS, *defines, "-I", str(CSRC), "-c", str(CSRC / src), "-o", str(obj)], f"compile {src}")
             return obj
 
