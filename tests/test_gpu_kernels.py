@@ -404,6 +404,53 @@ def test_attention_generic(dtype, hq, hkv, dh, page, S, sq):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize(
+    "hq, hkv, dh, page, sizes, window",
+    [(8, 2, 128, 16, [(300, 200), (70, 70), (40, 3)], 0), (6, 3, 48, 4, [(150, 90), (33, 33)], 0), (4, 4, 64, 8, [(260, 100), (90, 40)], 37),
+     (3, 1, 20, 5, [(100, 64), (50, 50)], 0), (16, 2, 256, 16, [(130, 50)], 100), (5, 5, 18, 3, [(80, 41)], 0)],
+)
+def test_attention_generic_for_prompt_portions_gives_the_bits_of_one_token_at_a_time(dtype, hq, hkv, dh, page, sizes, window):
+    """Steps with many tokens bring each block of 64 keys into LDS once for sixteen (token, head) pairs that
+    read it; the arithmetic per pair is the walk of a single wave, so the results are the same bits as when every
+    token is a step of its own (which takes the kernel that shares nothing).  Requests of different lengths in
+    one launch (blocks that straddle two requests walk alone), groups of 1, 2, 4 and 8 query heads per kv head,
+    head sizes that are no multiple of 4, a window, right against the plain attention."""
+    torch.manual_seed(dh + page)
+    k_all, v_all, q_all, seqs, poss, tables = [], [], [], [], [], []
+    n_pages = sum(-(-S // page) for S, _ in sizes) + 2
+    perm = torch.randperm(n_pages).tolist()
+    k_pages = torch.zeros(n_pages, hkv, page, dh, dtype=dtype)
+    v_pages = torch.zeros_like(k_pages)
+    width = max(-(-S // page) for S, _ in sizes)
+    want = []
+    for r, (S, sq) in enumerate(sizes):
+        q = torch.randn(sq, hq, dh) * 2
+        k, v = torch.randn(S, hkv, dh), torch.randn(S, hkv, dh)
+        if dtype == torch.bfloat16:
+            q, k, v = q.bfloat16().float(), k.bfloat16().float(), v.bfloat16().float()
+        table = [perm.pop() for _ in range(-(-S // page))]
+        for p_ in range(S):
+            k_pages[table[p_ // page], :, p_ % page] = k[p_].to(dtype)
+            v_pages[table[p_ // page], :, p_ % page] = v[p_].to(dtype)
+        tables.append(table + [-1] * (width - len(table)))
+        q_all.append(q.reshape(sq, hq * dh))
+        seqs += [r] * sq
+        poss += list(range(S - sq, S))
+        want.append(_windowed_plain(q, k, v, window))
+    qkv = torch.cat(q_all).to(dtype).to(DEV).contiguous()
+    k_pages, v_pages = k_pages.to(DEV), v_pages.to(DEV)
+    bt = _i32(tables)
+    fn = _ops().attention_generic
+    together = fn(qkv, hq, hkv, dh, k_pages, v_pages, _i32(seqs), _i32(poss), bt, window, dh ** -0.5)
+    assert len(seqs) >= 32
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=2 ** -7, atol=2 ** -7)
+    torch.testing.assert_close(together.float().cpu(), torch.cat(want).reshape(len(seqs), hq * dh), **tol)
+    for i in list(range(0, len(seqs), 7)) + [len(seqs) - 1]:
+        alone = fn(qkv[i : i + 1], hq, hkv, dh, k_pages, v_pages, _i32(seqs[i : i + 1]), _i32(poss[i : i + 1]), bt, window, dh ** -0.5)
+        assert torch.equal(alone[0], together[i]), f"token {i} differs from the same token alone"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize(
     "hq, hkv, dh, page, S, sq, window",
     [(4, 2, 16, 8, 37, 3, 0), (6, 3, 48, 4, 150, 9, 0), (8, 1, 128, 16, 700, 2, 0), (3, 3, 6, 32, 270, 5, 0), (2, 1, 256, 16, 65, 2, 0),
      (4, 4, 64, 1, 200, 4, 70), (5, 5, 32, 16, 1000, 3, 64), (2, 2, 80, 8, 129, 1, 0)],

@@ -4,6 +4,8 @@
 // absolute position, so a result depends only on the query's position and the cache contents,
 // never on how the step was batched.  This is the kernel of the 32-bit path and the fallback of
 // the bfloat16 path for sizes the MFMA kernels refuse.
+#include <limits.h>
+
 #include "common.h"
 
 namespace {
@@ -11,6 +13,7 @@ namespace {
 constexpr int kWavesPerBlock = 4;
 constexpr int kMaxHeadDim = 256;
 constexpr int kChanPerLane = kMaxHeadDim / kWave;
+constexpr int kTileMinTokens = 32;  // steps with at least this many tokens share keys and values through LDS
 
 // Four consecutive elements of a row as floats (the row is 16-byte aligned for float, 8-byte for bfloat16).
 __device__ __forceinline__ void load4(const float* p, float (&v)[4]) {
@@ -170,6 +173,171 @@ attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
   }
 }
 
+// The same result for prompt portions, with the keys and values shared: a block of 16 waves takes
+// kTileWaves / HB consecutive tokens and HB query heads that read the same kv head, and every block of 64
+// keys is brought into LDS once for all of them (as 32-bit floats, rows padded so that 64 lanes that read
+// 64 different rows meet different banks).  Each wave then computes its block exactly as block_partial
+// does, operation for operation, from LDS instead of from the pages, and lets it join its running result:
+// the same bits as one wave walking alone, at a sixteenth of the traffic.  Tokens of different requests
+// (a block that straddles two rows of the step) have different keys: such a block walks alone as above.
+constexpr int kTileWaves = 16;
+constexpr int kTilePad = 4;  // floats between LDS rows beyond head_dim: rows start four banks apart
+
+template <bool VEC, int CH>
+__device__ __forceinline__ void block_partial_lds(const float* qs, const float* k_t, const float* v_t, int pitch,
+                                                  int head_dim, int lo, int p, float scale, int j0, int lane,
+                                                  float& m_b, float& l_b, float (&o_b)[kChanPerLane]) {
+#pragma clang fp contract(off)
+  const int j = j0 + lane;
+  const bool valid = j >= lo && j <= p;
+  float s = -INFINITY;
+  if (valid) {
+    const float* kr = k_t + lane * pitch;
+    float dot = 0.f;
+    if (VEC) {
+      for (int d = 0; d < head_dim; d += 4) {
+        float kv[4];
+        load4(kr + d, kv);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) dot = fmaf(qs[d + u], kv[u], dot);
+      }
+    } else {
+      for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], kr[d], dot);
+    }
+    s = dot * scale;
+  }
+  m_b = wave_max(s);
+  const float pj = valid ? expf(s - m_b) : 0.f;
+  l_b = wave_sum(pj);
+#pragma unroll
+  for (int c = 0; c < kChanPerLane; ++c) o_b[c] = 0.f;
+  const int jj_lo = lo > j0 ? lo - j0 : 0;
+  const int jj_hi = p - j0 < kWave - 1 ? p - j0 : kWave - 1;
+  // jj is the same in every lane: the probability of key jj comes out of its lane as a scalar.  Only the
+  // CH channel slots that the head size fills are touched (the others stay zero, as in the walk alone, where
+  // they add zeros).
+  auto value = [&](int jj, int c) {
+    const int d = lane + c * kWave;
+    return (c + 1 < CH || d < head_dim) ? v_t[jj * pitch + d] : 0.f;
+  };
+  constexpr int U = 4;  // value rows asked for together; they are still added one after the other
+  int jj = jj_lo;
+  for (; jj + U - 1 <= jj_hi; jj += U) {
+    float pw[U], vv[U][CH];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      pw[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pj), jj + u));
+#pragma unroll
+      for (int c = 0; c < CH; ++c) vv[u][c] = value(jj + u, c);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int c = 0; c < CH; ++c) o_b[c] = fmaf(pw[u], vv[u][c], o_b[c]);
+  }
+  for (; jj <= jj_hi; ++jj) {
+    const float pw = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pj), jj));
+#pragma unroll
+    for (int c = 0; c < CH; ++c) o_b[c] = fmaf(pw, value(jj, c), o_b[c]);
+  }
+}
+
+template <typename T, bool VEC, int CH>
+__global__ void __launch_bounds__(kTileWaves* kWave)
+attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
+                      const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+                      const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
+                      const int32_t* __restrict__ block_table, int bt_stride, int n_tokens, int n_q_heads,
+                      int n_kv_heads, int head_dim, int page_size, int window, float scale, int heads_per_block) {
+  extern __shared__ __attribute__((aligned(16))) float tile_lds[];
+  const int pitch = head_dim + kTilePad;
+  float* q_lds = tile_lds;                          // [kTileWaves][head_dim]
+  float* k_t = tile_lds + kTileWaves * head_dim;    // [64][pitch]
+  float* v_t = k_t + kWave * pitch;                 // [64][pitch]
+  const int HB = heads_per_block;
+  const int QT = kTileWaves / HB;
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  const int t0 = blockIdx.x * QT;
+  const int t_raw = t0 + wave / HB;
+  const int h_raw = blockIdx.y * HB + wave % HB;
+  const bool active = t_raw < n_tokens && h_raw < n_q_heads;
+  const int t = t_raw < n_tokens ? t_raw : n_tokens - 1;  // idle waves shadow a real token, store nothing
+  const int h = h_raw < n_q_heads ? h_raw : n_q_heads - 1;
+  const T* qv = q + (size_t)t * q_stride + (size_t)h * head_dim;
+  for (int d = lane; d < head_dim; d += kWave) q_lds[wave * head_dim + d] = to_f32(qv[d]);
+  const Query<T> a = make_query<T>(q_lds + wave * head_dim, k_pages, v_pages, token_seq, positions, block_table,
+                                   bt_stride, t, h, n_q_heads, n_kv_heads, head_dim, page_size, window, scale);
+  // what the whole block sees: the same for every thread, from the tokens' own entries
+  const int last = min(t0 + QT, n_tokens) - 1;
+  const int seq0 = token_seq[t0];
+  bool together = true;
+  int blk_lo = INT_MAX, blk_hi = -1, key_lo = INT_MAX;
+  for (int i = t0; i <= last; ++i) {
+    together = together && token_seq[i] == seq0;
+    const int pi = positions[i];
+    const int li = (window > 0 && pi - window + 1 > 0) ? pi - window + 1 : 0;
+    blk_lo = min(blk_lo, li - li % kWave);
+    key_lo = min(key_lo, li);
+    blk_hi = max(blk_hi, pi);
+  }
+  __syncthreads();  // the queries are in LDS
+  // the wave's own bounds, as scalars (they are the same in all its lanes)
+  const int lo_u = __builtin_amdgcn_readfirstlane(a.lo), p_u = __builtin_amdgcn_readfirstlane(a.p);
+  float acc[kChanPerLane];
+#pragma unroll
+  for (int c = 0; c < kChanPerLane; ++c) acc[c] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  if (!together) {
+    for (int j0 = a.lo - a.lo % kWave; j0 <= a.p; j0 += kWave) {
+      float m_b, l_b, o_b[kChanPerLane];
+      block_partial<T, VEC>(a, j0, lane, m_b, l_b, o_b);
+      merge_block(m, l, acc, m_b, l_b, o_b);
+    }
+  } else {
+    const int g = (blockIdx.y * HB) / (n_q_heads / n_kv_heads);  // the kv head of all the block's heads
+    const int32_t* bt = block_table + (size_t)seq0 * bt_stride;
+    const size_t head_elems = (size_t)page_size * head_dim;
+    const int per_row = VEC ? head_dim / 4 : head_dim;  // pieces of a row: four elements, or one
+    for (int j0 = blk_lo; j0 <= blk_hi; j0 += kWave) {
+      if (j0 > blk_lo) __syncthreads();  // everybody has finished with the tiles of the block before
+      for (int idx = threadIdx.x; idx < kWave * per_row; idx += kTileWaves * kWave) {
+        const int r = idx / per_row, piece = idx % per_row;
+        const int j = j0 + r;
+        if (j < key_lo || j > blk_hi) continue;  // nobody in the block sees this key
+        const int page = bt[j / page_size];
+        if (page < 0) continue;  // a page that a window gave back: no token of the step sees its keys
+        const size_t row_at = ((size_t)page * n_kv_heads + g) * head_elems + (size_t)(j % page_size) * head_dim;
+        if (VEC) {
+          float kv[4], vv[4];
+          load4(k_pages + row_at + 4 * piece, kv);
+          load4(v_pages + row_at + 4 * piece, vv);
+          *reinterpret_cast<float4*>(k_t + r * pitch + 4 * piece) = float4{kv[0], kv[1], kv[2], kv[3]};
+          *reinterpret_cast<float4*>(v_t + r * pitch + 4 * piece) = float4{vv[0], vv[1], vv[2], vv[3]};
+        } else {
+          k_t[r * pitch + piece] = to_f32(k_pages[row_at + piece]);
+          v_t[r * pitch + piece] = to_f32(v_pages[row_at + piece]);
+        }
+      }
+      __syncthreads();
+      if (j0 >= lo_u - lo_u % kWave && j0 <= p_u) {  // (uniform per wave)
+        float m_b, l_b, o_b[kChanPerLane];
+        block_partial_lds<VEC, CH>(a.qs, k_t, v_t, pitch, head_dim, lo_u, p_u, scale, j0, lane, m_b, l_b, o_b);
+        merge_block(m, l, acc, m_b, l_b, o_b);
+      }
+    }
+  }
+  if (active) {
+    T* o = out + (size_t)t * out_stride + (size_t)h * head_dim;
+    const float inv_l = 1.0f / l;
+#pragma unroll
+    for (int c = 0; c < kChanPerLane; ++c) {
+      const int d = lane + c * kWave;
+      if (d < head_dim) o[d] = from_f32<T>(acc[c] * inv_l);
+    }
+  }
+}
+
 // The same result from many waves, for steps with few tokens and long contexts (decode): wave
 // (token, head, r) computes block r of the token's key range alone and leaves it in `partials`
 // ([token][head][r][head_dim + 2]: the sums, then maximum and sum of probabilities); a second kernel
@@ -279,6 +447,44 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
   dim3 grid(n_tokens, (n_q_heads + kWavesPerBlock - 1) / kWavesPerBlock);
   // rows of the pages start at multiples of head_dim elements from an allocation's start
   const bool vec = head_dim % 4 == 0 && ((uintptr_t)k_pages % 16) == 0;
+  // prompt portions: tokens and heads that read the same keys share them through LDS (same bits)
+  if (n_tokens >= kTileMinTokens) {
+    const int group = n_q_heads / n_kv_heads;
+    const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+    const int qt = kTileWaves / hb;
+    const size_t lds = ((size_t)kTileWaves * head_dim + 2 * (size_t)kWave * (head_dim + kTilePad)) * sizeof(float);
+    dim3 tgrid((n_tokens + qt - 1) / qt, (n_q_heads + hb - 1) / hb);
+#define TL_TILE_LAUNCH_CH(T, VEC, CH)                                                                            \
+  do {                                                                                                           \
+    if (lds > 48 * 1024) {                                                                                       \
+      hipError_t e = hipFuncSetAttribute((const void*)attention_tile_kernel<T, VEC, CH>,                         \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                  \
+      if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "attention: %s", hipGetErrorString(e));                    \
+    }                                                                                                            \
+    attention_tile_kernel<T, VEC, CH><<<tgrid, kTileWaves * kWave, lds, stream>>>(                               \
+        (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions,  \
+        block_table, bt_stride, n_tokens, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, hb);        \
+  } while (0)
+#define TL_TILE_LAUNCH(T, VEC)                                                                                   \
+  do {                                                                                                           \
+    if (head_dim <= 64) TL_TILE_LAUNCH_CH(T, VEC, 1);                                                            \
+    else if (head_dim <= 128) TL_TILE_LAUNCH_CH(T, VEC, 2);                                                      \
+    else if (head_dim <= 192) TL_TILE_LAUNCH_CH(T, VEC, 3);                                                      \
+    else TL_TILE_LAUNCH_CH(T, VEC, 4);                                                                           \
+  } while (0)
+    if (dtype == TL_F32) {
+      if (vec) TL_TILE_LAUNCH(float, true);
+      else TL_TILE_LAUNCH(float, false);
+    } else if (dtype == TL_BF16) {
+      if (vec) TL_TILE_LAUNCH(bf16_t, true);
+      else TL_TILE_LAUNCH(bf16_t, false);
+    } else {
+      return tl_fail(TL_ERR_ARG, "attention: unknown dtype %d", dtype);
+    }
+#undef TL_TILE_LAUNCH_CH
+#undef TL_TILE_LAUNCH
+    return tl_check_launch("attention_tile");
+  }
 #define TL_ATTN_LAUNCH(T, VEC)                                                                              \
   attention_generic_kernel<T, VEC><<<grid, kWavesPerBlock * kWave, 0, stream>>>(                            \
       (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions, \
