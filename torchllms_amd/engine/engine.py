@@ -19,7 +19,7 @@ from ..cache.manager import CacheManager, OutOfPages, group_layers
 from ..config.registry import ArchSpec, get_architecture, load_config
 from ..parts.model import Model
 from ..weights.loader import load_weights
-from ..weights.random_init import random_tensors
+from ..weights.random_init import random_tensor, random_tensors
 from .context import upload
 from .layout import StepEntry, StepLayout, build_step_layout
 
@@ -180,9 +180,16 @@ class Engine:
         if draw_on_device:
             tensors = random_tensors(expected, seed, dtype, norm_jitter, device=device)
         else:
-            tensors = {}
-            for name, t in random_tensors(expected, seed, torch.float32, norm_jitter).items():
-                tensors[name] = t.to(dtype).to(device)
+            # one tensor at a time (a few at once, each with a generator of its own), so that the host never
+            # holds more than a few tensors of the model in 32-bit
+            from concurrent.futures import ThreadPoolExecutor
+
+            def draw(item):
+                name, spec = item
+                return name, random_tensor(name, spec, seed, torch.float32, norm_jitter).to(dtype).to(device)
+
+            with ThreadPoolExecutor(max_workers=4) as pool:
+                tensors = dict(pool.map(draw, expected.items()))
         return cls(arch, config, tensors, dtype, device=device, **kw)
 
     # ------------------------------------------------------------------ requests
