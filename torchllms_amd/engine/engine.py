@@ -164,7 +164,16 @@ class Engine:
         expected = model.param_specs()
         ignore = model.ignorable_tensors()
         tensors = load_weights(folder, arch.weight_rules(config), expected, dtype, device=device, ignore_when_present=ignore)
-        return cls(arch, config, tensors, dtype, device=device, **kw)
+        return cls._from_tensors(arch, config, tensors, dtype, device, kw)
+
+    @classmethod
+    def _from_tensors(cls, arch, config, tensors, dtype, device, kw) -> "Engine":
+        engine = cls(arch, config, tensors, dtype, device=device, **kw)
+        # parts that fuse matrices (q|k|v, gate|up) hold copies; the separate ones go with this dictionary,
+        # and their memory goes back to the device instead of staying in torch's cache
+        tensors.clear()
+        torch.cuda.empty_cache()
+        return engine
 
     @classmethod
     def from_random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", norm_jitter: float = 0.0,
@@ -190,7 +199,7 @@ class Engine:
 
             with ThreadPoolExecutor(max_workers=4) as pool:
                 tensors = dict(pool.map(draw, expected.items()))
-        return cls(arch, config, tensors, dtype, device=device, **kw)
+        return cls._from_tensors(arch, config, tensors, dtype, device, kw)
 
     # ------------------------------------------------------------------ requests
     def admit(self, rid: Hashable) -> int:
