@@ -88,19 +88,45 @@ def _cut(rid, tokens, sizes, tail):
     return steps
 
 
+# the other shape that is benchmarked: hidden 2048, head size 64, tied head, rope factor 32 (Llama-3.2-1B)
+ONE_LAYER_SMALL = dict(
+    REAL, num_hidden_layers=1, hidden_size=2048, head_dim=64, intermediate_size=8192, tie_word_embeddings=True,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+)
+
+
+@pytest.fixture(scope="module")
+def one_layer_small(tmp_path_factory):
+    folder = make_folder(tmp_path_factory.mktemp("small") / "m", ONE_LAYER_SMALL, seed=6, dtype=torch.bfloat16, norm_jitter=0.1, sharpen=True)
+    cfg, weights = read_folder(folder)
+    return folder, cfg, weights
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_at_head_size_64(one_layer_small, dtype):
+    """The same at the 1B shape's sizes: the MFMA attention kernels of head size 64 behind long prefixes, a
+    tied head, another rope factor."""
+    _long_prompt(one_layer_small, dtype, head_dim=64)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_long_prompt_whole_and_in_portions_behind_a_long_prefix(one_layer, dtype):
     """4,700 tokens in one step (1,176 blocks of the prefill attention kernel: beyond the 1,024 up
     to which blocks hold two sets of waves), then the same request as 2,100 tokens, portions of 700,
     2, 1,000, 31 and 827 behind them, and the last 40 tokens one by one."""
+    _long_prompt(one_layer, dtype, head_dim=128)
+
+
+def _long_prompt(model, dtype, head_dim):
     from torchllms_amd.engine import Engine
     from torchllms_amd.kernels import ops
 
-    folder, cfg, weights = one_layer
+    folder, cfg, weights = model
     n = 4700
     tokens = random_tokens(n, ONE_LAYER["vocab_size"], 77)
     want = plain.forward(weights, cfg, tokens, torch.float32)
-    qpt = ops.prefill_queries_per_tile(32, 8, 128)
+    qpt = ops.prefill_queries_per_tile(32, 8, head_dim)
     assert -(-n // qpt) * 8 > ops.PREFILL_SPLIT_BLOCKS  # the whole prompt is a launch with one set of waves
     eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=-(-n // 16) + 1, max_seqs=2, max_model_len=8192)
     whole = run_trace(eng, _cut("w", tokens, [n], 0))
