@@ -110,6 +110,23 @@ def test_a_long_prompt_at_head_size_64(one_layer_small, dtype):
     _long_prompt(one_layer_small, dtype, head_dim=64)
 
 
+# head size 256, four query heads per kv head: the attention kernels' other tile sizes
+ONE_LAYER_WIDE_HEADS = dict(REAL, num_hidden_layers=1, hidden_size=2048, num_attention_heads=8, num_key_value_heads=2, head_dim=256,
+                            intermediate_size=4096)
+
+
+@pytest.fixture(scope="module")
+def one_layer_wide_heads(tmp_path_factory):
+    folder = make_folder(tmp_path_factory.mktemp("wide") / "m", ONE_LAYER_WIDE_HEADS, seed=7, dtype=torch.bfloat16, norm_jitter=0.1, sharpen=True)
+    cfg, weights = read_folder(folder)
+    return folder, cfg, weights
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_at_head_size_256(one_layer_wide_heads, dtype):
+    _long_prompt(one_layer_wide_heads, dtype, head_dim=256, heads=8, kv_heads=2, one_set_of_waves=False)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_long_prompt_whole_and_in_portions_behind_a_long_prefix(one_layer, dtype):
     """4,700 tokens in one step (1,176 blocks of the prefill attention kernel: beyond the 1,024 up
@@ -118,7 +135,7 @@ def test_a_long_prompt_whole_and_in_portions_behind_a_long_prefix(one_layer, dty
     _long_prompt(one_layer, dtype, head_dim=128)
 
 
-def _long_prompt(model, dtype, head_dim):
+def _long_prompt(model, dtype, head_dim, heads=32, kv_heads=8, one_set_of_waves=True):
     from torchllms_amd.engine import Engine
     from torchllms_amd.kernels import ops
 
@@ -126,8 +143,9 @@ def _long_prompt(model, dtype, head_dim):
     n = 4700
     tokens = random_tokens(n, ONE_LAYER["vocab_size"], 77)
     want = plain.forward(weights, cfg, tokens, torch.float32)
-    qpt = ops.prefill_queries_per_tile(32, 8, head_dim)
-    assert -(-n // qpt) * 8 > ops.PREFILL_SPLIT_BLOCKS  # the whole prompt is a launch with one set of waves
+    qpt = ops.prefill_queries_per_tile(heads, kv_heads, head_dim)
+    # the whole prompt is a launch with one set of waves a block, or with two
+    assert (-(-n // qpt) * kv_heads > ops.PREFILL_SPLIT_BLOCKS) == one_set_of_waves
     eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=-(-n // 16) + 1, max_seqs=2, max_model_len=8192)
     whole = run_trace(eng, _cut("w", tokens, [n], 0))
     parts = run_trace(eng, _cut("p", tokens, [2100, 700, 2, 1000, 31, 827], 40))
