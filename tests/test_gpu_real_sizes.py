@@ -216,9 +216,28 @@ def test_many_live_requests_of_unequal_lengths_decode_together(one_layer, many, 
     """24 and 64 live requests of 10 to 1,900 tokens: prompts prefilled eight to a step, then the
     last 20 tokens of every request decoded together, 24 or 64 rows a step, replayed from graphs
     whose key says that the lengths differ much (shorter key splits in the decode attention)."""
+    _many_live(one_layer, many, dtype, live)
+
+
+@pytest.fixture(scope="module")
+def many_small(one_layer_small):
+    folder, cfg, weights = one_layer_small
+    requests = {f"m{i}": random_tokens(n, ONE_LAYER["vocab_size"], 300 + i) for i, n in enumerate(MANY_LENGTHS)}
+    truth = {rid: plain.forward(weights, cfg, t, torch.float32) for rid, t in requests.items()}
+    return requests, truth
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_many_live_requests_at_head_size_64(one_layer_small, many_small, dtype):
+    """The same with 64 live requests at the 1B shape's sizes: the decode attention of head size 64 and the
+    decode products of a hidden size of 2,048, replayed from graphs."""
+    _many_live(one_layer_small, many_small, dtype, 64)
+
+
+def _many_live(model, many, dtype, live):
     from torchllms_amd.engine import Engine
 
-    folder, cfg, weights = one_layer
+    folder, cfg, weights = model
     all_requests, truth = many
     requests = dict(list(all_requests.items())[:live])
     tail = 20
