@@ -23,6 +23,11 @@ REAL = dict(
 LENGTHS = [150, 70, 333, 40]
 
 
+def _bf16_tolerance(weights, cfg, tokens, want):
+    yard = plain.forward(weights, cfg, tokens, torch.bfloat16, device="cuda:0").float().cpu()
+    return 2 * (yard - want).abs().amax(dim=-1) + 1e-3  # per position
+
+
 @pytest.fixture(scope="module")
 def real(tmp_path_factory):
     folder = make_folder(tmp_path_factory.mktemp("real") / "m", REAL, seed=3, dtype=torch.bfloat16, norm_jitter=0.1, sharpen=True)
@@ -57,17 +62,44 @@ def test_real_layer_sizes_match_the_plain_model_under_every_schedule(real, dtype
                 assert torch.equal(row, results["whole"][key]), f"{name} differs from whole at {key}"
 
 
+# the largest shape that is benchmarked: hidden 8192, 64 heads in 8 groups of 8, feed-forward 28672 (Llama-3.1-70B), one layer
+LARGE = dict(REAL, num_hidden_layers=1, hidden_size=8192, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+             intermediate_size=28672)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_largest_layer_sizes_match_the_plain_model(tmp_path_factory, dtype):
+    """Eight query heads per kv head, rows of 8,192 in the norms (the widest the norm that adds split sums
+    takes), matrices of 8,192 x 28,672: whole requests and the mixed schedule, with pages used again."""
+    from torchllms_amd.engine import Engine
+
+    folder = make_folder(tmp_path_factory.mktemp("large") / "m", LARGE, seed=9, dtype=torch.bfloat16, norm_jitter=0.1, sharpen=True)
+    cfg, weights = read_folder(folder)
+    requests = {f"r{i}": random_tokens(n, LARGE["vocab_size"], 60 + i) for i, n in enumerate([150, 70, 333, 40])}
+    truth = {rid: plain.forward(weights, cfg, t, torch.float32) for rid, t in requests.items()}
+    traces = {"whole": schedules.whole(requests), "mixed": schedules.mixed(requests)}
+    pool_tokens = max(schedules.max_live_tokens(t) for t in traces.values())
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=-(-pool_tokens // 16), max_seqs=4)
+    results = {name: run_trace(eng, trace) for name, trace in traces.items()}
+    tols = {rid: _bf16_tolerance(weights, cfg, t, truth[rid]) for rid, t in requests.items()} if dtype == "bfloat16" else None
+    for name, res in results.items():
+        for (rid, pos), row in res.items():
+            err = (row - truth[rid][pos]).abs().max().item()
+            if dtype == "float32":
+                assert err < 10 * FP32_ATOL, f"{name}: {rid} position {pos}: {err}"
+            else:
+                assert err <= tols[rid][pos].item(), f"{name}: {rid} position {pos}: {err} against {tols[rid][pos].item()}"
+    if dtype == "float32":
+        for key, row in results["mixed"].items():
+            assert torch.equal(row, results["whole"][key]), f"mixed differs from whole at {key}"
+
+
 # ----------------------------------------------------------------------------- the sizes that are benchmarked
 # One layer of the same sizes: long prompts (a prefill launch of more than 1,024 blocks, portions behind a
 # long prefix), decode steps replayed from graphs across context caps, and many live requests of very
 # unequal lengths.  The 32-bit truth is the plain model on the CPU; the bfloat16 yardstick is the plain
 # model in bfloat16, whose tensor operations torch runs on the GPU here (on the CPU they take minutes).
 ONE_LAYER = dict(REAL, num_hidden_layers=1)
-
-
-def _bf16_tolerance(weights, cfg, tokens, want):
-    yard = plain.forward(weights, cfg, tokens, torch.bfloat16, device="cuda:0").float().cpu()
-    return 2 * (yard - want).abs().amax(dim=-1) + 1e-3  # per position
 
 
 @pytest.fixture(scope="module")
