@@ -156,7 +156,7 @@ def one_layer_wide_heads(tmp_path_factory):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_long_prompt_at_head_size_256(one_layer_wide_heads, dtype):
-    _long_prompt(one_layer_wide_heads, dtype, head_dim=256, heads=8, kv_heads=2, one_set_of_waves=False)
+    _long_prompt(one_layer_wide_heads, dtype, head_dim=256, heads=8, kv_heads=2)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -177,7 +177,7 @@ def _long_prompt(model, dtype, head_dim, heads=32, kv_heads=8, one_set_of_waves=
     want = plain.forward(weights, cfg, tokens, torch.float32)
     qpt = ops.prefill_queries_per_tile(heads, kv_heads, head_dim)
     # the whole prompt is a launch with one set of waves a block, or with two
-    assert (-(-n // qpt) * kv_heads > ops.PREFILL_SPLIT_BLOCKS) == one_set_of_waves
+    assert (ops.prefill_key_groups(-(-n // qpt), kv_heads, n) == 1) == one_set_of_waves
     eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=-(-n // 16) + 1, max_seqs=2, max_model_len=8192)
     whole = run_trace(eng, _cut("w", tokens, [n], 0))
     parts = run_trace(eng, _cut("p", tokens, [2100, 700, 2, 1000, 31, 827], 40))

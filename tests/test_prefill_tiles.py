@@ -63,7 +63,9 @@ def test_a_long_launch_starts_its_longest_tiles_first():
 def test_two_sets_of_waves_for_launches_that_fit_at_once_and_then_longest_first():
     qo, kv, qpt, heads = [0, 2048], [2048], 32, 8
     n = prefill_tile_count(qo, 0, 1, qpt)
-    assert n * heads <= PREFILL_SPLIT_BLOCKS and prefill_key_groups(n, heads) == 2
+    assert n * heads <= PREFILL_SPLIT_BLOCKS and prefill_key_groups(n, heads, 2048) == 2
+    assert prefill_key_groups(n, heads, 2048 + 4096) == 1  # behind a long prefix two blocks a CU do better
+    assert prefill_key_groups(n // 2, heads, 2048 + 8192) == 2  # too few blocks to give every CU two
     rows, q0s = prefill_tiles(qo, 0, 1, qpt, kv, 0, heads, key_groups=2)
     costs = [_cost(r, q, qo, kv, qpt, 0) for r, q in zip(rows, q0s)]
     assert costs == sorted(costs, reverse=True)

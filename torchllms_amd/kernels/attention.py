@@ -70,7 +70,10 @@ def paged_attention(
             tiles = ctx.scratch.get(key)
             if tiles is None:
                 host = ctx.host
-                key_groups = ops.prefill_key_groups(ops.prefill_tile_count(host.qo_indptr, n_dec, host.n_seqs, qpt), n_kv_heads)
+                longest = int(max(host.kv_lens[n_dec : host.n_seqs]))
+                if window > 0:
+                    longest = min(longest, window + qpt)
+                key_groups = ops.prefill_key_groups(ops.prefill_tile_count(host.qo_indptr, n_dec, host.n_seqs, qpt), n_kv_heads, longest)
                 rows, q0s = ops.prefill_tiles(host.qo_indptr, n_dec, host.n_seqs, qpt, host.kv_lens, window, n_kv_heads, key_groups)
                 both = torch.tensor([rows, q0s], dtype=torch.int32).to(qkv.device)
                 tiles = (both[0], both[1], key_groups)

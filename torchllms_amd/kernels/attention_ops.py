@@ -258,18 +258,30 @@ def prefill_queries_per_tile(n_q_heads: int, n_kv_heads: int, head_dim: int) -> 
 
 #: blocks of the prefill kernel that the GPU holds at once: 256 CUs, two blocks each
 PREFILL_RESIDENT_BLOCKS = 512
-#: launches of up to this many blocks run with two sets of waves per block (measured at head size
-#: 128 with cold caches: 512 blocks 87 -> 72 us, 1,024 blocks 270 -> 257 us, 1,280 blocks 361 -> 391 us;
-#: at head size 64 the two are even at 768 and 1,024 blocks and one set wins from 1,280 on)
-PREFILL_SPLIT_BLOCKS = 1024
+#: launches of up to this many blocks run with two sets of waves per block, whatever their keys: one block of
+#: one set a CU leaves half of every CU idle
+PREFILL_SPLIT_ALWAYS = 256
+#: launches of up to this many blocks run with two sets of waves while no tile sees more than
+#: ``PREFILL_SPLIT_KEYS`` keys: behind a long prefix a block lives long enough for two independent blocks on a
+#: CU to overlap better than two sets in step.  Measured with cold caches at head size 128, one set against two
+#: (us): 256 blocks 41 / 35 without a prefix, 286 / 215 behind 8,192 keys; 384 blocks 57 / 46 without, 90 / 85
+#: behind 1,024, 121 / 123 behind 2,048, 313 / 367 behind 8,192; 512 blocks 75 / 69 without, 108 / 107 behind
+#: 1,024, 207 / 227 behind 4,096, 337 / 387 behind 8,192; 768 blocks 117 / 129 without, 578 / 588 behind 8,192;
+#: 1,024 blocks 194 / 201.
+PREFILL_SPLIT_BLOCKS = 512
+PREFILL_SPLIT_KEYS = 3072
 
 
-def prefill_key_groups(n_tiles: int, n_kv_heads: int) -> int:
+def prefill_key_groups(n_tiles: int, n_kv_heads: int, longest_keys: int = 0) -> int:
     """Sets of waves per block of the prefill kernel.  A launch whose blocks all fit the GPU at once
     takes as long as its longest block; with two sets of waves, each with every second tile of keys,
     that block's chain is half as long.  A launch of many more blocks keeps the CUs busy anyway, and
-    there two independent blocks on a CU overlap better than two sets of waves in step."""
-    return 2 if n_tiles * n_kv_heads <= PREFILL_SPLIT_BLOCKS else 1
+    there two independent blocks on a CU overlap better than two sets of waves in step.
+    ``longest_keys``: the most keys any tile of the launch sees."""
+    blocks = n_tiles * n_kv_heads
+    if blocks <= PREFILL_SPLIT_ALWAYS:
+        return 2
+    return 2 if blocks <= PREFILL_SPLIT_BLOCKS and longest_keys <= PREFILL_SPLIT_KEYS else 1
 
 
 def prefill_tile_count(qo_indptr, first_row: int, n_rows: int, queries_per_tile: int) -> int:

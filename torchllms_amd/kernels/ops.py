@@ -66,7 +66,9 @@ from .attention_ops import (  # noqa: F401
     DECODE_HEAD_DIMS,
     PREFILL_HEAD_DIMS,
     PREFILL_RESIDENT_BLOCKS,
+    PREFILL_SPLIT_ALWAYS,
     PREFILL_SPLIT_BLOCKS,
+    PREFILL_SPLIT_KEYS,
     attention_decode,
     attention_generic,
     attention_generic_split,
