@@ -1101,7 +1101,7 @@ def _prefill(rows, hq, hkv, dh, page, window=0, seed=0, key_groups=1):
     n = qo[-1]
     wide = torch.cat([torch.cat(qs), torch.randn(n, 2 * hkv * dh).bfloat16()], dim=1).to(DEV)
     qpt = ops.prefill_queries_per_tile(hq, hkv, dh)
-    trow, tq0 = ops.prefill_tiles(qo, 0, len(rows), qpt, kv, window, hkv, key_groups)  # in the balanced order the engine uses
+    trow, tq0 = ops.prefill_tiles(qo, 0, len(rows), qpt, kv, window)  # in the balanced order the engine uses
     out = torch.zeros(n, hq * dh, dtype=torch.bfloat16, device=DEV)
     ops.attention_prefill(wide, hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32(qo), _i32(kv), _i32(tables), _i32(trow), _i32(tq0),
                           window, dh ** -0.5, out, key_groups=key_groups)

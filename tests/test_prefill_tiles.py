@@ -4,7 +4,6 @@ tokens, ordered so that the launch is balanced."""
 import random
 
 from torchllms_amd.kernels.ops import (
-    PREFILL_RESIDENT_BLOCKS,
     PREFILL_SPLIT_BLOCKS,
     prefill_key_groups,
     prefill_tile_count,
@@ -32,7 +31,7 @@ def test_tiles_are_a_partition_whatever_the_order():
             qo.append(qo[-1] + q)
         qpt = rng.choice([8, 16, 32, 128])
         window = rng.choice([0, 0, 7, 100])
-        rows, q0s = prefill_tiles(qo, first, n_rows, qpt, kv, window, rng.choice([1, 8]), rng.choice([1, 2]))
+        rows, q0s = prefill_tiles(qo, first, n_rows, qpt, kv, window)
         want = sorted((r, q0) for r in range(first, n_rows) for q0 in range(0, q_lens[r], qpt))
         assert sorted(zip(rows, q0s)) == want
         assert prefill_tile_count(qo, first, n_rows, qpt) == len(want)
@@ -40,21 +39,9 @@ def test_tiles_are_a_partition_whatever_the_order():
         assert list(zip(plain_rows, plain_q0s)) == want
 
 
-def test_a_launch_that_fits_at_once_pairs_long_tiles_with_short_ones():
-    qo, kv, qpt, heads = [0, 2048], [2048], 32, 8
-    rows, q0s = prefill_tiles(qo, 0, 1, qpt, kv, 0, heads)
-    assert len(rows) * heads <= 2 * PREFILL_RESIDENT_BLOCKS
-    costs = [_cost(r, q, qo, kv, qpt, 0) for r, q in zip(rows, q0s)]
-    half = len(costs) // 2
-    assert costs[:half] == sorted(costs[:half], reverse=True) and costs[half:] == sorted(costs[half:])
-    sums = [costs[i] + costs[half + i] for i in range(half)]  # what meets on one CU
-    assert max(sums) - min(sums) <= 2 * qpt
-
-
-def test_a_long_launch_starts_its_longest_tiles_first():
+def test_a_launch_starts_its_longest_tiles_first():
     qo, kv, qpt = [0, 100, 8292], [5000, 8192], 32
-    rows, q0s = prefill_tiles(qo, 0, 2, qpt, kv, 0, 8)
-    assert len(rows) * 8 > 2 * PREFILL_RESIDENT_BLOCKS
+    rows, q0s = prefill_tiles(qo, 0, 2, qpt, kv, 0)
     costs = [_cost(r, q, qo, kv, qpt, 0) for r, q in zip(rows, q0s)]
     assert costs == sorted(costs, reverse=True)
     assert rows[0] == 1 and rows[-1] == 1 and 0 in rows  # the short row's tiles lie where their length puts them
@@ -66,7 +53,7 @@ def test_two_sets_of_waves_for_launches_that_fit_at_once_and_then_longest_first(
     assert n * heads <= PREFILL_SPLIT_BLOCKS and prefill_key_groups(n, heads, 2048) == 2
     assert prefill_key_groups(n, heads, 2048 + 4096) == 1  # behind a long prefix two blocks a CU do better
     assert prefill_key_groups(n // 2, heads, 2048 + 8192) == 2  # too few blocks to give every CU two
-    rows, q0s = prefill_tiles(qo, 0, 1, qpt, kv, 0, heads, key_groups=2)
+    rows, q0s = prefill_tiles(qo, 0, 1, qpt, kv, 0)
     costs = [_cost(r, q, qo, kv, qpt, 0) for r, q in zip(rows, q0s)]
     assert costs == sorted(costs, reverse=True)
     assert prefill_key_groups(prefill_tile_count([0, 8192], 0, 1, qpt), heads) == 1

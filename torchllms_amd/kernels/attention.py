@@ -74,7 +74,7 @@ def paged_attention(
                 if window > 0:
                     longest = min(longest, window + qpt)
                 key_groups = ops.prefill_key_groups(ops.prefill_tile_count(host.qo_indptr, n_dec, host.n_seqs, qpt), n_kv_heads, longest)
-                rows, q0s = ops.prefill_tiles(host.qo_indptr, n_dec, host.n_seqs, qpt, host.kv_lens, window, n_kv_heads, key_groups)
+                rows, q0s = ops.prefill_tiles(host.qo_indptr, n_dec, host.n_seqs, qpt, host.kv_lens, window)
                 both = torch.tensor([rows, q0s], dtype=torch.int32).to(qkv.device)
                 tiles = (both[0], both[1], key_groups)
                 ctx.scratch[key] = tiles

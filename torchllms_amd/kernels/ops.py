@@ -65,7 +65,6 @@ from .attention_ops import (  # noqa: F401
     ATTENTION_MAX_HEAD_DIM,
     DECODE_HEAD_DIMS,
     PREFILL_HEAD_DIMS,
-    PREFILL_RESIDENT_BLOCKS,
     PREFILL_SPLIT_ALWAYS,
     PREFILL_SPLIT_BLOCKS,
     PREFILL_SPLIT_KEYS,
