@@ -113,6 +113,11 @@ __device__ __forceinline__ void load_value_words(const bf16_t* src, uint32_t* ds
   }
 }
 
+// kPow2Pages: the page size is a power of two, so a key's page and offset are a shift and a mask;
+// the general kernel divides, inlined at each of the 25 places that look a page up (6.6 KB of code
+// against 4.7).  Both run at the same speed; they are two kernels so that neither carries the
+// other's code and branches.
+template <bool kPow2Pages>
 __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decode_kernel(DecodeArgs a) {
   extern __shared__ float red_o[];  // [kWaves][group][DH]: per-wave partial outputs for the block merge
   __shared__ float red_m[kWaves][16], red_l[kWaves][16];
@@ -162,8 +167,8 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
   // reads one row that the block has read already, not rows of the next split, which another block
   // reads (a quarter more traffic at splits of 256 keys).
   auto clamp_key = [&](int key) { return key < lo ? lo : (key > split_end ? split_end : key); };
-  auto block_of = [&](int key) { return a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size; };
-  auto offset_of = [&](int key) { return a.page_shift >= 0 ? key & (a.page_size - 1) : key % a.page_size; };
+  auto block_of = [&](int key) { return kPow2Pages ? key >> a.page_shift : key / a.page_size; };
+  auto offset_of = [&](int key) { return kPow2Pages ? key & (a.page_size - 1) : key % a.page_size; };
   auto row_ptr = [&](const bf16_t* pages, int page, int key) {
     return pages + ((size_t)page * a.n_kv_heads + kvh) * head_elems + (size_t)offset_of(key) * DH;
   };
@@ -182,6 +187,11 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
     for (int j = 0; j < 4; ++j) tp.v[j] = bt[block_of(clamp_key(base + 4 * g4 + j))];
     return tp;
   };
+
+  // The compiler may not move a load across this: without it, it sinks the prefetches of the next
+  // tile down to their first use, at the top of the next pass, and every tile waits a whole trip
+  // to memory.
+  auto keep_loads_here = [] { asm volatile("" ::: "memory"); };
 
   // Rolling prefetch: the keys of tile t+1 are requested as soon as the MFMAs of tile t have read
   // their registers, the values of tile t+1 as soon as the value operands of tile t are packed, so
@@ -208,6 +218,7 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
     const TilePages pages_now = fetch_pages(base);
     load_k(base, pages_now);
     load_v(base, pages_now);
+    keep_loads_here();
   }
   for (; base <= split_end; base += kWaves * kTile) {
     const int next = base + kWaves * kTile;
@@ -220,6 +231,7 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
       c = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kreg[u].half(1), qreg[u].half(1), c, 0, 0, 0);
     }
     load_k(next, pages_next);  // unconditional: past the split's end the keys are clamped and unused
+    keep_loads_here();
     float s[4];
     float tmax = -INFINITY;
 #pragma unroll
@@ -253,7 +265,9 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
       acc[e] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop, pop, acc[e], 0, 0, 0);
     }
     load_v(next, pages_next);
+    keep_loads_here();
     pages_next = fetch_pages(next + kWaves * kTile);  // for the tile after the next
+    keep_loads_here();
   }
 
   // the lane's own sums join over the four row groups
@@ -399,7 +413,10 @@ TL_EXPORT int tl_attn_decode(const void* q, int q_stride, void* out, int out_str
   dim3 grid(n_splits, n_kv_heads, n_tokens);
   const int threads = kWaves * kWave;
   const size_t lds = (size_t)kWaves * R * DH * sizeof(float);
-  attn_decode_kernel<<<grid, threads, lds, stream>>>(a);
+  if (a.page_shift >= 0)
+    attn_decode_kernel<true><<<grid, threads, lds, stream>>>(a);
+  else
+    attn_decode_kernel<false><<<grid, threads, lds, stream>>>(a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return variant_fail(TL_ERR_HIP, "attn_decode: %s", hipGetErrorString(e));
   if (n_splits > 1) {
