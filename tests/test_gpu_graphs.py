@@ -69,18 +69,17 @@ def test_graph_replays_match_eager_steps(tmp_path, name, dtype):
         eng.cache.check_invariants()
 
 
-@pytest.mark.skipif(False, reason="")
 def test_context_cap_buckets():
     from torchllms_amd.engine.graphs import context_cap
 
-    assert [context_cap(n) for n in (1, 512, 513, 1024, 5000, 8192)] == [512, 512, 1024, 1024, 8192, 8192]
+    assert [context_cap(n) for n in (1, 512, 513, 768, 769, 1024, 2176, 5000, 6144, 6145, 8192)] == [512, 512, 768, 768, 1024, 1024, 3072, 6144, 6144, 8192, 8192]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_prepared_decode_steps_match_plain_steps(tmp_path, dtype):
     """Decode steps prepared one step ahead (plan made and uploaded before the tokens are known)
     give the logits of steps planned when they run, across pages' edges and the context cap's
-    step from 512 to 1024, and a preparation that no longer fits is refused."""
+    step from 512 to 768, and a preparation that no longer fits is refused."""
     from torchllms_amd.engine import Engine, StepEntry
 
     cfg = TINY["B"]

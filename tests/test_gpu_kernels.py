@@ -792,9 +792,9 @@ def test_attention_decode_says_what_it_takes():
     assert ops.plan_decode_splits(8, 8, 8192) == (1024, 8)
     assert ops.plan_decode_splits(64, 8, 8192) == (8192, 1)
     assert ops.plan_decode_splits(64, 8, 8192, uneven=True) == (512, 16)
-    assert ops.plan_decode_splits(2, 8, 8192, uneven=True) == (512, 16)
-    assert ops.plan_decode_splits(2, 8, 4096) == (256, 16)  # 512 keys a split would leave 128 blocks
-    assert ops.plan_decode_splits(64, 8, 40) == (512, 1)
+    assert ops.plan_decode_splits(2, 8, 8192, uneven=True) == (256, 32)  # what equal requests would get is shorter still
+    assert ops.plan_decode_splits(2, 8, 4096) == (256, 16)
+    assert ops.plan_decode_splits(64, 8, 40) == (256, 1)
     assert ops.plan_decode_splits(1, 8, 8192) == (256, 32)
 
 

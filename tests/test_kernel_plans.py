@@ -6,19 +6,27 @@ import torch
 from torchllms_amd.kernels import attention_ops, ops, products
 
 
-def test_decode_splits_cover_the_range_with_about_512_blocks():
-    for n_tokens in (1, 2, 3, 8, 17, 64, 200):
-        for n_kv_heads in (1, 2, 8):
-            for longest in (1, 15, 256, 1000, 8192, 70000, 131072):
-                for uneven in (False, True):
-                    split, n_splits = ops.plan_decode_splits(n_tokens, n_kv_heads, longest, uneven=uneven)
-                    assert split % 64 == 0 and split >= 256
-                    assert n_splits >= 1 and (n_splits - 1) * split < max(longest, 1) <= n_splits * split
-                    if uneven:
-                        assert split <= attention_ops.DECODE_UNEVEN_SPLIT == 512
-                    elif n_splits > 1:
-                        # no more blocks than asked for, unless the shortest split allowed is reached
-                        assert split == 256 or n_tokens * n_kv_heads * n_splits <= 512 + n_tokens * n_kv_heads
+def test_decode_splits_cover_the_range_and_stay_under_a_cu_s_share_of_blocks():
+    for head_dim, per_cu in ((32, 3), (64, 3), (128, 2), (256, 1)):
+        for n_tokens in (1, 2, 3, 8, 17, 64, 200):
+            for n_kv_heads in (1, 2, 8):
+                for longest in (1, 15, 256, 1000, 8192, 70000, 131072):
+                    for uneven in (False, True):
+                        split, n_splits = ops.plan_decode_splits(n_tokens, n_kv_heads, longest, head_dim, uneven=uneven)
+                        assert split % 64 == 0 and split >= 256
+                        assert n_splits >= 1 and (n_splits - 1) * split < max(longest, 1) <= n_splits * split
+                        if uneven:
+                            assert split <= attention_ops.DECODE_UNEVEN_SPLIT == 512
+                        elif n_splits > 1:
+                            # never more blocks than the CUs take at a time, unless the shortest split allowed is reached
+                            assert split == 256 or n_tokens * n_kv_heads * n_splits <= 256 * per_cu
+                            # and no fewer splits than that allows: one split more would be too many
+                            shorter = split - 64
+                            assert shorter < 256 or n_tokens * n_kv_heads * -(-longest // shorter) > 256 * per_cu or -(-longest // shorter) == n_splits
+    # head sizes with fewer bytes a key take more blocks a CU
+    assert ops.plan_decode_splits(8, 8, 2176, 128) == (320, 7)
+    assert ops.plan_decode_splits(8, 8, 2176, 64) == (256, 9)
+    assert ops.plan_decode_splits(8, 4, 8192, 256) == (1024, 8)
 
 
 def test_a_sampled_row_is_cut_only_when_rows_are_few_and_long():

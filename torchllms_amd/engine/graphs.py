@@ -8,9 +8,9 @@ reference reaches for ``torch.compile(mode="reduce-overhead")`` here:
 torchllms/inference/llm.py:202-283.)
 
 A graph is keyed by what fixes its launches: the number of requests, the number of wanted logit
-rows, a power-of-two cap on the context length, which bounds the block tables' width and the
-number of key splits of the decode attention, and whether the requests differ much in length,
-which makes those splits shorter.  No memset node is recorded: buffers are written by
+rows, a cap on the context length (a power of two or one and a half times one), which bounds the
+block tables' width and fixes the key splits of the decode attention, and whether the requests
+differ much in length, which makes those splits shorter.  No memset node is recorded: buffers are written by
 kernels only.
 """
 
@@ -28,8 +28,14 @@ MIN_CONTEXT_CAP = 512
 
 
 def context_cap(max_kv_len: int) -> int:
+    """The smallest of 512, 768, 1,024, 1,536, 2,048, ... that holds ``max_kv_len``.  The decode
+    attention cuts the keys into splits for the cap, not for the contexts of the day, so a cap far
+    above them gives splits that are too long and too few: with powers of two alone, 8 requests of
+    2,176 tokens got the splits of 4,096 and the kernel took 24.9 us instead of 21.9."""
     cap = MIN_CONTEXT_CAP
     while cap < max_kv_len:
+        if cap // 2 * 3 >= max_kv_len:
+            return cap // 2 * 3
         cap *= 2
     return cap
 

@@ -137,21 +137,25 @@ def decode_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: i
 
 
 _DECODE_MIN_SPLIT = 256  # keys: shorter splits cost more in launch and merge than they gain in spread
+_N_CUS = 256
+#: blocks a CU takes at a time before a launch stops gaining from more splits, by head size: about
+#: 64 KB of keys and values in flight on a CU (a block's four waves fetch 64 keys and values a pass)
+_DECODE_BLOCKS_PER_CU = {32: 3, 64: 3, 128: 2, 256: 1}
 
 
 DECODE_UNEVEN_SPLIT = 512  # keys: the longest split when requests differ much in length (measured with 64 requests of 128 to 4,608 tokens: 1 to 1.5% more tokens a second than with 1,024, 12% more than with 2,048)
 
 
-def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, target_blocks: int = 512, uneven: bool = False):
+def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, head_dim: int = 128, uneven: bool = False):
     """``(split_size, n_splits)`` for a decode launch whose longest visible key range (counted from
-    its 16-aligned start) is ``longest``: enough splits for about two blocks on each of the 256
-    CUs, none shorter than 256 keys.  Measured from one request of 131,072 tokens to 128 requests
-    of 2,048, 512 blocks were the best or within 2% of it: a block's waves keep enough loads in
-    flight by themselves, and every further split costs its start, its partial results and its
-    share of the merge.  A batch with 512 (request, kv head) pairs or more is not split at all,
-    if the requests are about equally long.  (Alone and on pages in random order, 8 requests of
-    8,192 tokens ran a little faster with four splits of 2,048 keys than with eight of 1,024; inside
-    the decode step it was the other way round, 52.9 against 49.5 us, and the step decides.)
+    its 16-aligned start) is ``longest``: as many splits as give every CU its share of blocks and
+    no more (two blocks a CU at head size 128, one at 256, three at 64 and 32), none shorter than
+    256 keys.  A launch is as long as its most loaded CU, so a few blocks beyond a whole number a CU
+    cost as much as a whole further round, and every split costs its start, its partial results
+    and its share of the merge; staying under the limit was the best choice or within 1% of it on
+    average (at most 11%) over 1 to 100 requests of 700 to 20,000 tokens at each head size, where
+    always aiming at 512 blocks lost 3 to 16% on average.  A batch with that many (request, kv
+    head) pairs or more is not split at all, if the requests are about equally long.
 
     ``uneven``: the requests differ much in length.  Then all blocks of such a launch would be
     resident at once and stay where they were put, a CU with long requests' blocks working on
@@ -159,16 +163,12 @@ def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, target_bloc
     more blocks than fit, and those that wait go where others end.  (64 requests of 128 to 4,608
     tokens: 30% less time than unsplit; 64 equal ones: 10% more, hence the switch.)"""
     pairs = max(n_tokens * n_kv_heads, 1)
-    want = max(-(-target_blocks // pairs), 1)
+    limit = _N_CUS * _DECODE_BLOCKS_PER_CU.get(head_dim, 2)
+    want = max(limit // pairs, 1)
     split = -(-max(longest, 1) // want)
     if uneven:
         split = min(split, DECODE_UNEVEN_SPLIT)
     split = max(-(-split // _DECODE_BLOCK_KEYS) * _DECODE_BLOCK_KEYS, _DECODE_MIN_SPLIT)
-    # splits of 256 keys only while 512 keys would leave fewer than one block for each CU (measured
-    # with cold caches: 2 requests of 8,192 tokens 23.4 against 25.8 us, 8 of 2,048 21.7 against 23.3,
-    # 2 of 4,096, where 512 keys give 128 blocks, 20.0 against 18.4)
-    if split < 2 * _DECODE_MIN_SPLIT and pairs * -(-max(longest, 1) // (2 * _DECODE_MIN_SPLIT)) >= 256:
-        split = 2 * _DECODE_MIN_SPLIT
     return split, max(-(-max(longest, 1) // split), 1)
 
 
@@ -211,7 +211,7 @@ def attention_decode(
     if out is None:
         out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
     if split_size is None:
-        split_size, n_splits = plan_decode_splits(n, n_kv_heads, longest, uneven=uneven)
+        split_size, n_splits = plan_decode_splits(n, n_kv_heads, longest, head_dim, uneven=uneven)
     else:
         n_splits = max(-(-max(longest, 1) // split_size), 1)
     ws_o = ws_ml = None
