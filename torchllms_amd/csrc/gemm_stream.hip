@@ -151,19 +151,26 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     if (s >= nst) s -= nst;
     return step_lo + s;
   };
-  // The prefetches are unconditional (past the end they repeat the last step and are ignored): a
-  // load under a branch would make the wait before its use cover both paths, that is, wait for the
-  // prefetch itself.
+  // Inside the loop the prefetches are unconditional: a load under a branch would make the wait
+  // before its use cover both paths, that is, wait for the prefetch itself.  The last one or two
+  // steps stand behind the loop, so that nothing is fetched that nobody uses (with two to four
+  // steps a wave, as in the products with few columns, one spare fetch was a fifth of all).
   if (nst > 0) {
     fetch(step_of(0), w0, a0);
     int i = 0;
-    for (; i + 1 < nst; i += 2) {
+    for (; i + 2 < nst; i += 2) {
       fetch(step_of(i + 1), w1, a1);
       consume(w0, a0);
-      fetch(step_of(min(i + 2, nst - 1)), w0, a0);
+      fetch(step_of(i + 2), w0, a0);
       consume(w1, a1);
     }
-    if (i < nst) consume(w0, a0);  // an odd number of steps: the last one is already loaded
+    if (i + 1 < nst) {
+      fetch(step_of(i + 1), w1, a1);
+      consume(w0, a0);
+      consume(w1, a1);
+    } else {
+      consume(w0, a0);
+    }
   }
   // the partial step: pieces past K are read from a clamped address and the A side is zeroed, so the
   // out-of-range products vanish
