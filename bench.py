@@ -41,7 +41,8 @@ from ctypes import c_int, c_size_t, c_void_p
 
 HBM_GBS = 8000.0  # MI355X HBM3E, published
 PEAK_SIGNATURES = {"tl_peak_stream_read": [c_void_p, c_size_t, c_int, c_void_p, c_void_p],
-                   "tl_peak_mfma_bf16": [c_int, c_int, c_void_p, c_void_p]}
+                   "tl_peak_mfma_bf16": [c_int, c_int, c_void_p, c_void_p],
+                   "tl_peak_fma_f32": [c_int, c_int, c_void_p, c_void_p]}
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # dense MFMA, published
 
 # the model of the headline benchmark: Llama-3.1-8B layer sizes, random weights
@@ -292,8 +293,9 @@ def serve_run(args, shape) -> int:
 def peaks_run(args) -> int:
     """What this GPU reaches at its clocks of today, beside the published figures: a read of 4 GiB by a
     kernel of 16-byte loads, a device-to-device copy (its bytes counted once read, once written), MFMA
-    bfloat16 16x16x32 instructions issued from registers alone, and the library's product of two
-    8,192 x 8,192 bfloat16 matrices."""
+    bfloat16 16x16x32 instructions issued from registers alone, the library's product of two
+    8,192 x 8,192 bfloat16 matrices, and plain 32-bit multiply-adds from registers alone (the
+    arithmetic of the 32-bit path's products)."""
     import torch
 
     from torchllms_amd.kernels import lib
@@ -321,6 +323,9 @@ def peaks_run(args) -> int:
     iters, blocks = 20000, 256 * 8
     mfma_ms = best_ms(lambda: lib.check(peaks.tl_peak_mfma_bf16(iters, blocks, None, stream), peaks, "tl_variant_last_error"))
     mfma_tflops = blocks * 4 * iters * 8 * (2 * 16 * 16 * 32) / (mfma_ms * 1e-3) / 1e12
+    fma_iters = 4000
+    fma_ms = best_ms(lambda: lib.check(peaks.tl_peak_fma_f32(fma_iters, blocks, None, stream), peaks, "tl_variant_last_error"))
+    fma_tflops = blocks * 256 * fma_iters * 16 * 2 / (fma_ms * 1e-3) / 1e12
     a = torch.randn(8192, 8192, device=dev).to(torch.bfloat16)
     b = torch.randn(8192, 8192, device=dev).to(torch.bfloat16)
     mm_ms = best_ms(lambda: torch.matmul(a, b))
@@ -330,6 +335,7 @@ def peaks_run(args) -> int:
         "hbm_copy_gbs_read_plus_write": round(2 * src.numel() / (copy_ms * 1e-3) / 1e9, 1),
         "mfma_bf16_tflops": round(mfma_tflops, 1), "mfma_bf16_frac_of_published": round(mfma_tflops / PEAK_TFLOPS["bfloat16"], 4),
         "library_matmul_bf16_tflops": round(2 * 8192 ** 3 / (mm_ms * 1e-3) / 1e12, 1),
+        "fma_f32_tflops": round(fma_tflops, 1), "fma_f32_frac_of_published": round(fma_tflops / PEAK_TFLOPS["float32"], 4),
         "published": {"hbm_gbs": HBM_GBS, "mfma_bf16_tflops": PEAK_TFLOPS["bfloat16"], "fp32_tflops": PEAK_TFLOPS["float32"]},
     }))
     return 0

@@ -60,6 +60,23 @@ __global__ void __launch_bounds__(256) mfma_rate_kernel(int iters, float* sink) 
   for (int j = 0; j < 8; ++j) total += acc[j].x + acc[j].y + acc[j].z + acc[j].w;
   if (total == -1.f && sink) sink[0] = total;
 }
+// Sixteen independent 32-bit multiply-adds per lane and pass: what the vector units give the 32-bit
+// path's products, which are plain FMAs (compiled, like everything here, without packed 32-bit
+// instructions).
+__global__ void __launch_bounds__(256) fma_rate_kernel(int iters, float* sink) {
+  float acc[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) acc[j] = (float)(threadIdx.x + j);
+  const float a = 1.0f + 1e-7f * (float)threadIdx.x, b = 1e-9f * (float)blockIdx.x;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[j] = __builtin_fmaf(acc[j], a, b);
+  }
+  float total = 0.f;
+#pragma unroll
+  for (int j = 0; j < 16; ++j) total += acc[j];
+  if (total == -1.f && sink) sink[0] = total;
+}
 }  // namespace
 
 TL_EXPORT const char* tl_variant_last_error() { return g_error; }
@@ -78,4 +95,12 @@ TL_EXPORT int tl_peak_mfma_bf16(int iters, int blocks, void* sink, hipStream_t s
   mfma_rate_kernel<<<blocks, 256, 0, stream>>>(iters, (float*)sink);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? TL_OK : fail(TL_ERR_HIP, "peak_mfma_bf16: %s", hipGetErrorString(e));
+}
+
+// `blocks` blocks of 256 threads, each thread doing iters * 16 multiply-adds (2 flop each).
+TL_EXPORT int tl_peak_fma_f32(int iters, int blocks, void* sink, hipStream_t stream) {
+  if (iters <= 0 || blocks <= 0) return fail(TL_ERR_ARG, "peak_fma_f32: bad arguments");
+  fma_rate_kernel<<<blocks, 256, 0, stream>>>(iters, (float*)sink);
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? TL_OK : fail(TL_ERR_HIP, "peak_fma_f32: %s", hipGetErrorString(e));
 }
