@@ -348,6 +348,30 @@ class Engine:
         self.tokens_run += len(prepared.rids)
         return logits
 
+    @torch.inference_mode()
+    def step_prepared_on_device(self, prepared: "PreparedDecode", rids: Sequence[Hashable], token_ids: torch.Tensor) -> Optional[torch.Tensor]:
+        """``step_prepared`` for a step whose tokens the host does not know yet: ``token_ids`` is what
+        the sampling kernel returned for the last step, still on the device, one token for each of
+        ``rids``, which must be the prepared requests in their order, each wanting its one row.  The
+        step is queued behind the sampling; nothing waits.  The caller vouches for the tokens (the
+        sampling kernel returns token ids) and has to cope with a request that turns out to have
+        ended with the token it is fed here: its row is then wasted, the other rows are as good
+        as any.  None, with nothing run, when the preparation does not fit."""
+        last = self._last_decode
+        if last is None or last[2] is not prepared.previous or prepared.epoch != self.cache.epoch:
+            return None
+        if list(rids) != list(prepared.rids) or any(want != [0] for want in prepared.wants):
+            return None
+        if token_ids.dtype != torch.int32 or token_ids.numel() != len(prepared.rids) or token_ids.device != prepared.graph.dev.device:
+            return None
+        logits = prepared.graph.launch(token_ids)
+        for rid in prepared.rids:
+            self.cache.advance(rid, 1)
+        self._last_decode = (prepared.rids, prepared.wants, prepared.layout, self.cache.epoch)
+        self.steps_run += 1
+        self.tokens_run += len(prepared.rids)
+        return logits
+
     def plan(self, entries: Sequence[StepEntry]) -> StepLayout:
         """Reserve pages for the step's tokens (all or nothing) and lay the step out."""
         # decode steps follow one another with the same requests: such a step is planned from the

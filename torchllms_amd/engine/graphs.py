@@ -114,9 +114,14 @@ class DecodeGraph:
         self.pack(layout)
         return self.launch()
 
-    def launch(self) -> torch.Tensor:
-        """Upload the packed plan and replay."""
+    def launch(self, tokens_on_device: torch.Tensor = None) -> torch.Tensor:
+        """Upload the packed plan and replay.  ``tokens_on_device``: the step's token ids as an int32
+        tensor on the device, which take the place of the plan's (they need not be known on the host:
+        the copy is queued behind whatever produces them)."""
         self._upload()
+        if tokens_on_device is not None:
+            off = self.offsets[0]
+            self.dev[off : off + tokens_on_device.numel()].copy_(tokens_on_device)
         self.graph.replay()
         self.replays += 1
         return self.logits.clone()

@@ -40,7 +40,9 @@ class GenerationLoop:
         self.engine = engine
         self.sampler = sampler
         self.look_ahead = look_ahead
-        self.stats = {"prepared_steps": 0}
+        self.stats = {"prepared_steps": 0, "launched_ahead": 0}
+        self.launch_ahead = look_ahead  # (a switch of its own for measurements)
+        self._host_tokens = self._home = None
         self.scheduler = Scheduler(engine.cache, max_num_seqs, max_num_batched_tokens, max_model_len, prefill_chunk)
 
     def run(self, prompts: Sequence[Sequence[int]], params: Sequence[SamplingParams], on_step=None):
@@ -48,32 +50,64 @@ class GenerationLoop:
 
         While the GPU runs a decode step, an engine that can (``prepare_decode``) prepares the next
         one for the case that the same requests decode again; the scheduler still decides every
-        step, and the preparation is used only when its plan is that case."""
+        step, and the preparation is used only when its plan is that case.
+
+        An engine that can (``step_prepared_on_device``) is then given the prepared step at once,
+        with the sampled tokens still on the device, and the host reads them while that step runs:
+        the GPU does not wait for the host between two decode steps.  This is done only where no
+        request can reach its token budget with the sampled token, so the step is wrong only for a
+        request that ends on a stop token: its row is dropped, the other rows are the step that
+        the scheduler would have planned for them (one token each, pages taken by the
+        preparation), and requests that wait are admitted a step later."""
+        from ..engine.scheduler import ScheduledEntry, StepPlan
+
         sched = self.scheduler
         requests = [sched.add(("gen", id(self), i), p, sp) for i, (p, sp) in enumerate(zip(prompts, params))]
         prepare = getattr(self.engine, "prepare_decode", None) if self.look_ahead else None
         launch = getattr(self.sampler, "launch", None)
+        launch_ahead = getattr(self.engine, "step_prepared_on_device", None) if self.look_ahead and self.launch_ahead else None
         prepared = None
+        ahead = None  # (plan, logits) of a step that is already queued
         try:
             while sched.has_work:
-                plan = sched.schedule()
-                entries = plan.step_entries()
-                logits = None
-                if prepared is not None:
-                    logits = self.engine.step_prepared(prepared, entries)  # None: it is another step
-                    self.stats["prepared_steps"] += logits is not None
-                if logits is None:
-                    logits = self.engine.step(entries)
+                if ahead is not None:
+                    plan, logits = ahead
+                    ahead = None
+                else:
+                    plan = sched.schedule()
+                    entries = plan.step_entries()
+                    logits = None
+                    if prepared is not None:
+                        logits = self.engine.step_prepared(prepared, entries)  # None: it is another step
+                        self.stats["prepared_steps"] += logits is not None
+                    if logits is None:
+                        logits = self.engine.step(entries)
                 prepared = None
                 sampling = [e.request for e in plan.entries if e.samples]
                 counters = [len(r.output) for r in sampling]
+                next_logits = None
                 if prepare is not None and launch is not None and _decodes_on(plan):
                     pending = launch(logits, [r.params for r in sampling], counters)
+                    arriving = self._send_home(pending) if launch_ahead is not None else None
                     prepared = prepare()  # the GPU is busy with the step meanwhile
-                    tokens = pending.tolist()
+                    if prepared is not None and arriving is not None:
+                        next_logits = launch_ahead(prepared, [e.request.rid for e in plan.entries], pending)
+                    if next_logits is not None:
+                        prepared = None  # used
+                        self.stats["prepared_steps"] += 1
+                        self.stats["launched_ahead"] += 1
+                    tokens = self._arrived(arriving, pending.numel()) if arriving is not None else pending.tolist()
                 else:
                     tokens = self.sampler(logits, [r.params for r in sampling], counters)
                 sched.update(plan, tokens)
+                if next_logits is not None:
+                    # the step that is running: one token for every request that is still there
+                    rows = [i for i, e in enumerate(plan.entries) if not e.request.finished]
+                    if rows:
+                        if len(rows) < len(plan.entries):
+                            next_logits = next_logits[rows]
+                        going_on = [plan.entries[i].request for i in rows]
+                        ahead = (StepPlan(entries=[ScheduledEntry(r, [r.last_token], True) for r in going_on]), next_logits)
                 if on_step is not None:
                     on_step(plan)
         except BaseException:
@@ -83,6 +117,26 @@ class GenerationLoop:
                     sched.abort(r)
             raise
         return requests
+
+    def _send_home(self, pending):
+        """Queue the copy of the sampled token ids to pinned host memory right behind the sampling,
+        on the same stream, before anything else is queued: it is done as soon as the sampling
+        is, whatever follows it.  (A copy on a stream of its own, waiting for an event behind the
+        sampling, made every kernel of the step that ran meanwhile slower: a queue that waits is
+        polled.)  Returns the event behind the copy."""
+        import torch
+
+        n = pending.numel()
+        if self._host_tokens is None or self._host_tokens.numel() < n:
+            self._host_tokens = torch.empty((max(n, 64),), dtype=torch.int32, pin_memory=True)
+            self._home = torch.cuda.Event()
+        self._host_tokens[:n].copy_(pending, non_blocking=True)
+        self._home.record()
+        return self._home
+
+    def _arrived(self, event, n: int) -> list:
+        event.synchronize()
+        return self._host_tokens[:n].tolist()
 
 
 def _decodes_on(plan) -> bool:
