@@ -783,6 +783,73 @@ def test_attention_decode_batch_with_different_lengths():
         torch.testing.assert_close(out.float().cpu(), torch.cat(wants), rtol=2 ** -7, atol=2 ** -7)
 
 
+def _fill_pages(k_pages, v_pages, table, k, v):
+    """Write dense keys/values [S, Hkv, dh] into the pages ``table`` names, whole pages at a time."""
+    S, hkv, dh = k.shape
+    page = k_pages.shape[2]
+    blocks = -(-S // page)
+    pad = blocks * page - S
+    idx = torch.tensor(table[:blocks])
+    for pages, x in ((k_pages, k), (v_pages, v)):
+        if pad:
+            x = torch.cat([x, pages[idx[-1], :, page - pad :].transpose(0, 1).to(x.dtype)])
+        pages[idx] = x.view(blocks, page, hkv, dh).transpose(1, 2).to(pages.dtype)
+
+
+@pytest.mark.parametrize("batch, S", [(1, 32768), (8, 32768), (64, 8192)])
+def test_attention_decode_at_the_longest_contexts_that_are_measured(batch, S):
+    """32,768 keys for one request (64 splits of 512 keys) and for eight (8 splits of 4,096), and 64
+    requests of 8,192 (one block walks all keys of a request, no merge): the launches of the context
+    sweep and of the batch-64 measurement.  Random scores in most rows; in some a single key, near
+    the start, at a split's edge or at the end, that outweighs all others."""
+    ops = _ops()
+    hq, hkv, dh, page = 32, 8, 128, 16
+    assert ops.plan_decode_splits(batch, hkv, S) == {1: (512, 64), 8: (4096, 8), 64: (8192, 1)}[batch]
+    g = torch.Generator().manual_seed(batch)
+    lens = [S - (0, 1, 15, 16, 17, 700, 0, 63)[i % 8] for i in range(batch)]
+    sharp = {0: 4095 if batch > 1 else None, 1: 0, 2: 4096, 3: lens[3 % batch] - 1, 5: 511, 6: 512, 7: S // 2 + 17}
+    n_pages = sum(-(-n // page) for n in lens) + 5
+    k_pages = torch.full((n_pages, hkv, page, dh), 30.0, dtype=torch.bfloat16)
+    v_pages = torch.full((n_pages, hkv, page, dh), -30.0, dtype=torch.bfloat16)
+    free = torch.randperm(n_pages, generator=g).tolist()
+    tables, wants, qs = [], [], []
+    width = -(-S // page)
+    for i, n in enumerate(lens):
+        k = torch.randn(n, hkv, dh, generator=g).bfloat16()
+        v = torch.randn(n, hkv, dh, generator=g).bfloat16()
+        q = (torch.randn(1, hq, dh, generator=g) * 2).bfloat16()
+        far = sharp.get(i) if i < 8 else None
+        if far is not None:
+            direction = torch.randn(dh, generator=g)
+            direction /= direction.norm()
+            k[far] = (direction * 12).bfloat16()
+            q = (direction * 12 * math.sqrt(dh) / 3).expand(1, hq, dh).bfloat16()
+        table = [free.pop() for _ in range(-(-n // page))]
+        _fill_pages(k_pages, v_pages, table, k, v)
+        tables.append(table + [-1] * (width - len(table)))
+        wants.append(plain.attention(q.float().to(DEV), k.float().to(DEV), v.float().to(DEV)).cpu())
+        if far is not None:  # the one key's value, to a part in a thousand
+            assert (wants[-1].view(hq, dh) - v[far].float().repeat_interleave(hq // hkv, dim=0)).abs().max() < 0.05
+        qs.append(q.reshape(1, hq * dh))
+    out = ops.attention_decode(
+        torch.cat(qs).to(DEV), hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32(list(range(batch))), _i32([n - 1 for n in lens]),
+        _i32(tables), 0, dh ** -0.5, max(lens),
+    )
+    torch.testing.assert_close(out.float().cpu(), torch.cat(wants), rtol=2 ** -7, atol=2 ** -7)
+    if batch == 1:  # the one request again, with one key that outweighs the others, in turn at these places
+        k_dev, v_dev = k_pages.to(DEV), v_pages.to(DEV)
+        for far in (0, 511, 512, 20000, S - 65, S - 1):
+            direction = torch.randn(dh, generator=g)
+            direction /= direction.norm()
+            kept = k_dev[table[far // page], :, far % page].clone()
+            k_dev[table[far // page], :, far % page] = (direction * 12).bfloat16().to(DEV)
+            qq = (direction * 12 * math.sqrt(dh) / 3).expand(1, hq, dh).reshape(1, hq * dh).bfloat16().to(DEV)
+            got = ops.attention_decode(qq, hq, hkv, dh, k_dev, v_dev, _i32([0]), _i32([S - 1]), _i32(tables), 0, dh ** -0.5, S)
+            k_dev[table[far // page], :, far % page] = kept
+            err = (got.float().cpu().view(hq, dh) - v[far].float().repeat_interleave(hq // hkv, dim=0)).abs().max().item()
+            assert err < 3e-2, f"key {far}: {err}"
+
+
 def test_attention_decode_says_what_it_takes():
     ops = _ops()
     assert ops.decode_attention_supported(torch.bfloat16, 32, 8, 128)
@@ -1171,3 +1238,43 @@ def test_attention_prefill_sharp_scores_find_the_right_key():
                                   _i32(trow), _i32(tq0), 0, dh ** -0.5, out, key_groups=key_groups)
             err = (out.float().cpu() - want).abs().amax(dim=1)
             assert err.max().item() < 3e-2, f"distance {dist}, {key_groups} key groups: first bad query {int((err >= 3e-2).nonzero()[0])}"
+
+
+@pytest.mark.parametrize("key_groups", [1, 2])
+def test_attention_prefill_behind_a_prefix_of_32768_keys(key_groups):
+    """Two tile rows of new tokens behind 32,704 cached ones: 512 tiles of keys a block, block tables
+    of 2,048 pages.  Random scores first; then every query matches exactly one key, at a fixed
+    distance that reaches from its own position to the first pages of the prefix."""
+    ops = _ops()
+    hq, hkv, dh, page, S, sq = 32, 8, 128, 16, 32768, 64
+    g = torch.Generator().manual_seed(5)
+    n_pages = S // page + 4
+    table = torch.randperm(n_pages, generator=g)[: S // page].tolist()
+    qpt = ops.prefill_queries_per_tile(hq, hkv, dh)
+    trow, tq0 = ops.prefill_tiles([0, sq], 0, 1, qpt, [S])
+    assert len(trow) == 2
+
+    def run(q, k, v):
+        k_pages = torch.full((n_pages, hkv, page, dh), 40.0, dtype=torch.bfloat16)
+        v_pages = torch.full((n_pages, hkv, page, dh), -40.0, dtype=torch.bfloat16)
+        _fill_pages(k_pages, v_pages, table, k, v)
+        out = torch.zeros(sq, hq * dh, dtype=torch.bfloat16, device=DEV)
+        ops.attention_prefill(q.reshape(sq, hq * dh).to(DEV), hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32([0, sq]), _i32([S]),
+                              _i32([table]), _i32(trow), _i32(tq0), 0, dh ** -0.5, out, key_groups=key_groups)
+        return out.float().cpu()
+
+    k = (torch.randn(S, hkv, dh, generator=g) * 0.5).bfloat16()
+    v = torch.randn(S, hkv, dh, generator=g).bfloat16()
+    q = (torch.randn(sq, hq, dh, generator=g) * 2).bfloat16()
+    want = plain.attention(q.float().to(DEV), k.float().to(DEV), v.float().to(DEV)).cpu()
+    torch.testing.assert_close(run(q, k, v), want, rtol=2 ** -6, atol=2 ** -6)
+
+    dirs = torch.randn(S, dh, generator=g)
+    dirs /= dirs.norm(dim=-1, keepdim=True)
+    k = (dirs * 12)[:, None, :].expand(S, hkv, dh).bfloat16()
+    for dist in (0, 1, 63, 64, 8191, 20000, S - sq):
+        tgt = torch.arange(S - sq, S) - dist
+        q = (dirs[tgt] * 12 * math.sqrt(dh) / 3)[:, None, :].expand(sq, hq, dh).bfloat16()
+        got = run(q, k, v)
+        err = (got - v[tgt].float().repeat_interleave(hq // hkv, dim=1).reshape(sq, hq * dh)).abs().amax(dim=1)
+        assert err.max().item() < 3e-2, f"distance {dist}: first bad query {int((err >= 3e-2).nonzero()[0])}"

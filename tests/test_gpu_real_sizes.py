@@ -307,3 +307,126 @@ def _many_live(model, many, dtype, live):
         tols = {r: _bf16_tolerance(weights, cfg, requests[r], truth[r]) for r in {rid for _, rid, _ in worst}}
         for err, rid, pos in worst:
             assert err <= tols[rid][pos].item(), f"{rid} position {pos}: {err} against {tols[rid][pos].item()}"
+
+
+# ----------------------------------------------------------------------------- context 8,192: the sizes of the headline measurement
+def _plain_on_gpu(weights, cfg, tokens, dtype):
+    """The plain model's logits with torch's tensor operations run on the GPU (the same functions; a
+    sequence of 8,192 tokens takes minutes on the CPU), back on the CPU as 32-bit."""
+    out = plain.forward(weights, cfg, tokens, dtype, device="cuda:0").float().cpu()
+    torch.cuda.empty_cache()
+    return out
+
+
+def _check_rows(name, got, want, dtype, tol):
+    err = (got - want).abs().amax(dim=-1)
+    bad = (err >= 10 * FP32_ATOL).nonzero().flatten() if dtype == "float32" else (err > tol).nonzero().flatten()
+    assert bad.numel() == 0, f"{name}: first wrong position {int(bad[0])} of {bad.numel()}, error {err[bad[0]].item()}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_request_of_8192_tokens_whole_in_portions_and_decoded_across_the_last_context_caps(one_layer, dtype):
+    """One request that fills the context of 8,192: in one step (a prefill launch of 2,048 blocks); in
+    portions of 4,096, 2, 3,000, 31 and 971 tokens with the last 92 one by one; and with three runs of
+    decode steps, at contexts 4,061 to 4,120, 6,121 to 6,180 and 8,101 to 8,192, replayed from graphs
+    recorded for the context caps 4,096, 6,144 and 8,192 (the widest block tables and the most key
+    splits of the decode attention), prompt portions of about 2,000 tokens in between."""
+    from torchllms_amd.engine import Engine
+
+    folder, cfg, weights = one_layer
+    n = 8192
+    tokens = random_tokens(n, ONE_LAYER["vocab_size"], 81)
+    want = _plain_on_gpu(weights, cfg, tokens, torch.float32)
+    tol = 2 * (_plain_on_gpu(weights, cfg, tokens, torch.bfloat16) - want).abs().amax(dim=-1) + 1e-3 if dtype == "bfloat16" else None
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=n // 16 + 1, max_seqs=2, max_model_len=n, use_graphs=True)
+    results = {"whole": run_trace(eng, _cut("w", tokens, [n], 0))}
+    assert not eng.graphs.graphs
+    results["portions"] = run_trace(eng, _cut("p", tokens, [4096, 2, 3000, 31, 971], 92))
+    caps = sorted(key[2] for key in eng.graphs.graphs)
+    assert caps == [8192], caps
+    sizes = [4060] + [1] * 60 + [2000] + [1] * 60 + [1920]
+    results["decoded"] = run_trace(eng, _cut("d", tokens, sizes, 92))
+    caps = sorted(key[2] for key in eng.graphs.graphs)
+    assert caps == [4096, 6144, 8192], caps
+    assert sum(g.replays for g in eng.graphs.graphs.values()) >= 92 + 212 - 4 * 3
+    rows = {name: torch.stack([res[(name[0], pos)] for pos in range(n)]) for name, res in results.items()}
+    for name, got in rows.items():
+        _check_rows(name, got, want, dtype, tol)
+    if dtype == "float32":
+        for name in ("portions", "decoded"):
+            diff = (rows[name] != rows["whole"]).any(dim=-1).nonzero().flatten()
+            assert diff.numel() == 0, f"{name} differs from the whole prompt at {diff.numel()} positions, first {int(diff[0])}"
+
+
+class _Recorder:
+    """An engine as the generation loop sees it, which keeps the logits of every step by (request,
+    position).  Every way in which the loop runs a step goes through here."""
+
+    def __init__(self, engine):
+        self.engine, self.cache, self.rows = engine, engine.cache, {}
+        self.ways = {"step": 0, "step_prepared": 0, "step_prepared_on_device": 0}
+
+    def _note(self, way, wanted, logits):
+        if logits is None:
+            return None
+        self.ways[way] += 1
+        places = [(rid, self.cache.num_tokens(rid) - n + w) for rid, n, want in wanted for w in want]
+        assert logits.shape[0] == len(places)
+        for place, row in zip(places, logits.clone()):
+            assert place not in self.rows
+            self.rows[place] = row
+        return logits
+
+    def step(self, entries):
+        return self._note("step", [(e.rid, len(e.tokens), e.want) for e in entries], self.engine.step(entries))
+
+    def prepare_decode(self):
+        return self.engine.prepare_decode()
+
+    def step_prepared(self, prepared, entries):
+        return self._note("step_prepared", [(e.rid, 1, e.want) for e in entries], self.engine.step_prepared(prepared, entries))
+
+    def step_prepared_on_device(self, prepared, rids, token_ids):
+        return self._note("step_prepared_on_device", [(rid, 1, [0]) for rid in rids],
+                          self.engine.step_prepared_on_device(prepared, rids, token_ids))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_eight_requests_at_context_8192_through_the_generation_loop(one_layer, dtype):
+    """The shape whose speed is the headline figure: eight requests with prompts of 8,152 tokens,
+    admitted and cut into portions by the scheduler under a token budget of 8,192 (the first decodes
+    while the others' prompts come in), then 40 tokens generated for each, the decode steps of all eight
+    replayed from one graph at the context cap 8,192 and launched ahead of the host.  The logits of
+    every sampled position against the plain model run over the prompt and what was generated."""
+    from torchllms_amd.engine import Engine
+    from torchllms_amd.inference.llm import GenerationLoop
+    from torchllms_amd.sampling import Sampler, SamplingParams
+
+    folder, cfg, weights = one_layer
+    batch, prompt_len, new = 8, 8152, 40
+    prompts = [random_tokens(prompt_len, ONE_LAYER["vocab_size"], 500 + i) for i in range(batch)]
+    eng = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=batch * 513, max_seqs=batch, max_model_len=8192, use_graphs=True)
+    rec = _Recorder(eng)
+    loop = GenerationLoop(rec, Sampler(), max_num_seqs=batch, max_num_batched_tokens=8192, max_model_len=8192)
+    params = [SamplingParams(temperature=0.0, max_new_tokens=new, stop_token_ids=(), seed=i) for i in range(batch)]
+    requests = loop.run(prompts, params)
+    assert all(len(r.output) == new for r in requests)
+    eng.cache.check_invariants()
+    graph = eng.graphs.graphs.get((batch, batch, 8192, False))
+    assert graph is not None and graph.replays >= 20, {k: g.replays for k, g in eng.graphs.graphs.items()}
+    assert rec.ways["step_prepared_on_device"] >= 15, rec.ways
+    assert len(rec.rows) == batch * new
+    for i, r in enumerate(requests):
+        tokens = prompts[i] + list(r.output)
+        want = _plain_on_gpu(weights, cfg, tokens, torch.float32)
+        tol = 2 * (_plain_on_gpu(weights, cfg, tokens, torch.bfloat16) - want).abs().amax(dim=-1) + 1e-3 if dtype == "bfloat16" else None
+        places = [pos for (rid, pos) in rec.rows if rid == r.rid]
+        assert sorted(places) == list(range(prompt_len - 1, prompt_len + new - 1)), (i, sorted(places)[:3])
+        got = torch.stack([rec.rows[(r.rid, pos)].cpu() for pos in sorted(places)])
+        _check_rows(f"request {i}", got, want[prompt_len - 1 : prompt_len + new - 1], dtype, None if tol is None else tol[prompt_len - 1 : prompt_len + new - 1])
+        # greedy: each generated token is the plain model's choice wherever that choice is clear
+        top2 = want[prompt_len - 1 : prompt_len + new - 1].topk(2, dim=-1)
+        margin = 20 * FP32_ATOL if dtype == "float32" else 2 * tol[prompt_len - 1 : prompt_len + new - 1]
+        clear = (top2.values[:, 0] - top2.values[:, 1]) > margin
+        assert clear.any()
+        assert torch.equal(torch.tensor(r.output)[clear], top2.indices[:, 0][clear]), f"request {i}"
