@@ -306,6 +306,24 @@ def test_sizes_no_kernel_takes_are_refused_when_the_engine_is_built():
     del eng
 
 
+def test_a_context_longer_than_the_models_positions_is_refused_unless_asked_for(cases):
+    """The reference's table of angles ends at ``max_position_embeddings`` and a longer request fails
+    there (reference: networks.py:325-327).  Here angles come from positions, so it would run: the
+    engine refuses such a ``max_model_len`` unless told to go beyond, and ``LLM`` takes its ``max_len``
+    as a bound beside the model's own."""
+    from torchllms_amd.engine import Engine, StepEntry
+    from torchllms_amd.inference import LLM
+
+    folder = cases["A"].folder  # 128 positions
+    with pytest.raises(ValueError, match="max_model_len=129 exceeds the 128 positions"):
+        Engine.from_folder(folder, dtype="float32", max_seqs=1, max_model_len=129)
+    assert Engine.from_folder(folder, dtype="float32", max_seqs=1).max_model_len == 128
+    eng = Engine.from_folder(folder, dtype="float32", max_seqs=1, max_model_len=140, beyond_max_positions=True)
+    eng.admit("r")
+    assert eng.step([StepEntry("r", random_tokens(135, 256, 1), [134])]).shape == (1, 256)
+    assert LLM(str(folder), precision="float32", max_len=4096, max_bsz=1).max_len == 128
+
+
 def test_a_step_that_fails_leaves_nothing_behind(cases):
     """A step whose forward pass raises books nothing: the pages it took go back, the request is
     where it was, and the next step is planned afresh."""

@@ -131,26 +131,29 @@ def test_preparing_the_next_step_ahead_changes_no_token(model_b, precision):
 def test_steps_launched_ahead_cope_with_requests_that_end(model_b, precision):
     """A decode step that is launched with the sampled tokens still on the device is wrong for a
     request that ends on that very token.  Many requests with a fifth of the vocabulary as stop
-    tokens, four at a time with others waiting, greedy and sampled, with ample pages and with few:
-    the tokens and stop reasons are those of the loop that waits for the tokens before every
-    step, and every page comes back."""
+    tokens, four at a time with others waiting, greedy and sampled, with ample pages; and with a
+    twenty-third of it and so few pages that running requests are preempted for want of pages, in
+    the loop that launches ahead as in the other: the tokens and stop reasons are those of the loop
+    that waits for the tokens before every step, and every page comes back."""
     from torchllms_amd.inference import LLM
 
     folder, cfg, _ = model_b
     vocab = cfg["vocab_size"]
     prompts = [random_tokens(3 + (11 * i) % 40, vocab, 500 + i) for i in range(14)]
-    stops = list(range(0, vocab, 5))
     for pages, temperature in ((None, 0.0), (None, 1.3), (16, 1.3)):
         kw = dict(num_pages=pages) if pages else {}
+        stops = list(range(0, vocab, 23 if pages else 5))
         llm = LLM(str(folder), precision=precision, max_len=120, max_bsz=4, page_size=8, max_num_batched_tokens=24, **kw)
         llm.look_ahead = False
         want = llm.generate(prompt_token_ids=prompts, temperature=temperature, max_new_tokens=40, seed=11, stop_token_ids=stops)
         assert sum(r.stop_reason is not None for r in want) >= 5 and llm.last_stats["launched_ahead"] == 0
+        assert not pages or llm.last_stats["preemptions"] > 0
         llm.look_ahead = True
         got = llm.generate(prompt_token_ids=prompts, temperature=temperature, max_new_tokens=40, seed=11, stop_token_ids=stops)
         assert [r.token_ids for r in got] == [r.token_ids for r in want], (pages, temperature)
         assert [r.stop_reason for r in got] == [r.stop_reason for r in want]
         assert llm.last_stats["launched_ahead"] > 0
+        assert not pages or llm.last_stats["preemptions"] > 0
         llm.engine.cache.check_invariants()
         assert llm.engine.cache.live == [] and llm.engine.cache.free_pages() == llm.engine.cache.pools[0].num_pages
 

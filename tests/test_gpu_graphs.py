@@ -84,8 +84,8 @@ def test_prepared_decode_steps_match_plain_steps(tmp_path, dtype):
 
     cfg = TINY["B"]
     folder = make_folder(tmp_path / "m", cfg, seed=33, dtype=torch.bfloat16, sharpen=True)
-    plain = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=4, max_model_len=1100)
-    ahead = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=4, max_model_len=1100)
+    plain = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=4, max_model_len=1100, beyond_max_positions=True)
+    ahead = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=4, max_model_len=1100, beyond_max_positions=True)
     vocab = cfg["vocab_size"]
     toks = {r: random_tokens(600, vocab, 900 + i) for i, r in enumerate("abc")}
     start = {"a": 470, "b": 23, "c": 7}

@@ -4,15 +4,16 @@ another run's cache.  It is registered, built from random weights and stepped th
 in portions and mixed batches without any change to the framework's files, and compared with a
 plain whole-sequence computation written here."""
 
+import json
 from dataclasses import dataclass
-from typing import Dict, Tuple
+from typing import Dict
 
 import pytest
 import torch
 import torch.nn.functional as F
 
 from . import schedules
-from .helpers import random_tokens
+from .helpers import random_tokens, read_folder
 from .plain import llama as plain
 from .test_gpu_engine import run_trace
 
@@ -23,8 +24,15 @@ HIDDEN, STATE, VOCAB, HEADS, KV, DH, FFN, WINDOW, WINDOW_PAGE = 40, 24, 97, 4, 2
 
 @dataclass(frozen=True)
 class ToyConfig:
+    """(Nothing but what the toy models need: no ``architectures``, no end-of-sequence id, none of the
+    attributes of the framework's own configuration.)"""
+
     decay: float = 0.8
-    architectures: Tuple[str, ...] = ("ToyHybridForCausalLM",)
+    end_token: int = -1  # the token id that ends a generation, if any
+
+
+def _config_from_dict(d):
+    return ToyConfig(**{k: v for k, v in d.items() if k != "architectures"})
 
 
 def _register():
@@ -88,7 +96,7 @@ def _register():
                      "mixer.w_in.weight", "mixer.w_out.weight"]
         return [NameRule(n, n) for n in names] + [NameRule("layers.{}." + n, "layers.{}." + n) for n in per_layer]
 
-    return register_architecture(ArchSpec("ToyHybridForCausalLM", lambda d: ToyConfig(**d), spec, rules))
+    return register_architecture(ArchSpec("ToyHybridForCausalLM", _config_from_dict, spec, rules, stop_token_ids=lambda cfg: [cfg.end_token] if cfg.end_token >= 0 else []))
 
 
 def plain_toy(w: Dict[str, torch.Tensor], cfg: ToyConfig, tokens):
@@ -173,6 +181,43 @@ def test_toy_architecture_is_registered_built_and_stepped():
     eng.free("w")
 
 
+def test_toy_architecture_generates_through_the_host_path(tmp_path):
+    """The same toy architecture from a model folder through ``LLM.generate``: the folder is written by
+    the random-weights mode, config.json names the architecture, the scheduler and the sampling run as
+    for any model, and generation stops on the token id that the architecture gives for its
+    configuration.  Nothing on the way asks the configuration for what only the framework's own has."""
+    from torchllms_amd.inference import LLM
+    from torchllms_amd.weights import write_model_folder
+
+    arch = _register()
+    cfg = ToyConfig(decay=0.7)
+    folder = write_model_folder(tmp_path / "toy", cfg, seed=4, dtype=torch.float32, norm_jitter=0.1, arch=arch)
+    assert json.loads((folder / "config.json").read_text()) == {"decay": 0.7, "end_token": -1, "architectures": ["ToyHybridForCausalLM"]}
+    _, w = read_folder(folder)
+    prompts = [random_tokens(n, VOCAB, 40 + n) for n in (5, 23, 2)]
+    kw = dict(precision="float32", max_len=200, max_bsz=2, page_size=4, max_num_batched_tokens=16)
+    llm = LLM(str(folder), **kw)
+    assert llm.eos_ids == [] and llm.engine.graphs is None  # (the toy mixer's launches depend on the plan)
+    free = llm.generate(prompt_token_ids=prompts, max_new_tokens=30)
+    for p, r in zip(prompts, free):
+        toks = list(p)
+        for _ in range(30):
+            toks.append(int(plain_toy(w, cfg, toks)[-1].argmax()))
+        assert r.token_ids == toks[len(p):] and r.stop_reason is None
+    # the same weights with an end token in the configuration: one that the second request generates
+    end = free[1].token_ids[7]
+    folder = write_model_folder(tmp_path / "toy_end", ToyConfig(decay=0.7, end_token=end), seed=4, dtype=torch.float32, norm_jitter=0.1, arch=arch)
+    llm = LLM(str(folder), **kw)
+    assert llm.eos_ids == [end]
+    stopped = llm.generate(prompt_token_ids=prompts, max_new_tokens=30)
+    assert stopped[1].stop_reason == end and len(stopped[1].token_ids) <= 8
+    for a, b in zip(free, stopped):
+        cut = a.token_ids.index(end) + 1 if end in a.token_ids else 30
+        assert b.token_ids == a.token_ids[:cut] and b.stop_reason == (end if end in a.token_ids else None)
+    llm.engine.cache.check_invariants()
+    assert llm.engine.cache.live == []
+
+
 def _register_windowed():
     """Two attention layers from the framework's own parts, the second with a window of 20 keys in pages of
     8: every part is fit for a recorded graph, so decode steps of this model are replayed and prepared ahead."""
@@ -200,7 +245,7 @@ def _register_windowed():
                      "mixer.wq.weight", "mixer.wk.weight", "mixer.wv.weight", "mixer.wo.weight"]
         return [NameRule(n, n) for n in ("embed.weight", "final_norm.weight")] + [NameRule("layers.{}." + n, "layers.{}." + n) for n in per_layer]
 
-    arch = register_architecture(ArchSpec("ToyWindowedForCausalLM", lambda d: ToyConfig(**d), spec, rules))
+    arch = register_architecture(ArchSpec("ToyWindowedForCausalLM", _config_from_dict, spec, rules))
     return arch, window
 
 
@@ -213,7 +258,7 @@ def test_windowed_layers_decode_through_graphs_and_prepared_steps():
     from torchllms_amd.weights import random_tensors
 
     arch, window = _register_windowed()
-    cfg = ToyConfig(architectures=("ToyWindowedForCausalLM",))
+    cfg = ToyConfig()
     w = random_tensors(Model(arch.model_spec(cfg)).param_specs(), seed=5, dtype=torch.float32, norm_jitter=0.1)
     for name in w:
         if name.endswith(("wq.weight", "wk.weight")):

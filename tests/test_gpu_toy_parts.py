@@ -27,7 +27,6 @@ HIDDEN, VOCAB, HEADS, KV, DH, ROT, FFN, EXPERTS, SANDWICH_SCALE, WIDE_PAGE = 48,
 @dataclass(frozen=True)
 class ToyConfig:
     eps: float = 1e-4
-    architectures: Tuple[str, ...] = ("ToyRoutedForCausalLM",)
 
 
 def toy_frequencies() -> torch.Tensor:
@@ -179,7 +178,7 @@ def _register():
         per_layer += [f"ffn.experts.{e}.{m}.weight" for e in range(EXPERTS) for m in ("up", "down")]
         return [NameRule(n, n) for n in names] + [NameRule("layers.{}." + n, "layers.{}." + n) for n in per_layer]
 
-    return register_architecture(ArchSpec("ToyRoutedForCausalLM", lambda d: ToyConfig(**d), spec, rules))
+    return register_architecture(ArchSpec("ToyRoutedForCausalLM", lambda d: ToyConfig(**{k: v for k, v in d.items() if k != "architectures"}), spec, rules))
 
 
 def plain_toy(w: Dict[str, torch.Tensor], cfg: ToyConfig, tokens):

@@ -102,3 +102,40 @@ def test_libraries_built_in_the_tree_match_their_sources():
     from torchllms_amd.kernels import build
 
     assert build.stale_libraries() == []
+
+
+def test_launch_plans_take_the_device_s_own_figures(monkeypatch):
+    """Compute units and LDS size come from the device (the target's published figures where there is
+    no GPU, as here): a GPU with half the CUs gets half the splits, one with less LDS fewer buffers."""
+    from torchllms_amd.kernels import lib
+
+    assert lib.device_facts() == (256, 160 * 1024)
+    assert ops.plan_decode_splits(1, 8, 8192) == (256, 32) and ops.wide_fits(64, 2, 3) and ops.rmsnorm_max_hidden() == 40704
+    monkeypatch.setattr(lib, "_facts", (128, 64 * 1024))
+    assert ops.plan_decode_splits(1, 8, 8192) == (256, 32)  # (the shortest split allowed either way)
+    assert ops.plan_decode_splits(4, 8, 8192) == (1024, 8)  # 256 blocks at a time instead of 512
+    assert not ops.wide_fits(64, 2, 3) and ops.wide_fits(32, 1, 2) and ops.rmsnorm_max_hidden() == 16128
+
+
+def test_a_head_size_without_matrix_core_kernels_is_reported_once(caplog):
+    """A bfloat16 model whose head size only the plain attention kernel takes runs, right and slowly:
+    the attention part says so, once per shape, when the engine asks it about its sizes."""
+    import logging
+
+    from torchllms_amd.config.spec import PartSpec
+    from torchllms_amd.parts import MIXERS
+
+    def part(head_dim, heads=6, kv=3):
+        return MIXERS.build(PartSpec("attention", dict(
+            hidden_size=96, num_heads=heads, num_kv_heads=kv, head_dim=head_dim, qkv_bias=False, softmax_scale=head_dim ** -0.5, window=0,
+            position=PartSpec("rope", dict(head_dim=head_dim, rotary_dim=head_dim, theta=100.0, scaling=None)))))
+
+    with caplog.at_level(logging.WARNING, logger="torchllms_amd"):
+        part(64).check_sizes(torch.bfloat16)
+        part(96).check_sizes(torch.float32)
+        assert not caplog.records
+        part(96).check_sizes(torch.bfloat16)
+        part(96).check_sizes(torch.bfloat16)
+        assert len(caplog.records) == 1 and "head size 96" in caplog.text and "decode steps and prompts run the plain kernel" in caplog.text
+        part(256, heads=16, kv=1).check_sizes(torch.bfloat16)  # 16 query heads per kv head: prompts only
+        assert len(caplog.records) == 2 and "; decode steps run the plain kernel" in caplog.records[1].getMessage()

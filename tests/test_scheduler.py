@@ -321,10 +321,11 @@ class AheadEngine(FakeEngine):
     def step(self, entries):
         out = super().step(entries)
         self._decoded = [e.rid for e in entries] if all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries) else None
+        self._epoch = self.cache.epoch
         return out
 
     def prepare_decode(self):
-        if self._decoded is None:
+        if self._decoded is None or self._epoch != self.cache.epoch:  # (requests came or went since)
             return None
         need = sum(self.cache.new_pages_needed(r, 1)[0] for r in self._decoded)
         if need > self.cache.free_pages():
@@ -394,3 +395,163 @@ def test_prepared_steps_are_used_and_dropped():
     assert len(eng.calls) == 12
     assert eng.used == 11 - 2
     assert eng.prepared == eng.used + 1  # one was made in vain
+
+
+# ----------------------------------------------------------------------------- steps launched ahead of the host
+class LaunchAheadEngine(AheadEngine):
+    """A fake engine that also runs a prepared step before the host has seen the tokens it is fed
+    (they are "on the device": a tensor).  Like the real one it then runs a row for every request
+    of the preparation, also for one that ends on that very token."""
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.launched = 0
+        self.fed = []  # per launched step: (rid, position, token id fed)
+
+    def step_prepared_on_device(self, prepared, rids, token_ids):
+        from torchllms_amd.engine import StepEntry
+
+        known, epoch = prepared
+        if epoch != self.cache.epoch or list(rids) != known or token_ids.numel() != len(known):
+            return None
+        self.launched += 1
+        self.used += 1
+        self.fed.append([(rid, self.cache.num_tokens(rid), int(t)) for rid, t in zip(rids, token_ids)])
+        return self.step([StepEntry(rid, [int(t)], [0]) for rid, t in zip(rids, token_ids)])
+
+
+def _run(make, sampler, look_ahead, prompts, params, live=4, budget=64, chunk=None, **engine_kw):
+    eng = make(**engine_kw)
+    loop = GenerationLoop(eng, sampler, live, budget, 256, chunk, look_ahead=look_ahead)
+    steps = []
+    loop.launched_by_step = []  # steps launched ahead so far, as each step is booked
+
+    def on_step(plan):
+        steps.append([(e.request.rid[2], len(e.tokens)) for e in plan.entries])
+        loop.launched_by_step.append(loop.stats["launched_ahead"])
+
+    reqs = loop.run(prompts, params, on_step=on_step)
+    assert eng.cache.live == [] and all(eng.cache.free_pages(g) == p.num_pages for g, p in enumerate(eng.cache.pools))
+    eng.cache.check_invariants()
+    return reqs, eng, loop, steps
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_steps_launched_ahead_give_the_same_tokens(seed):
+    _launched_ahead_against_waiting(seed)
+
+
+def _launched_ahead_against_waiting(seed):
+    """Random workloads (stop tokens, budgets, late joiners, tight pools, preemptions) through the
+    loop that launches the prepared step with the tokens still on the device, against the loop that
+    waits before every step: the same tokens and stop reasons, every token fed ahead is the one
+    that was sampled, and a request that ended on the token it was fed leaves nothing behind."""
+    rng = random.Random(700 + seed)
+    n = rng.randint(3, 10)
+    prompts = [[1] * rng.randint(1, 30) for _ in range(n)]
+    news = [rng.randint(1, 30) for _ in range(n)]
+    stops = [(rng.randrange(VOCAB),) if rng.random() < 0.6 else () for _ in range(n)]
+    page = rng.choice([2, 4, 8])
+    longest = max(len(p) + m for p, m in zip(prompts, news))
+    kw = dict(num_pages=-(-longest // page) + rng.randint(0, 6), page_size=page, max_seqs=rng.randint(1, 4))
+    live, budget, chunk = rng.randint(1, 4), rng.choice([4, 5, 16, 64]), rng.choice([None, 3, 7])
+    params = [SamplingParams(max_new_tokens=m, stop_token_ids=s) for m, s in zip(news, stops)]
+    want, _, base, _ = _run(FakeEngine, greedy, False, prompts, params, live, budget, chunk, **kw)
+    got, eng, loop, _ = _run(LaunchAheadEngine, LaunchingSampler(), True, prompts, params, live, budget, chunk, **kw)
+    assert [r.output for r in got] == [r.output for r in want]
+    assert [r.stop_reason for r in got] == [r.stop_reason for r in want]
+    assert loop.stats["launched_ahead"] == eng.launched and loop.stats["prepared_steps"] == eng.used
+    for step in eng.fed:
+        for rid, pos, tok in step:
+            assert tok == pos % VOCAB  # the token the fake model gives for the position before
+    return loop.stats["launched_ahead"], loop.scheduler.stats["preemptions"], base.scheduler.stats["preemptions"]
+
+
+def test_the_random_workloads_launch_ahead_and_preempt():
+    """(The premise of the test above: among its workloads are some that launch steps ahead and
+    preempt requests in the same run.)"""
+    seen = [_launched_ahead_against_waiting(seed) for seed in range(12)]
+    assert sum(1 for launched, preempted, _ in seen if launched > 3 and preempted > 0) >= 2, seen
+    assert sum(launched for launched, _, _ in seen) > 50
+
+
+def test_a_request_that_ends_on_the_token_it_was_fed_ahead():
+    """Two requests decode side by side, steps launched ahead; the first ends on its stop token while
+    the step that feeds that token to it is already running.  Its row is dropped, the other request's
+    row of that step counts, and a third request that waited takes the seat one step later than in
+    the loop that waits for the tokens."""
+    prompts = [[1] * 3, [1] * 5, [1] * 2]
+    params = [SamplingParams(max_new_tokens=12, stop_token_ids=(9,)), SamplingParams(max_new_tokens=12), SamplingParams(max_new_tokens=4)]
+    want, _, _, base_steps = _run(FakeEngine, greedy, False, prompts, params, live=2, num_pages=32, page_size=4, max_seqs=2)
+    got, eng, loop, steps = _run(LaunchAheadEngine, LaunchingSampler(), True, prompts, params, live=2, num_pages=32, page_size=4, max_seqs=2)
+    assert [r.output for r in got] == [r.output for r in want]
+    assert got[0].output == [3, 4, 5, 6, 7, 8, 9] and got[0].stop_reason == 9 and len(got[1].output) == 12
+    # request 0 was fed its stop token (9, at position 9) by a step that was launched ahead
+    assert any((rid[2], pos, tok) == (0, 9, 9) for step in eng.fed for rid, pos, tok in step)
+    # that step counts for request 1 alone
+    first = lambda all_steps: next(i for i, s in enumerate(all_steps) if any(r == 2 for r, _ in s))
+    assert [0] not in [[r for r, _ in s] for s in steps] and [(1, 1)] in steps
+    assert first(steps) == first(base_steps) + 1
+    assert loop.stats["launched_ahead"] >= 8
+
+
+def test_every_request_ends_on_the_token_that_was_fed_ahead():
+    """Both requests end on the same step's token while the next step is already running for both:
+    nothing of that step counts, nothing is left in the cache, and the loop ends."""
+    prompts = [[1] * 4, [1] * 4]
+    params = [SamplingParams(max_new_tokens=20, stop_token_ids=(11,)) for _ in prompts]
+    got, eng, loop, steps = _run(LaunchAheadEngine, LaunchingSampler(), True, prompts, params, live=2, num_pages=16, page_size=4, max_seqs=2)
+    assert [r.output for r in got] == [list(range(4, 12))] * 2 and [r.stop_reason for r in got] == [11, 11]
+    assert eng.fed[-1] == [(r.rid, 11, 11) for r in got]  # the step in vain
+    assert len(steps) == len(eng.calls) - 1  # ... which the loop never booked
+
+
+def test_when_a_waiting_request_could_join_although_nobody_ends():
+    """The rule that keeps steps from being launched ahead of the scheduler: a request that waits
+    could be admitted while everybody else decodes on only if a seat is free and pages are there or
+    may come back (a window gives pages back during decoding; nothing else does)."""
+    def state(window, num_pages, max_seqs, prompts):
+        eng = FakeEngine(num_pages=num_pages, page_size=4, max_seqs=max_seqs, window=window)
+        sched = Scheduler(eng.cache, max_seqs, 64, 256)
+        for i, p in enumerate(prompts):
+            sched.add(i, [1] * p, SamplingParams(max_new_tokens=8))
+        plan = sched.schedule()
+        eng.step(plan.step_entries())
+        sched.update(plan, [5] * sum(e.samples for e in plan.entries))
+        return sched
+
+    assert not state(0, 16, 2, [8, 8]).may_admit_before_a_request_ends()  # nobody waits
+    assert not state(0, 16, 2, [8, 8, 8]).may_admit_before_a_request_ends()  # no seat
+    sched = state(0, 4, 3, [8, 8, 8])
+    assert len(sched.running) == 2 and sched.waiting and sched.cache.free_pages() == 0
+    assert not sched.may_admit_before_a_request_ends()  # a seat, but no page, and none can come back
+    sched = state(8, 4, 3, [8, 8, 8])
+    assert len(sched.running) == 2 and sched.waiting and sched.cache.free_pages() == 0
+    assert sched.may_admit_before_a_request_ends()  # the window will give pages back
+    sched = state(0, 5, 3, [8, 8, 8])
+    assert len(sched.running) == 3 and not sched.may_admit_before_a_request_ends()  # it has joined already
+
+
+def test_nothing_is_launched_ahead_while_a_waiting_request_could_join():
+    """While that rule says that somebody could join, the loop asks the scheduler before every step
+    and launches nothing ahead: the steps are those of the loop that waits for the tokens.  A third
+    request that waits for pages in a cache without a window, a seat being free, can only get them
+    from a request that ends, and steps are launched ahead while it waits."""
+    prompts = [[1] * 17, [1] * 17, [1] * 6]
+    params = [SamplingParams(max_new_tokens=12), SamplingParams(max_new_tokens=12), SamplingParams(max_new_tokens=30)]
+    kw = dict(live=3, budget=64, num_pages=4, page_size=16, max_seqs=3)  # two pages each for the first two: none is left
+    want, _, _, base_steps = _run(FakeEngine, greedy, False, prompts, params, **kw)
+    got, eng, loop, steps = _run(LaunchAheadEngine, LaunchingSampler(), True, prompts, params, **kw)
+    assert [r.output for r in got] == [r.output for r in want]
+    joined = next(i for i, s in enumerate(steps) if any(r == 2 for r, _ in s))
+    assert loop.launched_by_step[joined] >= 5, (steps[:joined], loop.launched_by_step)
+
+    eng = LaunchAheadEngine(num_pages=4, page_size=16, max_seqs=3)
+    loop = GenerationLoop(eng, LaunchingSampler(), 3, 64, 256)
+    loop.scheduler.may_admit_before_a_request_ends = lambda: bool(loop.scheduler.waiting)
+    steps = []
+    got = loop.run(prompts, params, on_step=lambda plan: steps.append(([(e.request.rid[2], len(e.tokens)) for e in plan.entries], loop.stats["launched_ahead"])))
+    assert [r.output for r in got] == [r.output for r in want]
+    joined = next(i for i, (s, _) in enumerate(steps) if any(r == 2 for r, _ in s))
+    assert [s for s, _ in steps[: joined + 1]] == base_steps[: joined + 1]
+    assert steps[joined][1] == 0 and loop.stats["launched_ahead"] > 10 and loop.stats["prepared_steps"] > loop.stats["launched_ahead"] + 5

@@ -3,6 +3,7 @@ from .registry import (
     ARCHITECTURES,
     ArchSpec,
     architecture_name,
+    architecture_of,
     get_architecture,
     load_config,
     register_architecture,
@@ -20,6 +21,7 @@ __all__ = [
     "PartSpec",
     "RopeScaling",
     "architecture_name",
+    "architecture_of",
     "get_architecture",
     "llama_model_spec",
     "load_config",

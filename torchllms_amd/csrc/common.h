@@ -21,6 +21,15 @@ int tl_fail(int code, const char* fmt, ...);
 // Checks hipGetLastError() after a launch.
 int tl_check_launch(const char* what);
 
+// What the current device says of itself (hipGetDeviceProperties, read once per device and process):
+// its compute units and the bytes of LDS a block may use.  Launch rules and size checks take these,
+// not a literal of the GPU they were first written for.
+struct TlDeviceFacts {
+  int compute_units;
+  int lds_bytes;
+};
+const TlDeviceFacts& tl_device_facts();
+
 #define TL_REQUIRE(cond, ...)                          \
   do {                                                 \
     if (!(cond)) return tl_fail(TL_ERR_ARG, __VA_ARGS__); \

@@ -22,7 +22,27 @@ int tl_check_launch(const char* what) {
   return TL_OK;
 }
 
+const TlDeviceFacts& tl_device_facts() {
+  constexpr int kMaxDevices = 64;
+  static TlDeviceFacts facts[kMaxDevices];  // zero until read; a race reads the same values twice
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+  if (facts[dev].compute_units == 0) {
+    hipDeviceProp_t prop;
+    TlDeviceFacts f = {256, 160 * 1024};  // MI355X, should the device refuse to answer
+    if (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) {
+      f.compute_units = prop.multiProcessorCount;
+      f.lds_bytes = (int)prop.sharedMemPerBlock;
+    }
+    facts[dev] = f;
+  }
+  return facts[dev];
+}
+
 TL_EXPORT const char* tl_last_error() { return g_last_error; }
+// The same figures for the host side's launch plans.
+TL_EXPORT int tl_device_compute_units() { return tl_device_facts().compute_units; }
+TL_EXPORT int tl_device_lds_bytes() { return tl_device_facts().lds_bytes; }
 TL_EXPORT int tl_abi_version() { return 1; }
 
 // ----------------------------------------------------------------------------- embedding
@@ -186,7 +206,7 @@ TL_EXPORT int tl_rmsnorm(const void* x, const void* delta, const int32_t* rows, 
                          int dtype, hipStream_t stream) {
   TL_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm: bad sizes n_rows=%d hidden=%d", n_rows, hidden);
   TL_REQUIRE(!(rows && h_out), "rmsnorm: h_out cannot be combined with a row gather");
-  TL_REQUIRE((size_t)hidden * sizeof(float) <= 160 * 1024 - 1024, "rmsnorm: hidden=%d does not fit LDS", hidden);
+  TL_REQUIRE((size_t)hidden * sizeof(float) <= (size_t)tl_device_facts().lds_bytes - 1024, "rmsnorm: hidden=%d does not fit LDS", hidden);
   if (n_rows == 0) return TL_OK;
   const size_t lds = (size_t)hidden * sizeof(float);
   const int vec = dtype == TL_F32 ? 4 : 8;

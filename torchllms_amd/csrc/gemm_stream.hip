@@ -300,12 +300,13 @@ int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M,
   TL_REQUIRE(out_dtype == TL_BF16 || out_dtype == TL_F32, "gemm_stream: out_dtype must be 0 or 1");
   if (M == 0) return TL_OK;
   if (waves == 0) {
-    // enough waves to keep loads in flight on 256 CUs: about 4096 in all, at least two steps each
+    // enough waves to keep loads in flight on every CU: about 16 a CU (4,096 on 256 CUs), at least two steps each
+    const int enough = 16 * tl_device_facts().compute_units;
     const int cols = epi == kGatedHalf ? kStrip / 2 : kStrip;
     const int strips = (N + cols - 1) / cols;
     const int steps = (K + kStepK - 1) / kStepK;
     waves = 1;
-    while (waves < 8 && strips * waves < 4096 && steps >= 2 * waves * 2) waves *= 2;
+    while (waves < 8 && strips * waves < enough && steps >= 2 * waves * 2) waves *= 2;
   }
   TL_REQUIRE(waves == 1 || waves == 2 || waves == 4 || waves == 8, "gemm_stream: waves must be 1, 2, 4 or 8");
   const bf16_t* a = (const bf16_t*)A;

@@ -314,9 +314,12 @@ int launch_kernel(const Launch& l) {
 
 template <int MC, int NCW, int STAGES>
 int launch_stages(const Launch& l) {
-  if constexpr (Shape<MC, NCW, STAGES>::kLdsBytes > 160 * 1024) {
+  if constexpr (Shape<MC, NCW, STAGES>::kLdsBytes > 160 * 1024) {  // (more than gfx950 has: not compiled at all)
     return tl_fail(TL_ERR_UNSUPPORTED, "gemm_wide: %d buffers for %d rows and %d strips per wave do not fit into LDS", STAGES, 16 * MC, NCW);
   } else {
+    if (Shape<MC, NCW, STAGES>::kLdsBytes > tl_device_facts().lds_bytes)
+      return tl_fail(TL_ERR_UNSUPPORTED, "gemm_wide: %d buffers for %d rows and %d strips per wave take %d bytes of LDS, this device has %d",
+                     STAGES, 16 * MC, NCW, (int)Shape<MC, NCW, STAGES>::kLdsBytes, tl_device_facts().lds_bytes);
     if (l.gated) return launch_kernel<MC, NCW, STAGES, bf16_t, true>(l);
     if (l.out_dtype == TL_BF16) return launch_kernel<MC, NCW, STAGES, bf16_t, false>(l);
     return launch_kernel<MC, NCW, STAGES, float, false>(l);

@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, OutOfPages, group_layers
-from ..config.registry import ArchSpec, get_architecture, load_config
+from ..config.registry import ArchSpec, architecture_of, load_config
 from ..parts.model import Model
 from ..weights.loader import load_weights
 from ..weights.random_init import random_tensor, random_tensors
@@ -73,6 +73,7 @@ class Engine:
         use_graphs: bool = True,
         tune_kernels: bool = True,
         kernel_table=None,
+        beyond_max_positions: bool = False,
     ):
         """``tensors``: the model's tensors under the parts' own names, on ``device``.
         Pool size: room for ``num_pages`` pages of ``page_size`` tokens, else what ``kv_memory_gb``
@@ -86,7 +87,10 @@ class Engine:
         JSON file of one) fills the table first; ``tune_kernels`` then measures what the table does
         not hold yet.  Kernels differ in rounding, so two processes agree bit for bit in bfloat16
         only when they run from the same table; with ``tune_kernels=False`` and no table every shape
-        follows a fixed rule of sizes (``ops.linear_choice``)."""
+        follows a fixed rule of sizes (``ops.linear_choice``).
+
+        ``max_model_len`` (default: the configuration's maximum of positions) may exceed that
+        maximum only with ``beyond_max_positions``."""
         self.device = require_gpu(device)
         self.arch = arch
         self.config = config
@@ -99,6 +103,14 @@ class Engine:
             raise ValueError(f"page_size must be positive, got {page_size}")
         self.model.bind(tensors)
         self.vocab_size = self.spec.vocab_size
+        # the reference's table of rotation angles ends at the configuration's maximum and a longer
+        # request fails there (reference: networks.py:325-327); angles are computed from positions
+        # here, so a longer context would run, on positions the model never saw: only when asked
+        if max_model_len is not None and max_model_len > self.spec.max_positions and not beyond_max_positions:
+            raise ValueError(
+                f"max_model_len={max_model_len} exceeds the {self.spec.max_positions} positions of the model's "
+                "configuration; pass beyond_max_positions=True to run longer contexts all the same"
+            )
         self.max_model_len = int(max_model_len or self.spec.max_positions)
         self.page_size = page_size
         from ..kernels import ops
@@ -177,12 +189,12 @@ class Engine:
 
     @classmethod
     def from_random(cls, config, seed: int = 0, dtype="bfloat16", device="cuda:0", norm_jitter: float = 0.0,
-                    draw_on_device: bool = False, **kw) -> "Engine":
+                    draw_on_device: bool = False, arch: Optional[ArchSpec] = None, **kw) -> "Engine":
         """Random weights without a folder: same values as ``write_model_folder`` with this seed
         when drawn on the CPU; ``draw_on_device`` draws on the GPU instead (large models)."""
         device = require_gpu(device)
         dtype = parse_dtype(dtype)
-        arch = get_architecture(config.architectures[0])
+        arch = arch or architecture_of(config)
         model = Model(arch.model_spec(config))
         model.check_sizes(dtype)
         expected = model.param_specs()

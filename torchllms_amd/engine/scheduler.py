@@ -145,6 +145,18 @@ class Scheduler:
     def has_work(self) -> bool:
         return bool(self.waiting or self.running)
 
+    def may_admit_before_a_request_ends(self) -> bool:
+        """Could a request that waits be admitted while the running ones all go on decoding?  A
+        seat must be free for it, and if it waits for pages, pages must be able to come back
+        meanwhile: only a group with a window gives pages back while its requests decode; without
+        one, the pages that are free now are all it can hope for.  (Whoever runs decode steps
+        without asking ``schedule`` may do so while this is False.)"""
+        if not self.waiting or len(self.running) >= self.max_num_seqs or self.cache.free_slots == 0:
+            return False
+        if any(g.window > 0 for g in self.cache.groups):
+            return True
+        return all(pool.free_count >= p for pool, p in zip(self.cache.pools, self.cache.pages_for_new_request(1)))
+
     def _most_pages_held(self, group: int, n_tokens: int) -> int:
         """The pages of ``group`` that a request of ``n_tokens`` cannot do without.  A group that
         keeps every key needs them all; a group with a window gives pages back as the window passes

@@ -58,7 +58,11 @@ class GenerationLoop:
         request can reach its token budget with the sampled token, so the step is wrong only for a
         request that ends on a stop token: its row is dropped, the other rows are the step that
         the scheduler would have planned for them (one token each, pages taken by the
-        preparation), and requests that wait are admitted a step later."""
+        preparation).  A step launched ahead is not put before the scheduler, so it is launched
+        only while the scheduler could admit nobody anyway unless a request ends (nobody waits, or
+        no seat is free, or pages are short and no layer gives pages back while it decodes): a
+        request that waits is then admitted one step later than it would have been only when a
+        request ended on the token that the step ahead was fed."""
         from ..engine.scheduler import ScheduledEntry, StepPlan
 
         sched = self.scheduler
@@ -90,7 +94,7 @@ class GenerationLoop:
                     pending = launch(logits, [r.params for r in sampling], counters)
                     arriving = self._send_home(pending) if launch_ahead is not None else None
                     prepared = prepare()  # the GPU is busy with the step meanwhile
-                    if prepared is not None and arriving is not None:
+                    if prepared is not None and arriving is not None and not sched.may_admit_before_a_request_ends():
                         next_logits = launch_ahead(prepared, [e.request.rid for e in plan.entries], pending)
                     if next_logits is not None:
                         prepared = None  # used
@@ -127,7 +131,10 @@ class GenerationLoop:
         import torch
 
         n = pending.numel()
-        if self._host_tokens is None or self._host_tokens.numel() < n:
+        if not pending.is_cuda:  # an engine on the host (the tests' fake ones): nothing travels
+            self._host_tokens = pending
+            return _ARRIVED
+        if self._host_tokens is None or self._host_tokens.numel() < n or not self._host_tokens.is_pinned():
             self._host_tokens = torch.empty((max(n, 64),), dtype=torch.int32, pin_memory=True)
             self._home = torch.cuda.Event()
         self._host_tokens[:n].copy_(pending, non_blocking=True)
@@ -137,6 +144,14 @@ class GenerationLoop:
     def _arrived(self, event, n: int) -> list:
         event.synchronize()
         return self._host_tokens[:n].tolist()
+
+
+class _Arrived:
+    def synchronize(self) -> None:
+        pass
+
+
+_ARRIVED = _Arrived()
 
 
 def _decodes_on(plan) -> bool:
@@ -172,7 +187,7 @@ class LLM:
     ):
         """``ckpt_paths``: the model folder (config.json + safetensors), or a list whose first
         entry is that folder or a file in it.  ``precision``: "bfloat16" or "float32"; None takes
-        config.json's ``torch_dtype``.  ``max_len`` bounds prompt + generated tokens of a request,
+        config.json's ``torch_dtype``.  ``max_len`` bounds prompt + generated tokens of a request (as does the model's own maximum of positions),
         ``max_bsz`` the requests running at once.  ``model_kwargs`` may override ``max_seq_len``
         (reference: throughput_bench.py:1057-1060).  ``look_ahead``: prepare the next decode step
         while the GPU runs the current one (the tokens are the same either way).  ``kernel_table``:
@@ -204,11 +219,13 @@ class LLM:
             dtype=precision, device=device, page_size=page_size, num_pages=num_pages, kv_memory_gb=kv_memory_gb,
             kv_memory_fraction=kv_memory_fraction, max_seqs=max_bsz, max_model_len=max_len, kernel_table=kernel_table,
         )
-        if random_weights:
-            from ..config.registry import load_config
+        from ..config.registry import load_config
 
-            _, config = load_config(folder)
-            self.engine = Engine.from_random(config, seed=seed, **engine_kw)
+        arch, config = load_config(folder)
+        # ``max_len`` is a bound, and so is the model's own maximum of positions
+        engine_kw["max_model_len"] = min(max_len, arch.model_spec(config).max_positions)
+        if random_weights:
+            self.engine = Engine.from_random(config, seed=seed, arch=arch, **engine_kw)
         else:
             self.engine = Engine.from_folder(folder, **engine_kw)
         self.max_len = self.engine.max_model_len
@@ -225,8 +242,7 @@ class LLM:
         if self.template is not None and self.template.stop_token_ids:
             eos_ids = list(self.template.stop_token_ids)  # reference: llm.py:188-189
         if eos_ids is None:
-            eos = self.engine.config.eos_token_id
-            eos_ids = [] if eos is None else (list(eos) if isinstance(eos, (list, tuple)) else [eos])
+            eos_ids = self.engine.arch.default_stop_token_ids(self.engine.config)
         self.eos_ids = list(eos_ids)
         self.sampler = Sampler()
 

@@ -18,6 +18,7 @@ from .base import (  # noqa: F401
     _stream,
     check,
     core,
+    device_facts,
     dtype_code,
     resolved,
     variant,
@@ -27,6 +28,27 @@ from .base import (  # noqa: F401
 #: the largest head size any attention kernel here takes (the plain kernel's; the MFMA kernels take
 #: ``DECODE_HEAD_DIMS`` / ``PREFILL_HEAD_DIMS``, everything else below this runs the plain kernel)
 ATTENTION_MAX_HEAD_DIM = 256
+
+
+def _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq, positions, block_table, out):
+    """What both launches of the plain kernel ask of their arguments; returns (tokens, page size, out)."""
+    _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
+    _i32(token_seq, "token_seq")
+    _i32(positions, "positions")
+    n = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
+        raise KernelError("attention: qkv must be row-major with at least Hq * dh columns")
+    if token_seq.numel() != n or positions.numel() != n:
+        raise KernelError("attention: token_seq and positions need one entry per token")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("attention: block_table must be an int32 matrix")
+    page_size = k_pages.shape[2]
+    for pg in (k_pages, v_pages):
+        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+            raise KernelError("attention: pages must be contiguous [pages, Hkv, page_size, dh] of the query's dtype")
+    if out is None:
+        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    return n, page_size, out
 
 
 def attention_generic(
@@ -45,22 +67,7 @@ def attention_generic(
 ) -> torch.Tensor:
     """Attention of each token's query heads (the first Hq * dh columns of ``qkv``) over the paged
     keys and values of its request; returns [n, Hq * dh]."""
-    _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
-    _i32(token_seq, "token_seq")
-    _i32(positions, "positions")
-    n = qkv.shape[0]
-    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
-        raise KernelError("attention: qkv must be row-major with at least Hq * dh columns")
-    if token_seq.numel() != n or positions.numel() != n:
-        raise KernelError("attention: token_seq and positions need one entry per token")
-    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
-        raise KernelError("attention: block_table must be an int32 matrix")
-    page_size = k_pages.shape[2]
-    for pg in (k_pages, v_pages):
-        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
-            raise KernelError("attention: pages must be contiguous [pages, Hkv, page_size, dh] of the query's dtype")
-    if out is None:
-        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    n, page_size, out = _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq, positions, block_table, out)
     check(
         core().tl_attention_generic(
             qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
@@ -92,22 +99,7 @@ def attention_generic_split(
     keys is computed by a wave of its own and a second kernel joins the blocks in order.  The same
     blocks, operations and order as the one-wave form: the same bits.  ``longest``: an upper bound of
     the keys any token sees (its position + 1, or the window)."""
-    _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
-    _i32(token_seq, "token_seq")
-    _i32(positions, "positions")
-    n = qkv.shape[0]
-    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
-        raise KernelError("attention: qkv must be row-major with at least Hq * dh columns")
-    if token_seq.numel() != n or positions.numel() != n:
-        raise KernelError("attention: token_seq and positions need one entry per token")
-    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
-        raise KernelError("attention: block_table must be an int32 matrix")
-    page_size = k_pages.shape[2]
-    for pg in (k_pages, v_pages):
-        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
-            raise KernelError("attention: pages must be contiguous [pages, Hkv, page_size, dh] of the query's dtype")
-    if out is None:
-        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    n, page_size, out = _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq, positions, block_table, out)
     # blocks are aligned to absolute positions: a range of `longest` keys touches at most this many
     max_blocks = max(int(longest), 1) // 64 + 2
     partials = torch.empty((n, n_q_heads, max_blocks, head_dim + 2), dtype=torch.float32, device=qkv.device)
@@ -137,7 +129,6 @@ def decode_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: i
 
 
 _DECODE_MIN_SPLIT = 256  # keys: shorter splits cost more in launch and merge than they gain in spread
-_N_CUS = 256
 #: blocks a CU takes at a time before a launch stops gaining from more splits, by head size: about
 #: 64 KB of keys and values in flight on a CU (a block's four waves fetch 64 keys and values a pass)
 _DECODE_BLOCKS_PER_CU = {32: 3, 64: 3, 128: 2, 256: 1}
@@ -163,7 +154,7 @@ def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, head_dim: i
     more blocks than fit, and those that wait go where others end.  (64 requests of 128 to 4,608
     tokens: 30% less time than unsplit; 64 equal ones: 10% more, hence the switch.)"""
     pairs = max(n_tokens * n_kv_heads, 1)
-    limit = _N_CUS * _DECODE_BLOCKS_PER_CU.get(head_dim, 2)
+    limit = device_facts()[0] * _DECODE_BLOCKS_PER_CU.get(head_dim, 2)
     want = max(limit // pairs, 1)
     split = -(-max(longest, 1) // want)
     if uneven:

@@ -7,7 +7,7 @@ from typing import Optional
 
 import torch
 
-from .lib import KernelError, check, core, variant
+from .lib import KernelError, check, core, device_facts, variant  # noqa: F401
 
 F32, BF16 = 0, 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}

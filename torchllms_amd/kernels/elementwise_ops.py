@@ -18,14 +18,17 @@ from .base import (  # noqa: F401
     _stream,
     check,
     core,
+    device_facts,
     dtype_code,
     resolved,
     variant,
 )
 
 
-#: the widest row the norm kernels take: a row is kept in LDS as 32-bit floats (160 KB less 1 KB)
-RMSNORM_MAX_HIDDEN = (160 * 1024 - 1024) // 4
+def rmsnorm_max_hidden() -> int:
+    """The widest row the norm kernels take: a row is kept in LDS as 32-bit floats (the device's LDS,
+    160 KB on gfx950, less 1 KB)."""
+    return (device_facts()[1] - 1024) // 4
 
 
 def embed(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:

@@ -73,6 +73,29 @@ def core() -> ctypes.CDLL:
     return _core
 
 
+#: the GPU this package is written for (MI355X): what launch plans assume where no GPU is to be asked
+TARGET_COMPUTE_UNITS, TARGET_LDS_BYTES = 256, 160 * 1024
+_facts: Optional[tuple] = None
+
+
+def device_facts() -> tuple:
+    """``(compute units, bytes of LDS a block may use)`` of the GPU, as the device itself gives them
+    (read once, by the core library); the target's own figures where there is no GPU, so that launch
+    plans can be made and tested on a host without one."""
+    global _facts
+    if _facts is None:
+        import torch
+
+        if torch.cuda.is_available():
+            lib = core()
+            lib.tl_device_compute_units.restype = lib.tl_device_lds_bytes.restype = c_int
+            lib.tl_device_compute_units.argtypes = lib.tl_device_lds_bytes.argtypes = []
+            _facts = (int(lib.tl_device_compute_units()), int(lib.tl_device_lds_bytes()))
+        else:
+            _facts = (TARGET_COMPUTE_UNITS, TARGET_LDS_BYTES)
+    return _facts
+
+
 def variant(kind: str, value: int, signatures) -> ctypes.CDLL:
     """A size-specific library (see ``build.VARIANTS``), built on first use."""
     key = _build.variant_name(kind, value)

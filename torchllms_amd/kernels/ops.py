@@ -19,12 +19,13 @@ from .base import (  # noqa: F401
     SplitSums,
     check,
     core,
+    device_facts,
     dtype_code,
     resolved,
     variant,
 )
 from .elementwise_ops import (  # noqa: F401
-    RMSNORM_MAX_HIDDEN,
+    rmsnorm_max_hidden,
     add_bias_,
     embed,
     rmsnorm,

@@ -19,6 +19,7 @@ from .base import (  # noqa: F401
     _stream,
     check,
     core,
+    device_facts,
     dtype_code,
     resolved,
     variant,
@@ -261,10 +262,10 @@ WIDE_CHOICES = ((1, 1, 3), (2, 1, 3), (2, 1, 2), (1, 4, 3), (1, 8, 3), (2, 8, 3)
 
 
 def wide_fits(rows: int, strips_per_wave: int, stages: int) -> bool:
-    """Whether the buffers of such a launch fit the 160 KB of LDS: a buffer holds 4 KB for every 16
-    rows of the row tile (32, 64 or 128) and 16 KB for every strip per wave."""
+    """Whether the buffers of such a launch fit the device's LDS (160 KB on gfx950): a buffer holds
+    4 KB for every 16 rows of the row tile (32, 64 or 128) and 16 KB for every strip per wave."""
     tile = 32 if rows <= 32 else 64 if rows <= 64 else 128
-    return stages * (tile // 16 * 4 + strips_per_wave * 16) <= 160
+    return stages * (tile // 16 * 4 + strips_per_wave * 16) * 1024 <= device_facts()[1]
 
 #: how a product is used: alone; as the first half of ``linear_glu`` / ``qkv_rope_store``, whose
 #: second half (gate, rotation and cache write) some kernels take into themselves; or ("sum",

@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import logging
 from typing import Dict, Optional
 
 import torch
@@ -10,6 +11,10 @@ from ..config.spec import PartSpec
 from ..kernels import ops
 from ..kernels.attention import paged_attention
 from .base import MIXERS, POSITIONS, KVNeed, Mixer, ParamSpec
+
+
+#: (heads, kv heads, head size) whose fall to the plain attention kernel has been reported
+_SAID_SLOW: set = set()
 
 
 @MIXERS.register("attention")
@@ -77,6 +82,18 @@ class Attention(Mixer):
                 f"attention: head size {self.head_dim}; the attention kernels take head sizes up to "
                 f"{ops.ATTENTION_MAX_HEAD_DIM} (any number of heads and of query heads per kv head)"
             )
+        if dtype == torch.bfloat16:
+            fast = (ops.decode_attention_supported(dtype, self.num_heads, self.num_kv_heads, self.head_dim),
+                    ops.prefill_attention_supported(dtype, self.num_heads, self.num_kv_heads, self.head_dim))
+            said = (self.num_heads, self.num_kv_heads, self.head_dim)
+            if not all(fast) and said not in _SAID_SLOW:
+                _SAID_SLOW.add(said)
+                logging.getLogger("torchllms_amd").warning(
+                    "attention with %d heads in %d groups of head size %d: the matrix-core kernels take head sizes %s with at "
+                    "most 16 query heads per kv head (8 at head size 256 in decode steps); %s run the plain kernel (right, and several times slower)",
+                    self.num_heads, self.num_kv_heads, self.head_dim, "/".join(str(d) for d in ops.DECODE_HEAD_DIMS),
+                    "decode steps and prompts" if not any(fast) else "decode steps" if not fast[0] else "prompts",
+                )
         rot = self.position.rotary_args()
         if rot is not None and (rot.rotary_dim % 2 or rot.rotary_dim > self.head_dim):
             raise ValueError(f"attention: {rot.rotary_dim} rotated channels of a head of {self.head_dim} (even, at most the head size)")

@@ -27,8 +27,8 @@ class RMSNorm(Norm):
         return {"weight": ParamSpec((self.size,), kind="vector", init="ones")}
 
     def check_sizes(self, dtype: torch.dtype) -> None:
-        if not 0 < self.size <= ops.RMSNORM_MAX_HIDDEN:
-            raise ValueError(f"rmsnorm: rows of {self.size} elements; the kernel takes 1 to {ops.RMSNORM_MAX_HIDDEN}")
+        if not 0 < self.size <= ops.rmsnorm_max_hidden():
+            raise ValueError(f"rmsnorm: rows of {self.size} elements; the kernel takes 1 to {ops.rmsnorm_max_hidden()}")
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors["weight"].contiguous()

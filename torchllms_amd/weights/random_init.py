@@ -10,12 +10,13 @@ lacks (reference: torchllms/models/utils.py:197-214, networks.py:192-193).  Valu
 from __future__ import annotations
 
 import hashlib
+import json
 from pathlib import Path
 from typing import Dict, Optional
 
 import torch
 
-from ..config.registry import ArchSpec, get_architecture
+from ..config.registry import ArchSpec, architecture_of, get_architecture
 from ..parts.base import ParamSpec
 from ..parts.model import Model
 
@@ -69,7 +70,7 @@ def write_model_folder(
     model of this configuration with random weights."""
     from safetensors.torch import save_file
 
-    arch = arch or get_architecture(config.architectures[0])
+    arch = arch or architecture_of(config)
     folder = Path(folder)
     folder.mkdir(parents=True, exist_ok=True)
     model = Model(arch.model_spec(config))
@@ -86,7 +87,8 @@ def write_model_folder(
                 break
         else:
             raise KeyError(f"no rule names the tensor {name}")
-    config.save(folder)
+    with open(folder / "config.json", "w") as f:
+        json.dump(arch.config_json(config), f, indent=2)
     save_file(tensors, str(folder / "model.safetensors"), metadata={"format": "pt"})
     return folder
 
