@@ -145,61 +145,121 @@ gemm_f32_kernel(const float* __restrict__ A, int lda, const float* __restrict__ 
 // of an element over the lanes of a wave:
 //   * a block of 4 waves takes 16 columns of the result, 4 per wave, and all rows (at most MR);
 //   * K is walked in rounds of 1,024 = 64 groups: lane j computes group j of the round for its wave's
-//     4 columns and every row (W: 64 contiguous bytes per lane and column, the wave reads 4 KB on end;
+//     4 columns and every row (W: the wave reads a column's 4 KB of the round 1 KB per instruction and
+//     turns it through a piece of LDS of its own, so that lane j holds elements 16 j .. 16 j + 15;
 //     A: the round's slice of every row lies in LDS, loaded once per block, transposed so that the 64
-//     lanes read 64 consecutive words);
+//     lanes read 64 consecutive words); what the next round needs travels from memory into registers
+//     while this round is multiplied;
 //   * the groups' sums then have to join the running sums in the order of the groups: they go through
 //     LDS, transposed, and lane p of the wave adds the 64 sums of (column, row) pair p one after the other.
 constexpr int kRowsCols = 4;               // columns per wave
 constexpr int kRowsWaves = 4;              // waves per block
 constexpr int kRound = 64 * BK;            // k per round
 constexpr int kPad = 65;                   // row stride of transposed tables in LDS (odd: no bank conflicts)
+constexpr int kTurned = kRound + kRound / 4;  // a column's round of W in LDS: four words of padding behind every group
 
-template <int MR>
+template <int MR, bool kVec>
 __global__ void __launch_bounds__(kRowsWaves * kWave)
 gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
                      float* __restrict__ C, int ldc, int M, int N, int K) {
   constexpr int kPairs = kRowsCols * MR;   // (column, row) pairs of a wave: at most 64
+  constexpr int kWaveRegion = kPairs * kPad > kTurned ? kPairs * kPad : kTurned;
   extern __shared__ float lds[];
   float* xs = lds;                                          // [MR][BK][kPad]: element u of group j of row m at (m * BK + u) * kPad + j
-  float* ps = lds + MR * BK * kPad;                         // [waves][kPairs][kPad]
+  float* ps = lds + MR * BK * kPad;                         // [waves][kWaveRegion]: a wave's own piece
   const int tid = threadIdx.x;
   const int wave = tid / kWave;
   const int lane = tid % kWave;
-  float* my_ps = ps + wave * kPairs * kPad;
+  float* my_ps = ps + wave * kWaveRegion;                   // [kPairs][kPad] sums, or a column's round of W being turned
   const int n0 = (blockIdx.x * kRowsWaves + wave) * kRowsCols;
 
   float acc = 0.f;  // lane p < kPairs: running sum of pair p = (column p / MR, row p % MR)
 
+  // What a round needs from memory is asked for a round ahead and waits in registers while the round
+  // before it is multiplied.  Thread t moves elements 4 t .. 4 t + 3 of every row's slice of A; lane l
+  // moves, of each of the wave's four columns of W, elements 256 q + 4 l .. + 3 for q = 0 .. 3 (the wave
+  // reads 1 KB on end per instruction).
+  // Two kernels (kVec): with rows of A and W on 16-byte boundaries and K a multiple of 4 everything is
+  // fetched sixteen bytes a lane, otherwise element by element (one kernel with both forms under a branch
+  // came out of the compiler with the element-wise loads for both).  Rows past M and elements past K are
+  // read from a valid place (the row's last elements) and replaced by zeros when the round begins:
+  // nothing here looks at a loaded value, or the wave would wait for each load in turn.
+  float a_next[MR][4];
+  float w_next[kRowsCols][BK];
+  auto fetch = [&](int k0) {
+    const int ka = k0 + 4 * tid;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const float* arow = A + (size_t)(m < M ? m : 0) * lda;
+      if constexpr (kVec) {
+        const float4 v = *reinterpret_cast<const float4*>(arow + min(ka, K - 4));
+        a_next[m][0] = v.x; a_next[m][1] = v.y; a_next[m][2] = v.z; a_next[m][3] = v.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a_next[m][e] = arow[min(ka + e, K - 1)];
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < kRowsCols; ++c) {
+      const int n = n0 + c;
+      const float* wrow = W + (size_t)(n < N ? n : N - 1) * ldw;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int k = k0 + 256 * q + 4 * lane;
+        if constexpr (kVec) {
+          const float4 v = *reinterpret_cast<const float4*>(wrow + min(k, K - 4));
+          w_next[c][4 * q] = v.x; w_next[c][4 * q + 1] = v.y; w_next[c][4 * q + 2] = v.z; w_next[c][4 * q + 3] = v.w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w_next[c][4 * q + e] = wrow[min(k + e, K - 1)];
+        }
+      }
+    }
+  };
+
+  fetch(0);
   for (int k0 = 0; k0 < K; k0 += kRound) {
     __syncthreads();  // everybody has finished with the slice of the round before
-    for (int i = tid; i < MR * kRound; i += kRowsWaves * kWave) {
-      const int m = i / kRound, kk = i % kRound, k = k0 + kk;
-      xs[(m * BK + kk % BK) * kPad + kk / BK] = (m < M && k < K) ? A[(size_t)m * lda + k] : 0.f;
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int kk = 4 * tid + e;
+        xs[(m * BK + kk % BK) * kPad + kk / BK] = (m < M && k0 + kk < K) ? a_next[m][e] : 0.f;
+      }
+    // the wave turns its columns of W through its own piece of LDS (free: the sums of the round before
+    // have been added): lane j gets group j, elements 16 j .. 16 j + 15 of the round.  A wave's LDS
+    // instructions are carried out in their order, so no barrier stands between the writes and the reads.
+    float w[kRowsCols][BK];
+#pragma unroll
+    for (int c = 0; c < kRowsCols; ++c) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int kk = 256 * q + 4 * lane;
+        const int left = K - (k0 + kk);  // elements of the row from here on: past them, zeros
+        *reinterpret_cast<float4*>(my_ps + kk + 4 * (kk / BK)) =
+            float4{left > 0 ? w_next[c][4 * q] : 0.f, left > 1 ? w_next[c][4 * q + 1] : 0.f,
+                   left > 2 ? w_next[c][4 * q + 2] : 0.f, left > 3 ? w_next[c][4 * q + 3] : 0.f};
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int u = 0; u < BK; u += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(my_ps + (BK + 4) * lane + u);
+        w[c][u] = v.x; w[c][u + 1] = v.y; w[c][u + 2] = v.z; w[c][u + 3] = v.w;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
     }
+    // (asked for as soon as the registers are free, before the barrier: the fewer cycles a wave has no
+    // load under way, the better; with two blocks a CU nobody else fills the gap)
+    if (k0 + kRound < K) fetch(k0 + kRound);
     __syncthreads();
-    const int kg = k0 + BK * lane;  // this lane's group of the round
     float part[kRowsCols][MR];
 #pragma unroll
     for (int c = 0; c < kRowsCols; ++c)
 #pragma unroll
       for (int m = 0; m < MR; ++m) part[c][m] = 0.f;
-    float w[kRowsCols][BK];
-#pragma unroll
-    for (int c = 0; c < kRowsCols; ++c) {
-      const int n = n0 + c;
-      const float* wrow = W + (size_t)(n < N ? n : N - 1) * ldw;
-      if (kg + BK <= K && (ldw % 4) == 0 && ((uintptr_t)W % 16) == 0) {
-#pragma unroll
-        for (int u = 0; u < BK; u += 4) {
-          const float4 v = *reinterpret_cast<const float4*>(wrow + kg + u);
-          w[c][u] = v.x; w[c][u + 1] = v.y; w[c][u + 2] = v.z; w[c][u + 3] = v.w;
-        }
-      } else {
-#pragma unroll
-        for (int u = 0; u < BK; ++u) w[c][u] = kg + u < K ? wrow[kg + u] : 0.f;
-      }
-    }
 #pragma unroll
     for (int u = 0; u < BK; ++u) {
 #pragma unroll
@@ -218,7 +278,16 @@ gemm_f32_rows_kernel(const float* __restrict__ A, int lda, const float* __restri
     if (lane < kPairs) {
       const float* mine = my_ps + lane * kPad;
       const int groups = min(64, (K - k0 + BK - 1) / BK);  // groups of this round that exist
-      for (int g = 0; g < groups; ++g) acc += mine[g];
+      if (groups == 64) {
+        // all 64 sums are asked for before the first is added (a loop would wait for LDS 64 times in a row)
+        float sums[64];
+#pragma unroll
+        for (int g = 0; g < 64; ++g) sums[g] = mine[g];
+#pragma unroll
+        for (int g = 0; g < 64; ++g) acc += sums[g];
+      } else {
+        for (int g = 0; g < groups; ++g) acc += mine[g];
+      }
     }
   }
   if (lane < kPairs) {
@@ -237,15 +306,21 @@ TL_EXPORT int tl_gemm_f32(const float* A, int lda, const float* W, int ldw, floa
   if (M <= 16) {
     // decode steps: the same sums, spread over a wave (see above)
     const unsigned blocks = (N + kRowsWaves * kRowsCols - 1) / (kRowsWaves * kRowsCols);
+    const bool vec = K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0;
 #define TL_ROWS_LAUNCH(MR)                                                                               \
   do {                                                                                                   \
-    const size_t lds = ((size_t)MR * BK * kPad + (size_t)kRowsWaves * kRowsCols * MR * kPad) * sizeof(float); \
+    const size_t region = (size_t)kRowsCols * MR * kPad > (size_t)kTurned ? (size_t)kRowsCols * MR * kPad : (size_t)kTurned; \
+    const size_t lds = ((size_t)MR * BK * kPad + (size_t)kRowsWaves * region) * sizeof(float);               \
     if (lds > 48 * 1024) {                                                                               \
-      hipError_t e = hipFuncSetAttribute((const void*)gemm_f32_rows_kernel<MR>,                          \
+      hipError_t e = hipFuncSetAttribute(vec ? (const void*)gemm_f32_rows_kernel<MR, true>               \
+                                             : (const void*)gemm_f32_rows_kernel<MR, false>,             \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);          \
       if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "gemm_f32: %s", hipGetErrorString(e));             \
     }                                                                                                    \
-    gemm_f32_rows_kernel<MR><<<blocks, kRowsWaves * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K); \
+    if (vec)                                                                                             \
+      gemm_f32_rows_kernel<MR, true><<<blocks, kRowsWaves * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K); \
+    else                                                                                                 \
+      gemm_f32_rows_kernel<MR, false><<<blocks, kRowsWaves * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K); \
   } while (0)
     if (M == 1) TL_ROWS_LAUNCH(1);
     else if (M == 2) TL_ROWS_LAUNCH(2);
