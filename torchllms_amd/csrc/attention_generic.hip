@@ -26,6 +26,20 @@ __device__ __forceinline__ void load4(const bf16_t* p, float (&v)[4]) {
   v[2] = __uint_as_float(x.y << 16); v[3] = __uint_as_float(x.y & 0xffff0000u);
 }
 
+// The same in two steps: the load as it comes from memory, and its elements as floats later.
+template <typename T> struct Raw4;
+template <> struct Raw4<float> { float4 x; };
+template <> struct Raw4<bf16_t> { uint2 x; };
+__device__ __forceinline__ Raw4<float> load_raw4(const float* p) { return {*reinterpret_cast<const float4*>(p)}; }
+__device__ __forceinline__ Raw4<bf16_t> load_raw4(const bf16_t* p) { return {*reinterpret_cast<const uint2*>(p)}; }
+__device__ __forceinline__ void unpack4(const Raw4<float>& r, float (&v)[4]) {
+  v[0] = r.x.x; v[1] = r.x.y; v[2] = r.x.z; v[3] = r.x.w;
+}
+__device__ __forceinline__ void unpack4(const Raw4<bf16_t>& r, float (&v)[4]) {
+  v[0] = __uint_as_float(r.x.x << 16); v[1] = __uint_as_float(r.x.x & 0xffff0000u);
+  v[2] = __uint_as_float(r.x.y << 16); v[3] = __uint_as_float(r.x.y & 0xffff0000u);
+}
+
 // What a wave needs to know about its (token, query head).
 template <typename T>
 struct Query {
@@ -60,11 +74,24 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
     const T* kr = a.k_pages + row_at;
     float dot = 0.f;
     if (VEC) {
-      for (int d = 0; d < a.head_dim; d += 4) {
-        float kv[4];
-        load4(kr + d, kv);
+      // eight pieces of the row are asked for before the first is multiplied (a piece past the row's end is
+      // the row's first once more, and not used): left to itself the compiler waited for every load of a
+      // bfloat16 row in turn
+      constexpr int kAhead = 8;
+      for (int d0 = 0; d0 < a.head_dim; d0 += 4 * kAhead) {
+        Raw4<T> raw[kAhead];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) dot = fmaf(a.qs[d + u], kv[u], dot);
+        for (int u = 0; u < kAhead; ++u) raw[u] = load_raw4(kr + (d0 + 4 * u < a.head_dim ? d0 + 4 * u : 0));
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+          const int d = d0 + 4 * u;
+          if (d < a.head_dim) {
+            float kv[4];
+            unpack4(raw[u], kv);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dot = fmaf(a.qs[d + e], kv[e], dot);
+          }
+        }
       }
     } else {
       for (int d = 0; d < a.head_dim; ++d) dot = fmaf(a.qs[d], to_f32(kr[d]), dot);
@@ -80,7 +107,9 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
   const int jj_hi = a.p - j0 < kWave - 1 ? a.p - j0 : kWave - 1;
   constexpr int U = 8;  // value rows in flight
   for (int jj = jj_lo; jj <= jj_hi; jj += U) {
-    float vv[U][kChanPerLane];
+    // the rows' elements as they come from memory (a channel past the head's size reads channel 0 and
+    // counts as zero below): nothing looks at a loaded value before all U rows are asked for
+    T vv[U][kChanPerLane];
     float pw[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -90,14 +119,17 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
 #pragma unroll
       for (int c = 0; c < kChanPerLane; ++c) {
         const int d = lane + c * kWave;
-        vv[u][c] = d < a.head_dim ? to_f32(vr[d]) : 0.f;
+        if (c * kWave < a.head_dim) vv[u][c] = vr[d < a.head_dim ? d : 0];
       }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
       if (jj + u <= jj_hi) {
 #pragma unroll
-        for (int c = 0; c < kChanPerLane; ++c) o_b[c] = fmaf(pw[u], vv[u][c], o_b[c]);
+        for (int c = 0; c < kChanPerLane; ++c) {
+          const int d = lane + c * kWave;
+          if (c * kWave < a.head_dim) o_b[c] = fmaf(pw[u], d < a.head_dim ? to_f32(vv[u][c]) : 0.f, o_b[c]);
+        }
       }
   }
 }
