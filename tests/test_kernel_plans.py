@@ -13,19 +13,21 @@ def test_decode_splits_cover_the_range_and_stay_under_a_cu_s_share_of_blocks():
                 for longest in (1, 15, 256, 1000, 8192, 70000, 131072):
                     for uneven in (False, True):
                         split, n_splits = ops.plan_decode_splits(n_tokens, n_kv_heads, longest, head_dim, uneven=uneven)
-                        assert split % 64 == 0 and split >= 256
+                        assert split % 64 == 0 and split >= 128
                         assert n_splits >= 1 and (n_splits - 1) * split < max(longest, 1) <= n_splits * split
                         if uneven:
                             assert split <= attention_ops.DECODE_UNEVEN_SPLIT == 512
                         elif n_splits > 1:
+                            # (few long rows at head size 128 aim at one block a CU)
+                            at_a_time = 256 * (1 if head_dim == 128 and n_tokens * n_kv_heads <= 32 else per_cu)
                             # never more blocks than the CUs take at a time, unless the shortest split allowed is reached
-                            assert split == 256 or n_tokens * n_kv_heads * n_splits <= 256 * per_cu
+                            assert split == 128 or n_tokens * n_kv_heads * n_splits <= at_a_time
                             # and no fewer splits than that allows: one split more would be too many
                             shorter = split - 64
-                            assert shorter < 256 or n_tokens * n_kv_heads * -(-longest // shorter) > 256 * per_cu or -(-longest // shorter) == n_splits
+                            assert shorter < 128 or n_tokens * n_kv_heads * -(-longest // shorter) > at_a_time or -(-longest // shorter) == n_splits
     # head sizes with fewer bytes a key take more blocks a CU
     assert ops.plan_decode_splits(8, 8, 2176, 128) == (320, 7)
-    assert ops.plan_decode_splits(8, 8, 2176, 64) == (256, 9)
+    assert ops.plan_decode_splits(8, 8, 2176, 64) == (192, 12)
     assert ops.plan_decode_splits(8, 4, 8192, 256) == (1024, 8)
 
 
@@ -110,10 +112,10 @@ def test_launch_plans_take_the_device_s_own_figures(monkeypatch):
     from torchllms_amd.kernels import lib
 
     assert lib.device_facts() == (256, 160 * 1024)
-    assert ops.plan_decode_splits(1, 8, 8192) == (256, 32) and ops.wide_fits(64, 2, 3) and ops.rmsnorm_max_hidden() == 40704
+    assert ops.plan_decode_splits(1, 8, 8192) == (256, 32) and ops.plan_decode_splits(8, 8, 8192) == (1024, 8)
+    assert ops.wide_fits(64, 2, 3) and ops.rmsnorm_max_hidden() == 40704
     monkeypatch.setattr(lib, "_facts", (128, 64 * 1024))
-    assert ops.plan_decode_splits(1, 8, 8192) == (256, 32)  # (the shortest split allowed either way)
-    assert ops.plan_decode_splits(4, 8, 8192) == (1024, 8)  # 256 blocks at a time instead of 512
+    assert ops.plan_decode_splits(1, 8, 8192) == (512, 16) and ops.plan_decode_splits(8, 8, 8192) == (2048, 4)  # half the blocks at a time
     assert not ops.wide_fits(64, 2, 3) and ops.wide_fits(32, 1, 2) and ops.rmsnorm_max_hidden() == 16128
 
 

@@ -128,10 +128,15 @@ def decode_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: i
     return n_q_heads // n_kv_heads <= (16 if head_dim <= 128 else 8)
 
 
-_DECODE_MIN_SPLIT = 256  # keys: shorter splits cost more in launch and merge than they gain in spread
+_DECODE_MIN_SPLIT = 128  # keys: shorter splits cost more in the merge than they gain in spread (with 256, short contexts at small batches left most CUs idle: one request of 2,176 keys 12.5 -> 10.0 us, eight of 1,024 15.9 -> 14.6)
 #: blocks a CU takes at a time before a launch stops gaining from more splits, by head size: about
 #: 64 KB of keys and values in flight on a CU (a block's four waves fetch 64 keys and values a pass)
 _DECODE_BLOCKS_PER_CU = {32: 3, 64: 3, 128: 2, 256: 1}
+#: up to this many (request, kv head) pairs a launch at head size 128 aims at one block a CU: the splits are long
+#: then, a CU's one block keeps its loads in flight by itself, and half as many partial results go through the merge
+#: (two requests of 8,192 keys: 21.6 -> 20.7 us; one of 16,384: 23.4 -> 21.9, of 32,768: 37.6 -> 32.8; four of 4,096:
+#: 21.5 -> 19.6; at head size 64 two and three blocks a CU stayed better at every size)
+_DECODE_FEW_PAIRS = 32
 
 
 DECODE_UNEVEN_SPLIT = 512  # keys: the longest split when requests differ much in length (measured with 64 requests of 128 to 4,608 tokens: 1 to 1.5% more tokens a second than with 1,024, 12% more than with 2,048)
@@ -141,7 +146,7 @@ def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, head_dim: i
     """``(split_size, n_splits)`` for a decode launch whose longest visible key range (counted from
     its 16-aligned start) is ``longest``: as many splits as give every CU its share of blocks and
     no more (two blocks a CU at head size 128, one at 256, three at 64 and 32), none shorter than
-    256 keys.  A launch is as long as its most loaded CU, so a few blocks beyond a whole number a CU
+    128 keys.  A launch is as long as its most loaded CU, so a few blocks beyond a whole number a CU
     cost as much as a whole further round, and every split costs its start, its partial results
     and its share of the merge; staying under the limit was the best choice or within 1% of it on
     average (at most 11%) over 1 to 100 requests of 700 to 20,000 tokens at each head size, where
@@ -154,7 +159,10 @@ def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, head_dim: i
     more blocks than fit, and those that wait go where others end.  (64 requests of 128 to 4,608
     tokens: 30% less time than unsplit; 64 equal ones: 10% more, hence the switch.)"""
     pairs = max(n_tokens * n_kv_heads, 1)
-    limit = device_facts()[0] * _DECODE_BLOCKS_PER_CU.get(head_dim, 2)
+    per_cu = _DECODE_BLOCKS_PER_CU.get(head_dim, 2)
+    if head_dim == 128 and pairs <= _DECODE_FEW_PAIRS:
+        per_cu = 1
+    limit = device_facts()[0] * per_cu
     want = max(limit // pairs, 1)
     split = -(-max(longest, 1) // want)
     if uneven:
