@@ -141,3 +141,17 @@ def test_a_head_size_without_matrix_core_kernels_is_reported_once(caplog):
         assert len(caplog.records) == 1 and "head size 96" in caplog.text and "decode steps and prompts run the plain kernel" in caplog.text
         part(256, heads=16, kv=1).check_sizes(torch.bfloat16)  # 16 query heads per kv head: prompts only
         assert len(caplog.records) == 2 and "; decode steps run the plain kernel" in caplog.records[1].getMessage()
+
+
+def test_near_ties_of_the_measurement_are_decided_by_rule_not_by_the_stopwatch():
+    """Candidates within 4% of the fastest count as equal; among them one that does the whole use in its own
+    kernels wins over one that needs a kernel behind it, a kernel of the package over the library, and the
+    candidates' fixed order decides the rest: the table, and with it the bfloat16 bits, does not flip from
+    run to run on a tie."""
+    lib, split, whole = None, ("wide", 1, 2, 3), ("wide", 2, 1, 3)
+    assert products.pick([(lib, 17.9), (split, 18.4), (whole, 22.0)], "qkv") == split  # rotates in its second kernel
+    assert products.pick([(lib, 18.4), (split, 17.9)], "qkv") == split
+    assert products.pick([(lib, 17.0), (split, 18.4)], "qkv") is lib  # 8% apart: no tie
+    assert products.pick([(lib, 50.0), (whole, 50.5), (split, 50.2)], "glu") == whole  # the gate ends a whole product
+    assert products.pick([(lib, 10.0), (split, 10.3), (whole, 10.2)], "sum") == split  # first of the package's in the list
+    assert products.pick([(lib, 10.0)], "plain") is lib

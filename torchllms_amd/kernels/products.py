@@ -258,7 +258,7 @@ ROW_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128)
 STREAM_WAVE_CHOICES = (0, 4)
 #: (strips per wave, splits of K, buffers) that ``tune_linear`` tries from 17 rows on: whole-K
 #: launches for matrices with many rows, splits of K for those with few
-WIDE_CHOICES = ((1, 1, 3), (2, 1, 3), (2, 1, 2), (1, 4, 3), (1, 8, 3), (2, 8, 3), (2, 8, 2))
+WIDE_CHOICES = ((1, 1, 3), (2, 1, 3), (2, 1, 2), (1, 2, 3), (1, 4, 3), (2, 4, 3), (2, 4, 2), (1, 8, 3), (2, 8, 3), (2, 8, 2))
 
 
 def wide_fits(rows: int, strips_per_wave: int, stages: int) -> bool:
@@ -454,7 +454,7 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
                 return lambda w: run_glu(choice, x, w)
             return lambda w: run_choice(choice, x, w, out_dtype, leave_split=use == "sum")
 
-        best, best_time = None, cost(bucket, None, run(None))
+        timed = [(None, cost(bucket, None, run(None)))]
         if bucket <= STREAM_MAX_ROWS and use == "glu":
             candidates = [("stream", waves, cols) for waves in STREAM_WAVE_CHOICES for cols in (8, 16)]
         elif bucket <= STREAM_MAX_ROWS:
@@ -465,11 +465,24 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
             candidates = [c for c in candidates if c[3] == 3 or not wide_fits(bucket, c[1], 3)]
         else:
             candidates = []
-        for choice in candidates:
-            t = cost(bucket, choice, run(choice))
-            if t < best_time:
-                best, best_time = choice, t
-        LINEAR_CHOICE[(n, k, bucket, use)] = best
+        timed += [(choice, cost(bucket, choice, run(choice))) for choice in candidates]
+        LINEAR_CHOICE[(n, k, bucket, use)] = pick(timed, use)
+
+
+#: two candidates whose times differ by less than this share are taken to be equal: which of them a stopwatch
+#: puts first changes from run to run (the library's product with a rotary kernel behind it against the split
+#: product that rotates in its second kernel, at 64 rows of the 8B shape, did), and with it the bfloat16 bits
+TUNE_TIE = 0.04
+
+
+def pick(timed, use: str):
+    """The choice among ``[(choice, time)]``: the fastest, except that among those within ``TUNE_TIE`` of the
+    fastest one that does the whole of ``use`` in its own kernels comes before one that does not, and a kernel
+    of this package before the library; among equals the first in the list (the candidates' fixed order)."""
+    least = min(t for _, t in timed)
+    close = [c for c, t in timed if t <= least * (1.0 + TUNE_TIE)]
+    close.sort(key=lambda c: (not fuses_tail(c, use), c is None))  # (a stable sort: the list's order breaks ties)
+    return close[0]
 
 
 def run_choice(choice, x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, leave_split: bool = False):
