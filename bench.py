@@ -2,7 +2,7 @@
 bfloat16 weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
-                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels]
+                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products]
 
 Everything runs through the generation loop: the scheduler admits the requests, cuts their prompts
 into portions under its token budget, and plans every decode step; the step function runs it; the
@@ -28,6 +28,9 @@ a read of 4 GiB with 16-byte loads, a device copy, a loop of MFMA instructions o
 library's large matrix product.  ``--workload small-kernels`` times what a norm kernel adds to a
 replayed graph of large products, without a profiler (under rocprofv3 no dispatch is shorter than
 about 4.6 us, an empty kernel included, so a kernel trace overstates the small kernels of a step).
+``--workload attention``: the decode attention and the merge of its splits alone, by batch size, context and
+split size.  ``--workload products``: a decode layer's four products alone at 1 to 128 rows, the library against
+this package's kernels.  Both as a step runs them: in a replayed graph, caches flushed.
 """
 
 from __future__ import annotations
@@ -79,7 +82,7 @@ def parse_args(argv=None):
     p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the headline's)")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels"])
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products"])
     p.add_argument("--token-budget", type=int, default=8192, help="tokens a step may hold (the scheduler cuts prompts to it)")
     p.add_argument("--no-reference-workload", action="store_true",
                    help="leave out the reference's benchmark (2,048-token prompts, 256 new tokens at batch 1, 8, 64)")
@@ -391,6 +394,118 @@ def small_kernels_run(args, shape) -> int:
     return 0
 
 
+def _cold_graph_us(fn, repeats: int, flush) -> float:
+    """Microseconds per call of ``fn(i)``, i = 0 .. repeats - 1, recorded into one HIP graph and replayed with the
+    caches flushed before each of five replays (the least counts): as a kernel runs inside a decode step."""
+    import gc
+
+    import torch
+
+    with torch.inference_mode():
+        for i in range(repeats):
+            fn(i)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                for i in range(repeats):
+                    fn(i)
+        finally:
+            if collecting:
+                gc.enable()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        best = float("inf")
+        for _ in range(5):
+            flush.sum()
+            start.record()
+            graph.replay()
+            stop.record()
+            stop.synchronize()
+            best = min(best, start.elapsed_time(stop) * 1e3)
+    return best / repeats
+
+
+def attention_run(args, shape) -> int:
+    """The decode attention kernel and the merge of its splits alone: every request at context C, behind a
+    gate/up product that evicts the caches, in a replayed graph; per batch size and context the time with the
+    planned splits and with splits of 128 to 2,048 keys."""
+    import torch
+
+    from torchllms_amd.kernels import ops
+
+    dev = "cuda:0"
+    hq, hkv, dh, page = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"], args.page_size
+    x = torch.randn(8, shape["hidden_size"], device=dev).to(torch.bfloat16)
+    big = [torch.randn(2 * shape["intermediate_size"], shape["hidden_size"], device=dev).mul_(0.02).to(torch.bfloat16) for _ in range(4)]
+    flush = torch.zeros(512 << 18, device=dev)
+    layers = 8
+    between = lambda i: ops.gemm_stream_glu(x, big[i % 4], 0, 16)
+    base = _cold_graph_us(between, layers, flush)
+    table = {}
+    for batch in (1, 2, 4, 8, 16, 64):
+        for ctx in (2176, 8192, 32768):
+            if batch * ctx > 600000:
+                continue
+            n_pages = batch * ctx // page
+            caches = [(torch.randn(n_pages, hkv, page, dh, device=dev).to(torch.bfloat16), torch.randn(n_pages, hkv, page, dh, device=dev).to(torch.bfloat16))
+                      for _ in range(3)]
+            tables = torch.arange(n_pages, dtype=torch.int32, device=dev).view(batch, -1).contiguous()
+            q = torch.randn(batch, (hq + 2 * hkv) * dh, device=dev).to(torch.bfloat16)
+            seq = torch.arange(batch, dtype=torch.int32, device=dev)
+            pos = torch.full((batch,), ctx - 1, dtype=torch.int32, device=dev)
+            row = {}
+            for split in (None, 128, 256, 512, 1024, 2048):
+                if split is not None and ctx // split > 512:
+                    continue
+
+                def step(i, split=split):
+                    between(i)
+                    k, v = caches[i % 3]
+                    ops.attention_decode(q, hq, hkv, dh, k, v, seq, pos, tables, 0, dh ** -0.5, ctx, split_size=split)
+
+                row["planned" if split is None else str(split)] = round(_cold_graph_us(step, layers, flush) - base, 1)
+            plan = ops.plan_decode_splits(batch, hkv, ctx, dh)
+            mb = batch * ctx * hkv * dh * 4 / 1e6
+            table[f"b{batch}_ctx{ctx}"] = {"plan": list(plan), "mb": round(mb, 1), "us": row}
+            del caches
+    print(json.dumps({"metric": "decode attention and merge alone, cold, behind a large product", "unit": "us",
+                      "model": SHAPE_NAMES[args.shape], "by_split_size": table}))
+    return 0
+
+
+def products_run(args, shape) -> int:
+    """The four matrix products of a decode layer alone at 1 to 128 rows, cold weights in a replayed graph: the
+    library, and the kernels of this package in the launch that the measurement at engine start would pick."""
+    import torch
+
+    from torchllms_amd.kernels import ops, products
+
+    dev = "cuda:0"
+    d, f = shape["hidden_size"], shape["intermediate_size"]
+    qkv = (shape["num_attention_heads"] + 2 * shape["num_key_value_heads"]) * shape["head_dim"]
+    shapes = {"qkv": (qkv, d, "qkv"), "o": (d, shape["num_attention_heads"] * shape["head_dim"], "sum"), "gate_up": (2 * f, d, "glu"), "down": (d, f, "sum")}
+    flush = torch.zeros(512 << 18, device=dev)
+    out = {}
+    for name, (n, k, use) in shapes.items():
+        weights = [torch.randn(n, k, device=dev).mul_(0.02).to(torch.bfloat16) for _ in range(4)]
+        timed = {}
+        ops.tune_linear(weights, torch.bfloat16, use, report=lambda bucket, choice, us: timed.setdefault(bucket, []).append((choice, us)))
+        rows = {}
+        for bucket, cands in sorted(timed.items()):
+            chosen = products.LINEAR_CHOICE[(n, k, bucket, use)]
+            lib = next(us for c, us in cands if c is None)
+            best = min(us for _, us in cands)
+            rows[str(bucket)] = {"library_us": round(lib, 1), "chosen": None if chosen is None else list(chosen),
+                                 "chosen_us": round(next(us for c, us in cands if c == chosen), 1), "least_us": round(best, 1)}
+        out[name] = {"n": n, "k": k, "use": use, "mb": round(n * k * 2 / 1e6, 1), "by_rows": rows}
+        del weights
+    print(json.dumps({"metric": "decode products alone, cold weights in a replayed graph (times as the engine's measurement charges them)",
+                      "unit": "us", "model": SHAPE_NAMES[args.shape], "products": out}))
+    return 0
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     if args.gpus != 1:
@@ -401,6 +516,10 @@ def main(argv=None) -> int:
         return serve_run(args, shape)
     if args.workload == "small-kernels":
         return small_kernels_run(args, shape)
+    if args.workload == "attention":
+        return attention_run(args, shape)
+    if args.workload == "products":
+        return products_run(args, shape)
     if args.workload == "peaks":
         return peaks_run(args)
     import torch

@@ -798,13 +798,13 @@ def _fill_pages(k_pages, v_pages, table, k, v):
 
 @pytest.mark.parametrize("batch, S", [(1, 32768), (8, 32768), (64, 8192)])
 def test_attention_decode_at_the_longest_contexts_that_are_measured(batch, S):
-    """32,768 keys for one request (32 splits of 1,024 keys) and for eight (8 splits of 4,096), and 64
-    requests of 8,192 (one block walks all keys of a request, no merge): the launches of the context
-    sweep and of the batch-64 measurement.  Random scores in most rows; in some a single key, near
+    """32,768 keys for one request and for eight (32 splits of 1,024 keys), and 64 requests of 8,192 (8 splits;
+    and unsplit, one block walking all keys of a request, no merge): the launches of the context sweep and of
+    the batch-64 measurement.  Random scores in most rows; in some a single key, near
     the start, at a split's edge or at the end, that outweighs all others."""
     ops = _ops()
     hq, hkv, dh, page = 32, 8, 128, 16
-    assert ops.plan_decode_splits(batch, hkv, S) == {1: (1024, 32), 8: (4096, 8), 64: (8192, 1)}[batch]
+    assert ops.plan_decode_splits(batch, hkv, S) == {1: (1024, 32), 8: (1024, 32), 64: (1024, 8)}[batch]
     g = torch.Generator().manual_seed(batch)
     lens = [S - (0, 1, 15, 16, 17, 700, 0, 63)[i % 8] for i in range(batch)]
     sharp = {0: 4095 if batch > 1 else None, 1: 0, 2: 4096, 3: lens[3 % batch] - 1, 5: 1023, 6: 1024, 7: S // 2 + 17}
@@ -836,6 +836,12 @@ def test_attention_decode_at_the_longest_contexts_that_are_measured(batch, S):
         _i32(tables), 0, dh ** -0.5, max(lens),
     )
     torch.testing.assert_close(out.float().cpu(), torch.cat(wants), rtol=2 ** -7, atol=2 ** -7)
+    if batch == 64:  # and without splits
+        whole = ops.attention_decode(
+            torch.cat(qs).to(DEV), hq, hkv, dh, k_pages.to(DEV), v_pages.to(DEV), _i32(list(range(batch))), _i32([n - 1 for n in lens]),
+            _i32(tables), 0, dh ** -0.5, max(lens), split_size=S,
+        )
+        torch.testing.assert_close(whole.float().cpu(), torch.cat(wants), rtol=2 ** -7, atol=2 ** -7)
     if batch == 1:  # the one request again, with one key that outweighs the others, in turn at these places
         k_dev, v_dev = k_pages.to(DEV), v_pages.to(DEV)
         for far in (0, 1023, 1024, 20000, S - 65, S - 1):
@@ -857,7 +863,7 @@ def test_attention_decode_says_what_it_takes():
     assert not ops.decode_attention_supported(torch.bfloat16, 6, 3, 48)
     assert not ops.decode_attention_supported(torch.bfloat16, 16, 1, 256)
     assert ops.plan_decode_splits(8, 8, 8192) == (1024, 8)
-    assert ops.plan_decode_splits(64, 8, 8192) == (8192, 1)
+    assert ops.plan_decode_splits(64, 8, 8192) == (1024, 8) and ops.plan_decode_splits(64, 8, 4095) == (4095 + 1, 1)
     assert ops.plan_decode_splits(64, 8, 8192, uneven=True) == (512, 16)
     assert ops.plan_decode_splits(2, 8, 8192, uneven=True) == (512, 16)
     assert ops.plan_decode_splits(6, 8, 4096) == (448, 10) and ops.plan_decode_splits(6, 8, 4096, uneven=True) == (448, 10)  # what equal requests get is shorter still

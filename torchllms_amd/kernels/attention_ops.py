@@ -139,6 +139,12 @@ _DECODE_BLOCKS_PER_CU = {32: 3, 64: 3, 128: 2, 256: 1}
 _DECODE_FEW_PAIRS = 32
 
 
+#: from this many keys on no split is longer than ``_DECODE_LONGEST_SPLIT``: a launch of few long blocks ends when
+#: its slowest block does, and blocks that wait for a free CU even that out (alone, cold, planned -> capped, us: two
+#: requests of 32,768 keys 64 -> 55, four 107 -> 98, eight 199 -> 193; sixteen of 8,192 108 -> 101, sixty-four 382 ->
+#: 372; sixty-four of 2,176 keys lose 14% when cut, hence the threshold)
+_DECODE_LONG = 4096
+_DECODE_LONGEST_SPLIT = 1024
 DECODE_UNEVEN_SPLIT = 512  # keys: the longest split when requests differ much in length (measured with 64 requests of 128 to 4,608 tokens: 1 to 1.5% more tokens a second than with 1,024, 12% more than with 2,048)
 
 
@@ -151,7 +157,8 @@ def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, head_dim: i
     and its share of the merge; staying under the limit was the best choice or within 1% of it on
     average (at most 11%) over 1 to 100 requests of 700 to 20,000 tokens at each head size, where
     always aiming at 512 blocks lost 3 to 16% on average.  A batch with that many (request, kv
-    head) pairs or more is not split at all, if the requests are about equally long.
+    head) pairs or more is not split at all, if the requests are about equally long and hold fewer than
+    4,096 keys; from there on no split is longer than 1,024 keys.
 
     ``uneven``: the requests differ much in length.  Then all blocks of such a launch would be
     resident at once and stay where they were put, a CU with long requests' blocks working on
@@ -165,6 +172,8 @@ def plan_decode_splits(n_tokens: int, n_kv_heads: int, longest: int, head_dim: i
     limit = device_facts()[0] * per_cu
     want = max(limit // pairs, 1)
     split = -(-max(longest, 1) // want)
+    if longest >= _DECODE_LONG:
+        split = min(split, _DECODE_LONGEST_SPLIT)
     if uneven:
         split = min(split, DECODE_UNEVEN_SPLIT)
     split = max(-(-split // _DECODE_BLOCK_KEYS) * _DECODE_BLOCK_KEYS, _DECODE_MIN_SPLIT)
