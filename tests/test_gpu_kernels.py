@@ -909,6 +909,116 @@ def test_gemm_stream_glu_equals_the_product_followed_by_the_gate(m, f, k):
     torch.testing.assert_close(_ops().linear_glu(x, w).float(), ref, rtol=2 ** -6, atol=2 ** -6 * ref.abs().max().item())
 
 
+def _pieces_of_squares(rows: torch.Tensor, n_pieces: int) -> torch.Tensor:
+    """float32 [n_pieces, 16] whose columns add up to each row's sum of squares: the squares of the
+    elements dealt out to the pieces in turn; the columns past the last row hold rubbish."""
+    sq = rows.float() ** 2
+    pad = (-sq.shape[1]) % n_pieces
+    sq = torch.nn.functional.pad(sq, (0, pad))
+    out = torch.full((n_pieces, 16), float("nan"), device=rows.device)
+    out[:, : rows.shape[0]] = sq.reshape(sq.shape[0], -1, n_pieces).sum(1).T
+    return out
+
+
+@pytest.mark.parametrize("m, n, k", [(1, 4096, 4096), (8, 4096, 14336), (16, 300, 96), (9, 260, 688), (13, 2048, 1024), (3, 16, 8),
+                                     (5, 36, 136), (4, 2052, 128)])
+def test_gemm_stream_residual_adds_the_product_to_its_rows_and_leaves_their_sums_of_squares(m, n, k):
+    """The sum is the one the norm kernel would have formed from the stored product (product rounded,
+    added in 32-bit, rounded), bit for bit; beside it the same rows times the gain, and the squares
+    of the stored rows by 16 columns."""
+    torch.manual_seed(4)
+    x = torch.randn(m, k).bfloat16().to(DEV)
+    w = (torch.randn(n, k) * k ** -0.5).bfloat16().to(DEV)
+    h = (torch.randn(m, n) * torch.logspace(-1, 1, m)[:, None]).bfloat16().to(DEV)
+    gain = (0.3 + 2 * torch.rand(n)).bfloat16().to(DEV)
+    for waves in (0, 1, 2, 4, 8):
+        got, gained, sums = _ops().gemm_stream_residual(x, w, h, gain, waves=waves)
+        want = (h.float() + _ops().gemm_stream(x, w, torch.bfloat16, waves=waves).float()).bfloat16()
+        assert torch.equal(got, want), f"waves={waves}"
+        assert torch.equal(gained, (want.float() * gain.float()).bfloat16()), f"waves={waves}"
+        sq = torch.nn.functional.pad(want.float() ** 2, (0, (-n) % 16)).reshape(m, -1, 16).sum(-1)
+        assert sums.shape == (sq.shape[1], 16)
+        torch.testing.assert_close(sums[:, :m].T, sq, rtol=1e-5, atol=1e-30, msg=f"waves={waves}")
+    pending = _ops().PendingProduct(x, w, 0)
+    assert pending.shape == (m, n) and torch.equal(_ops().resolved(pending), _ops().gemm_stream(x, w))
+    rows, normed = pending.added_to(h, gain, 1e-3)
+    assert torch.equal(rows, want) and normed.rows is rows and normed.shape == (m, n)
+    # what the statistics stand for is the norm kernel's result on the new rows
+    assert torch.equal(_ops().resolved(normed), _ops().rmsnorm(want, gain, 1e-3))
+
+
+def test_gemm_stream_residual_says_its_limits():
+    from torchllms_amd.kernels.lib import KernelError
+
+    def z(*shape):
+        return torch.zeros(*shape, dtype=torch.bfloat16, device=DEV)
+
+    x = z(2, 64)
+    with pytest.raises(KernelError, match="multiple of 4"):
+        _ops().gemm_stream_residual(x, z(30, 64), z(2, 30), z(30))
+    with pytest.raises(KernelError, match="rows to add to"):
+        _ops().gemm_stream_residual(x, z(32, 64), z(3, 32), z(32))
+    with pytest.raises(KernelError, match="a gain of shape"):
+        _ops().gemm_stream_residual(x, z(32, 64), z(2, 32), z(31))
+    # the statistics must be those of the rows that are multiplied
+    norm = _ops().NormedRows(x, x.clone(), torch.ones(4, 16, device=DEV), 1e-5, z(64))
+    with pytest.raises(KernelError, match="do not belong"):
+        _ops().gemm_stream_glu(x, z(32, 64), norm=norm)
+
+
+@pytest.mark.parametrize("m, f, k, pieces", [(1, 4096, 1024, 64), (8, 1024, 4096, 256), (5, 100, 136, 9), (16, 688, 96, 6), (12, 24, 8, 1),
+                                             (3, 13, 264, 33), (16, 64, 2048, 300)])
+def test_gemm_stream_glu_applies_a_norm_from_the_rows_sums_of_squares(m, f, k, pieces):
+    """Rows of very different sizes, so another row's factor shows; an eps that counts for the small
+    rows; any number of pieces, more than the lanes of a row hold ahead included."""
+    torch.manual_seed(5)
+    eps = 1e-2
+    x = (torch.randn(m, k) * torch.logspace(-1.5, 1.5, m)[:, None]).bfloat16().to(DEV)
+    w = (torch.randn(2 * f, k) * k ** -0.5).bfloat16().to(DEV)
+    gain = (0.3 + 2 * torch.rand(k)).bfloat16().to(DEV)
+    norm = _ops().NormedRows(x, (x.float() * gain.float()).bfloat16(), _pieces_of_squares(x, pieces), eps, gain)
+    xn = x.float() * torch.rsqrt((x.float() ** 2).mean(-1, keepdim=True) + eps) * gain.float()
+    ref = torch.nn.functional.silu(xn @ w[:f].float().T) * (xn @ w[f:].float().T)
+    tol = dict(rtol=2 ** -6, atol=2 ** -6 * ref.abs().max().item())
+    torch.testing.assert_close(_ops().resolved(norm).float(), xn, rtol=2 ** -6, atol=1e-6)
+    for waves in (0, 1, 2, 4, 8):
+        for cols in (16, 8):
+            got = _ops().gemm_stream_glu(norm.gained, w, waves=waves, cols=cols, norm=norm)
+            torch.testing.assert_close(got.float(), ref, **tol, msg=f"waves={waves} cols={cols}")
+    torch.testing.assert_close(_ops().linear_glu(norm, w).float(), ref, **tol)
+
+
+@pytest.mark.parametrize("m, hq, hkv, dh, rot, page, k, pieces", [(8, 32, 8, 128, 128, 16, 4096, 256), (1, 4, 4, 64, 64, 16, 256, 16),
+                                                                   (13, 6, 3, 48, 24, 4, 136, 9), (16, 5, 1, 20, 0, 8, 64, 40), (3, 2, 2, 16, 16, 2, 8, 1)])
+def test_gemm_stream_qkv_applies_a_norm_from_the_rows_sums_of_squares(m, hq, hkv, dh, rot, page, k, pieces):
+    """Against the norm kernel followed by the fused projection: queries, and keys and values in their pages."""
+    torch.manual_seed(6)
+    eps = 1e-3
+    width = (hq + 2 * hkv) * dh
+    x = (torch.randn(m, k) * torch.logspace(-1.5, 1.5, m)[:, None]).bfloat16().to(DEV)
+    w = (torch.randn(width, k) * k ** -0.5).bfloat16().to(DEV)
+    gain = (0.3 + 2 * torch.rand(k)).bfloat16().to(DEV)
+    norm = _ops().NormedRows(x, (x.float() * gain.float()).bfloat16(), _pieces_of_squares(x, pieces), eps, gain)
+    pos = torch.randint(0, 9000, (m,))
+    inv_freq = plain.rope_inverse_frequencies(rot, 500000.0, None).to(DEV) if rot else None
+    table = _ops().rope_table(_i32(pos.tolist()), inv_freq) if rot else None
+    n_pages = 40
+    sm = _i32(torch.randperm(n_pages * page)[:m].tolist())
+    ka, va = _pages(n_pages, hkv, page, dh, torch.bfloat16)
+    qa = _ops().gemm_stream_qkv(_ops().rmsnorm(x, gain, eps), w, hq, hkv, dh, rot, table, ka, va, sm, page)
+    for waves in (0, 1, 2, 4, 8):
+        kb, vb = _pages(n_pages, hkv, page, dh, torch.bfloat16)
+        qb = _ops().gemm_stream_qkv(norm.gained, w, hq, hkv, dh, rot, table, kb, vb, sm, page, waves=waves, norm=norm)
+        tol = dict(rtol=2 ** -6, atol=2 ** -7 * qa[:, : hq * dh].float().abs().max().item())
+        torch.testing.assert_close(qb[:, : hq * dh].float(), qa[:, : hq * dh].float(), **tol, msg=f"waves={waves}")
+        torch.testing.assert_close(kb.float(), ka.float(), **tol)
+        torch.testing.assert_close(vb.float(), va.float(), **tol)
+    kc, vc = _pages(n_pages, hkv, page, dh, torch.bfloat16)
+    qc = _ops().qkv_rope_store(norm, w, None, hq, hkv, dh, _i32(pos.tolist()), inv_freq, rot, 0, table, kc, vc, sm, page)
+    torch.testing.assert_close(qc[:, : hq * dh].float(), qa[:, : hq * dh].float(), **tol)
+    torch.testing.assert_close(kc.float(), ka.float(), **tol)
+
+
 def test_gemm_stream_takes_strided_rows_and_says_its_limits():
     from torchllms_amd.kernels.lib import KernelError
 

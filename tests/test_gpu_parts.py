@@ -37,6 +37,7 @@ def _step(cache, rid, n_tokens, want=()):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_part_whole_and_in_portions(dtype):
     from torchllms_amd.config.spec import PartSpec
+    from torchllms_amd.kernels import ops
     from torchllms_amd.parts import MIXERS
 
     torch.manual_seed(0)
@@ -72,7 +73,8 @@ def test_attention_part_whole_and_in_portions(dtype):
         outs, at = [], 0
         for n in cuts:
             ctx = _step(cache, "r", n)
-            outs.append(part.forward(x[at : at + n].to(DEV).contiguous(), ctx, cache.kv_view(0)))
+            # (a mixer may leave its last product to whoever adds it to the residual stream)
+            outs.append(ops.resolved(part.forward(x[at : at + n].to(DEV).contiguous(), ctx, cache.kv_view(0))))
             cache.advance("r", n)
             at += n
         torch.testing.assert_close(torch.cat(outs).float().cpu(), want, **tol)
@@ -83,6 +85,7 @@ def test_attention_part_whole_and_in_portions(dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_feed_forward_norm_embedding_head_and_block(dtype):
     from torchllms_amd.config.spec import PartSpec
+    from torchllms_amd.kernels import ops
     from torchllms_amd.parts import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
 
     torch.manual_seed(1)
@@ -93,7 +96,7 @@ def test_feed_forward_norm_embedding_head_and_block(dtype):
     ffn.bind({k: v.to(DEV) for k, v in w.items()})
     x = torch.randn(S, D).to(dtype)
     want = plain.swiglu(x.float(), w["w1.weight"].float(), w["w3.weight"].float(), w["w2.weight"].float())
-    torch.testing.assert_close(ffn.forward(x.to(DEV), None).float().cpu(), want, **tol)
+    torch.testing.assert_close(ops.resolved(ffn.forward(x.to(DEV), None)).float().cpu(), want, **tol)
 
     norm = NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=1e-3)))
     nw = (1 + 0.2 * torch.randn(D)).to(dtype)
@@ -155,3 +158,66 @@ def test_pre_norm_block_matches_the_plain_block():
     cache2 = _ctx_and_cache(S, 3, 16, 4, torch.float32)
     h2, d2 = block.forward((x * 0.5).to(DEV), (x * 0.5).to(DEV), _step(cache2, "r", S), {"mixer": cache2.kv_view(0)})
     torch.testing.assert_close((h2 + d2).cpu(), want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("intermediate", [104, 100])
+def test_pre_norm_blocks_in_bfloat16_leave_their_norms_to_the_products(intermediate):
+    """On bfloat16 steps of few rows the products do the norms' work: the product that ends a branch
+    adds it to the residual stream and leaves the rows' statistics, the product that reads the rows
+    (times the norm's gain) applies them.  Two blocks
+    in a row against the plain blocks, with few rows (fused) and with many (the norm kernel), which
+    agree with each other too.  An intermediate size that the weight-streaming kernel does not take
+    (100, no multiple of 8) leaves that product, and the norm behind it, to the other kernels."""
+    from torchllms_amd.config.spec import PartSpec
+    from torchllms_amd.kernels import ops
+    from torchllms_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
+
+    torch.manual_seed(7)
+    D, hq, hkv, dh, eps = 80, 5, 1, 16, 1e-2
+    cfg = dict(hidden_size=D, num_attention_heads=hq, num_key_value_heads=hkv, head_dim=dh, intermediate_size=intermediate, rms_norm_eps=eps)
+    pos_spec = PartSpec("rope", dict(head_dim=dh, rotary_dim=dh, theta=10000.0, scaling=None))
+    blocks, weights = [], []
+    for _ in range(2):
+        block = BLOCKS["pre_norm"](
+            {
+                "mixer": MIXERS.build(PartSpec("attention", dict(hidden_size=D, num_heads=hq, num_kv_heads=hkv, head_dim=dh, qkv_bias=False,
+                                                                 softmax_scale=dh ** -0.5, window=0, position=pos_spec))),
+                "ffn": FEED_FORWARDS.build(PartSpec("swiglu", dict(hidden_size=D, intermediate_size=intermediate))),
+                "mixer_norm": NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=eps))),
+                "ffn_norm": NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=eps))),
+            }
+        )
+        # gains far from one, so that a gain applied twice or not at all shows
+        w = {n: ((torch.randn(s.shape) * 0.15) if s.init == "normal" else (0.3 + torch.rand(s.shape) * 2.0)).bfloat16() for n, s in block.param_specs().items()}
+        block.bind({k: v.to(DEV) for k, v in w.items()})
+        blocks.append(block)
+        weights.append({"wq": w["mixer.wq.weight"], "wk": w["mixer.wk.weight"], "wv": w["mixer.wv.weight"], "wo": w["mixer.wo.weight"],
+                        "w1": w["ffn.w1.weight"], "w3": w["ffn.w3.weight"], "w2": w["ffn.w2.weight"],
+                        "attention_norm": w["mixer_norm.weight"], "ffn_norm": w["ffn_norm.weight"]})
+    seen = []
+    for block in blocks:
+        for part in (block.mixer, block.ffn):
+            def spy(x, *rest, _inner=part.forward):
+                seen.append(type(x).__name__)
+                return _inner(x, *rest)
+            part.forward = spy
+
+    def run(S):
+        x = (torch.randn(S, D, generator=torch.Generator().manual_seed(S)) * 2).bfloat16()
+        want = x.float()
+        for lw in weights:
+            want = plain.block(want, {k: v.float() for k, v in lw.items()}, cfg, torch.arange(S), plain.rope_inverse_frequencies(dh, 10000.0, None))
+        h, delta = x.to(DEV), None
+        del seen[:]
+        for i, block in enumerate(blocks):
+            cache = _ctx_and_cache(S, hkv, dh, 4, torch.bfloat16)
+            h, delta = block.forward(h, delta, _step(cache, "r", S), {"mixer": cache.kv_view(0)})
+        got = h.float() + ops.resolved(delta).float()
+        torch.testing.assert_close(got.cpu(), want, rtol=0.05, atol=0.03 * want.abs().max().item())
+        return x, got.cpu(), list(seen)
+
+    x, few, kinds = run(7)
+    streamed = intermediate % 8 == 0  # whether the product back to the model's width takes the weight-streaming kernel
+    assert kinds == ["Tensor", "NormedRows", "NormedRows" if streamed else "Tensor", "NormedRows"]
+    _, many, kinds = run(40)
+    assert kinds == ["Tensor"] * 4

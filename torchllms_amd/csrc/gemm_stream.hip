@@ -26,6 +26,14 @@
 //     key heads are rotated by position (interleaved pairs, cosines and sines from a table), keys
 //     and values go straight into their cache pages, queries into C: the rotary kernel's work, done
 //     on the 32-bit sums after the rounding the unfused product would have applied.
+//   * a root-mean-square norm around the products, without a kernel of its own.  norm(x) W^T =
+//     ((x * gain) W^T) / sqrt(mean(x^2) + eps): the gain is applied to the rows, the factor per row
+//     commutes with the product.  The product that ends a branch adds its result to the residual rows
+//     (residual variant), stores the new rows, the new rows times the next norm's gain, and the sums
+//     of squares of the new rows, one per block of 16 columns; the gated and the query/key/value
+//     variants, which read the rows with the gain as A, add the pieces up (each lane a few, asked
+//     for before the walk along K, then lanes and waves in a fixed order) and scale their 32-bit sums
+//     by the factor before anything else happens to them.
 #include "common.h"
 #include "qkv_epilogue.h"
 
@@ -44,7 +52,27 @@ constexpr int kTileElems = 16 * kPitch;
 __device__ __forceinline__ short4_t lo_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[0], v[1]}); }
 __device__ __forceinline__ short4_t hi_half(u32x4_t v) { return __builtin_bit_cast(short4_t, u32x2_t{v[2], v[3]}); }
 
-enum Epilogue { kPlain = 0, kGated = 1, kQkv = 2, kGatedHalf = 3 };
+enum Epilogue { kPlain = 0, kGated = 1, kQkv = 2, kGatedHalf = 3, kResidual = 4 };
+
+// What the variants need that stand in for a norm.
+struct NormArgs {
+  // kGated, kGatedHalf, kQkv: the rows of A are to be read as A[m] / sqrt(sum[m] / width + eps);
+  // row_sums [n_row_sums][16] are pieces of sum[m] (piece by piece, the 16 rows side by side).  Null: A as it is.
+  const float* row_sums;
+  int n_row_sums;
+  float width, eps;
+  // kResidual: C = residual + product (the product rounded to bfloat16 first, then the sum),
+  // gained = C * gain (rounded; same leading dimension as C), and sums_out [blocks][16] receives
+  // sum(C[m][block's columns]^2) of the rounded rows.
+  const bf16_t* residual;
+  int ldr;
+  const bf16_t* gain;  // [N]
+  bf16_t* gained;
+  float* sums_out;
+};
+
+constexpr int kHeldSums = 16;  // pieces of a row's sum of squares that a lane asks for ahead
+constexpr int kSumRows = 16;   // rows side by side in a piece of the sums of squares
 
 // MR: groups of four rows of A that are fetched (M <= 4 * MR).  WAVES: waves per block = splits of K.
 // EPI kGated, kGatedHalf: W holds 2 N rows, gate rows then up rows; C[M, N] = silu(A gate^T) * (A up^T);
@@ -52,7 +80,7 @@ enum Epilogue { kPlain = 0, kGated = 1, kQkv = 2, kGatedHalf = 3 };
 template <int MR, int WAVES, typename OutT, int EPI>
 __global__ void __launch_bounds__(WAVES* kWave)
 gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-                   OutT* __restrict__ C, int ldc, int M, int N, int K, QkvArgs qa) {
+                   OutT* __restrict__ C, int ldc, int M, int N, int K, QkvArgs qa, NormArgs na) {
   constexpr bool GLU = EPI == kGated;
   constexpr int NW = GLU ? 2 : 1;  // W tiles per step
   // per wave: a tile of W [16][kPitch], then a tile of A [4 MR][kPitch] (rows past 4 MR are read as
@@ -102,6 +130,27 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   // the walk along K ends (asked for at the end, it would be one more round trip to memory)
   QkvOperands qkv_operands = {};
   if constexpr (EPI == kQkv) qkv_operands = qkv_fetch(min(n16, M - 1), n0 + 4 * g4, qa);
+
+  // so are the pieces of the rows' sums of squares (lane = row n16; the row's 4 * WAVES lanes share
+  // the pieces between them) and the residual variant's four elements of the rows it adds to.  The
+  // loads stand under no branch, so that nothing of theirs is waited for before the walk: without
+  // sums they read the start of A, which nobody uses.
+  constexpr bool NORMED = EPI == kGated || EPI == kGatedHalf || EPI == kQkv;
+  constexpr int kSumLanes = 4 * WAVES;
+  const int sum_first = 4 * wave + g4;
+  const bool normed = NORMED && na.row_sums != nullptr;
+  const float* sum_row = (normed ? na.row_sums : reinterpret_cast<const float*>(A)) + (normed && n16 < M ? n16 : 0);
+  const int sum_last = normed ? na.n_row_sums - 1 : 0;
+  float held[kHeldSums];
+  if constexpr (NORMED) {
+#pragma unroll
+    for (int j = 0; j < kHeldSums; ++j) held[j] = sum_row[(size_t)min(sum_first + j * kSumLanes, sum_last) * kSumRows];
+  }
+  u32x2_t residual = {0u, 0u}, gain = {0u, 0u};
+  if constexpr (EPI == kResidual) {
+    residual = *reinterpret_cast<const u32x2_t*>(na.residual + (size_t)min(n16, M - 1) * na.ldr + min(n0 + 4 * g4, N - 4));
+    gain = *reinterpret_cast<const u32x2_t*>(na.gain + min(n0 + 4 * g4, N - 4));
+  }
 
   auto fetch = [&](int st, u32x4_t* w, u32x4_t* a) {
     const int k0 = st * kStepK;
@@ -188,8 +237,18 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     consume(w0, a0);
   }
 
+  // this lane's share of its row's sum of squares: the pieces asked for at the start, then any further ones
+  float squares = 0.f;
+  if constexpr (NORMED) {
+    if (normed) {
+#pragma unroll
+      for (int j = 0; j < kHeldSums; ++j) squares += sum_first + j * kSumLanes <= sum_last ? held[j] : 0.f;
+      for (int p = sum_first + kHeldSums * kSumLanes; p <= sum_last; p += kSumLanes) squares += sum_row[(size_t)p * kSumRows];
+    }
+  }
+
   // acc[t][i] = C^T[n0 + 4 g4 + i][n16]; add the waves' shares in wave order (the wave's own W tile
-  // in LDS serves as its slot)
+  // in LDS serves as its slot, the lanes' shares of the sums of squares behind the products')
   if (WAVES > 1) {
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     float* slot = reinterpret_cast<float*>(w_lds);
@@ -197,6 +256,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     for (int t = 0; t < NW; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) slot[(t * kWave + lane) * 4 + i] = acc[t][i];
+    if constexpr (NORMED) slot[NW * kWave * 4 + lane] = squares;
     __syncthreads();
     if (wave != 0) return;
 #pragma unroll
@@ -209,6 +269,23 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
           sum += reinterpret_cast<const float*>(lds + (size_t)w2 * kWaveElems)[(t * kWave + lane) * 4 + i];
         acc[t][i] = sum;
       }
+    if constexpr (NORMED) {
+      squares = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < WAVES; ++w2) squares += reinterpret_cast<const float*>(lds + (size_t)w2 * kWaveElems)[NW * kWave * 4 + lane];
+    }
+  }
+  if constexpr (NORMED) {
+    // the four lanes of a row: 16 and 32 lanes apart (every lane of the wave is here)
+    squares += __shfl_xor(squares, 16, kWave);
+    squares += __shfl_xor(squares, 32, kWave);
+    if (normed) {
+      const float scale = 1.0f / sqrtf(squares / na.width + na.eps);
+#pragma unroll
+      for (int t = 0; t < NW; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[t][i] *= scale;
+    }
   }
   if constexpr (EPI == kQkv) {
     // the lane's four columns are channels of one head (N % 4 == 0)
@@ -234,6 +311,31 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
         C[(size_t)n16 * ldc + n] = from_f32<OutT>(act * u);
       }
     }
+  } else if constexpr (EPI == kResidual) {
+    // the lane's four columns n0 + 4 g4 .. + 3 of row n16 (N % 4 == 0): new row = residual + product
+    const int n = n0 + 4 * g4;
+    const bool mine = n16 < M && n < N;
+    float sq = 0.f;
+    uint32_t packed[2], packed_gained[2];
+    auto wide = [](uint32_t word, int i) { return __builtin_bit_cast(float, i % 2 ? word & 0xFFFF0000u : word << 16); };
+    auto bits = [](bf16_t v) { return (uint32_t)__builtin_bit_cast(uint16_t, v); };
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bf16_t sum = from_f32<bf16_t>(wide(residual[i / 2], i) + to_f32(from_f32<bf16_t>(acc[0][i])));
+      const float f = to_f32(sum);
+      sq += f * f;
+      const bf16_t with_gain = from_f32<bf16_t>(f * wide(gain[i / 2], i));
+      packed[i / 2] = i % 2 ? packed[i / 2] | (bits(sum) << 16) : bits(sum);
+      packed_gained[i / 2] = i % 2 ? packed_gained[i / 2] | (bits(with_gain) << 16) : bits(with_gain);
+    }
+    if (mine) {
+      *reinterpret_cast<u32x2_t*>(C + (size_t)n16 * ldc + n) = u32x2_t{packed[0], packed[1]};
+      *reinterpret_cast<u32x2_t*>(na.gained + (size_t)n16 * ldc + n) = u32x2_t{packed_gained[0], packed_gained[1]};
+    }
+    sq = mine ? sq : 0.f;
+    sq += __shfl_xor(sq, 16, kWave);
+    sq += __shfl_xor(sq, 32, kWave);
+    if (g4 == 0 && n16 < M) na.sums_out[(size_t)blockIdx.x * kSumRows + n16] = sq;
   } else if (n16 < M) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -253,7 +355,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
 
 template <int MR, int WAVES, typename OutT, int EPI>
 int launch_typed(const bf16_t* A, int lda, const bf16_t* W, int ldw, OutT* C, int ldc, int M, int N, int K,
-                 const QkvArgs& qa, hipStream_t stream) {
+                 const QkvArgs& qa, const NormArgs& na, hipStream_t stream) {
   const size_t lds = (size_t)WAVES * 2 * kTileElems * sizeof(bf16_t);
   static bool raised = false;  // blocks past 64 KB of LDS have to be allowed once per kernel
   if (lds > 64 * 1024 && !raised) {
@@ -264,33 +366,34 @@ int launch_typed(const bf16_t* A, int lda, const bf16_t* W, int ldw, OutT* C, in
   }
   constexpr int kCols = EPI == kGatedHalf ? kStrip / 2 : kStrip;  // columns of C per block
   const dim3 grid((N + kCols - 1) / kCols);
-  gemm_stream_kernel<MR, WAVES, OutT, EPI><<<grid, WAVES * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, qa);
+  gemm_stream_kernel<MR, WAVES, OutT, EPI><<<grid, WAVES * kWave, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, qa, na);
   return tl_check_launch("gemm_stream");
 }
 
 template <int MR, int WAVES>
 int launch(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N, int K,
-           int out_dtype, int epi, const QkvArgs& qa, hipStream_t stream) {
-  if (epi == kGated) return launch_typed<MR, WAVES, bf16_t, kGated>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
-  if (epi == kGatedHalf) return launch_typed<MR, WAVES, bf16_t, kGatedHalf>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
-  if (epi == kQkv) return launch_typed<MR, WAVES, bf16_t, kQkv>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
-  if (out_dtype == TL_BF16) return launch_typed<MR, WAVES, bf16_t, kPlain>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, stream);
-  return launch_typed<MR, WAVES, float, kPlain>(A, lda, W, ldw, (float*)C, ldc, M, N, K, qa, stream);
+           int out_dtype, int epi, const QkvArgs& qa, const NormArgs& na, hipStream_t stream) {
+  if (epi == kResidual) return launch_typed<MR, WAVES, bf16_t, kResidual>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, na, stream);
+  if (epi == kGated) return launch_typed<MR, WAVES, bf16_t, kGated>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, na, stream);
+  if (epi == kGatedHalf) return launch_typed<MR, WAVES, bf16_t, kGatedHalf>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, na, stream);
+  if (epi == kQkv) return launch_typed<MR, WAVES, bf16_t, kQkv>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, na, stream);
+  if (out_dtype == TL_BF16) return launch_typed<MR, WAVES, bf16_t, kPlain>(A, lda, W, ldw, (bf16_t*)C, ldc, M, N, K, qa, na, stream);
+  return launch_typed<MR, WAVES, float, kPlain>(A, lda, W, ldw, (float*)C, ldc, M, N, K, qa, na, stream);
 }
 
 template <int MR>
 int launch_waves(int waves, const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, int M, int N,
-                 int K, int out_dtype, int epi, const QkvArgs& qa, hipStream_t stream) {
+                 int K, int out_dtype, int epi, const QkvArgs& qa, const NormArgs& na, hipStream_t stream) {
   switch (waves) {
-    case 1: return launch<MR, 1>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
-    case 2: return launch<MR, 2>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
-    case 4: return launch<MR, 4>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
-    default: return launch<MR, 8>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
+    case 1: return launch<MR, 1>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, na, stream);
+    case 2: return launch<MR, 2>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, na, stream);
+    case 4: return launch<MR, 4>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, na, stream);
+    default: return launch<MR, 8>(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, epi, qa, na, stream);
   }
 }
 
 int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K, int out_dtype,
-        int waves, int epi, const QkvArgs& qa, hipStream_t stream) {
+        int waves, int epi, const QkvArgs& qa, const NormArgs& na, hipStream_t stream) {
   TL_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_stream: bad sizes M=%d N=%d K=%d", M, N, K);
   if (M > 16) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream: M=%d exceeds 16", M);
   if (K % 8) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream: K=%d is not a multiple of 8", K);
@@ -298,6 +401,18 @@ int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M,
   TL_REQUIRE(lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0,
              "gemm_stream: rows must start on 16-byte boundaries");
   TL_REQUIRE(out_dtype == TL_BF16 || out_dtype == TL_F32, "gemm_stream: out_dtype must be 0 or 1");
+  if (na.row_sums != nullptr) {
+    TL_REQUIRE(epi != kPlain && epi != kResidual, "gemm_stream: only the gated and the query/key/value variants scale their rows");
+    TL_REQUIRE(na.n_row_sums > 0 && na.width > 0.f && ((uintptr_t)na.row_sums % 4) == 0, "gemm_stream: bad sums of squares");
+  }
+  if (epi == kResidual) {
+    TL_REQUIRE(na.residual != nullptr && na.sums_out != nullptr && na.gain != nullptr && na.gained != nullptr,
+               "gemm_stream_residual: rows to add to, a gain and places for the results are needed");
+    if (N % 4) return tl_fail(TL_ERR_UNSUPPORTED, "gemm_stream_residual: N=%d is not a multiple of 4", N);
+    TL_REQUIRE(na.ldr >= N && na.ldr % 4 == 0 && ldc % 4 == 0 && ((uintptr_t)na.residual % 8) == 0 && ((uintptr_t)C % 8) == 0 &&
+                   ((uintptr_t)na.gain % 8) == 0 && ((uintptr_t)na.gained % 8) == 0,
+               "gemm_stream_residual: rows must start on 8-byte boundaries");
+  }
   if (M == 0) return TL_OK;
   if (waves == 0) {
     // enough waves to keep loads in flight on every CU: about 16 a CU (4,096 on 256 CUs), at least two steps each
@@ -311,9 +426,9 @@ int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M,
   TL_REQUIRE(waves == 1 || waves == 2 || waves == 4 || waves == 8, "gemm_stream: waves must be 1, 2, 4 or 8");
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
-  if (M <= 4) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
-  if (M <= 8) return launch_waves<2>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
-  return launch_waves<4>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, stream);
+  if (M <= 4) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, na, stream);
+  if (M <= 8) return launch_waves<2>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, na, stream);
+  return launch_waves<4>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, na, stream);
 }
 
 }  // namespace
@@ -323,30 +438,53 @@ int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M,
 // waves = 0 picks the number of K splits from the sizes.
 TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
                              int K, int out_dtype, int waves, hipStream_t stream) {
-  return run(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, waves, kPlain, QkvArgs{}, stream);
+  return run(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, waves, kPlain, QkvArgs{}, NormArgs{}, stream);
 }
 
 // The gated pair of products: W [2 N, K] = gate rows | up rows; C [M, N] bfloat16 =
 // silu(A gate^T) * (A up^T), rounded as the two products, the activation and the final product
 // would be if each were stored in bfloat16.  cols: 16 or 8 columns of C per block.
+// row_sums [n_row_sums][16] 32-bit or null: pieces of a sum of squares per row, as tl_gemm_stream_residual
+// leaves them; then row m of both products is scaled by 1 / sqrt(sum / K + eps) before the roundings.
 TL_EXPORT int tl_gemm_stream_glu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
-                                 int K, int waves, int cols, hipStream_t stream) {
+                                 int K, int waves, int cols, const float* row_sums, int n_row_sums, float eps,
+                                 hipStream_t stream) {
   TL_REQUIRE(cols == 8 || cols == 16, "gemm_stream_glu: cols must be 8 or 16");
-  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, cols == 8 ? kGatedHalf : kGated, QkvArgs{}, stream);
+  NormArgs na = {};
+  na.row_sums = row_sums; na.n_row_sums = n_row_sums; na.width = (float)K; na.eps = eps;
+  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, cols == 8 ? kGatedHalf : kGated, QkvArgs{}, na, stream);
+}
+
+// C [M, N] bfloat16 = residual [M, N] + A W^T (the product rounded to bfloat16, then the sum in
+// 32-bit, rounded); gained [M, N] (leading dimension ldc) = C * gain [N], rounded; and sums_out
+// [ceil(N / 16)][16] 32-bit = the sums of squares of the rows of C by blocks of 16 columns, the rows
+// side by side (only the first M of each 16 are written): what a root-mean-square norm of those
+// rows needs, for the product that reads `gained` next.  N a multiple of 4.
+TL_EXPORT int tl_gemm_stream_residual(const void* A, int lda, const void* W, int ldw, const void* residual, int ldr,
+                                      const void* gain, void* C, void* gained, int ldc, float* sums_out, int M,
+                                      int N, int K, int waves, hipStream_t stream) {
+  NormArgs na = {};
+  na.residual = (const bf16_t*)residual; na.ldr = ldr; na.gain = (const bf16_t*)gain; na.gained = (bf16_t*)gained;
+  na.sums_out = sums_out;
+  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, kResidual, QkvArgs{}, na, stream);
 }
 
 // The query/key/value projection with the rotary kernel's work in its epilogue.  W [(Hq + 2 Hkv) *
 // head_dim, K]; C [M, that width] receives the rotated queries (and keys and values when no pages are
 // given).  cos_sin [M][rotary_dim / 2][2]: cosine and sine of each row's position (interleaved pairs
 // only).  k_pages / v_pages [page][Hkv][page_size][head_dim]; slot_mapping [M].  head_dim % 4 == 0.
+// row_sums, n_row_sums, eps: as for tl_gemm_stream_glu.
 TL_EXPORT int tl_gemm_stream_qkv(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int K,
                                  int n_q_heads, int n_kv_heads, int head_dim, int rotary_dim,
                                  const float* cos_sin, void* k_pages, void* v_pages,
-                                 const int32_t* slot_mapping, int page_size, int waves, hipStream_t stream) {
+                                 const int32_t* slot_mapping, int page_size, int waves, const float* row_sums,
+                                 int n_row_sums, float eps, hipStream_t stream) {
   QkvArgs qa;
   const int rc = qkv_args("gemm_stream_qkv", n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages,
                           slot_mapping, page_size, C, ldc, &qa);
   if (rc != TL_OK) return rc;
   const int N = (n_q_heads + 2 * n_kv_heads) * head_dim;
-  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, kQkv, qa, stream);
+  NormArgs na = {};
+  na.row_sums = row_sums; na.n_row_sums = n_row_sums; na.width = (float)K; na.eps = eps;
+  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, kQkv, qa, na, stream);
 }

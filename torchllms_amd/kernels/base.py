@@ -39,7 +39,15 @@ def _i32(t: Optional[torch.Tensor], what: str) -> None:
         raise KernelError(f"{what} must be a contiguous int32 tensor")
 
 
-class SplitSums:
+class Unfinished:
+    """A result whose last kernel has not run yet, because the kernel that reads it can do that work
+    on the way.  ``resolve()`` runs it and returns the tensor; ``resolved(x)`` does so for anything."""
+
+    def resolve(self) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class SplitSums(Unfinished):
     """A matrix product that was split along K and not yet added up: ``partial`` float32
     [splits, rows, columns].  The product is the sum of the slices in their order, rounded to
     ``dtype``; ``rmsnorm`` takes it as ``delta`` and adds the slices while it reads them, which
@@ -61,6 +69,7 @@ class SplitSums:
 
 
 def resolved(x):
-    """``x`` as a tensor: a ``SplitSums`` is added up, a tensor is returned as it is.  For code that
-    does arithmetic of its own on what a mixer or feed-forward returned."""
-    return x.resolve() if isinstance(x, SplitSums) else x
+    """``x`` as a tensor: an ``Unfinished`` result (a ``SplitSums``, a ``PendingProduct``, ``NormedRows``)
+    is finished, a tensor is returned as it is.  For code that does arithmetic of its own on what a
+    norm, mixer or feed-forward returned."""
+    return x.resolve() if isinstance(x, Unfinished) else x

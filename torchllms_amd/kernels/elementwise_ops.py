@@ -12,6 +12,7 @@ from .base import (  # noqa: F401
     F32,
     KernelError,
     SplitSums,
+    Unfinished,
     _gpu,
     _i32,
     _ptr,
@@ -61,6 +62,8 @@ def rmsnorm(
         hidden = x.shape[-1]
         if x.dtype == torch.bfloat16 and hidden % 8 == 0 and hidden <= 8192 and delta.shape == tuple(x.shape):
             return _rmsnorm_split(x, weight, eps, delta, rows, return_sum)
+        delta = delta.resolve()
+    elif isinstance(delta, Unfinished):
         delta = delta.resolve()
     _gpu(x, weight, delta, rows)
     _i32(rows, "rows")

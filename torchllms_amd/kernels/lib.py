@@ -36,8 +36,9 @@ _CORE_SIGNATURES = {
     "tl_attention_generic_split": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
     "tl_gemm_f32": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
-    "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
-    "tl_gemm_stream_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _P],
+    "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _P],
+    "tl_gemm_stream_residual": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
+    "tl_gemm_stream_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _P, _I, _F, _P],
     "tl_gemm_wide": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P],
     "tl_gemm_wide_splits": [_I, _I],
     "tl_gemm_wide_reduce": [_P, _P, _I, _I, _I, _I, _I, _P],

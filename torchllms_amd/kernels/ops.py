@@ -5,7 +5,7 @@ assume, launches on torch's current HIP stream and raises ``KernelError`` when a
 Tensors must live on the GPU: there is no CPU path.  Only what parts and callers use is named here;
 a module's own helpers and tables stay in the module.
 
-``base``             dtype codes, argument checks, ``SplitSums``
+``base``             dtype codes, argument checks, ``Unfinished`` results (``SplitSums``)
 ``elementwise_ops``  embedding, RMS norm, rotary + cache write, gate, bias
 ``products``         matrix products and the measurement that picks their kernel
 ``attention_ops``    plain, decode and prefill attention with their launch plans
@@ -17,6 +17,7 @@ from .base import (  # noqa: F401
     F32,
     KernelError,
     SplitSums,
+    Unfinished,
     check,
     core,
     device_facts,
@@ -49,6 +50,9 @@ from .products import (  # noqa: F401
     gemm_stream,
     gemm_stream_glu,
     gemm_stream_qkv,
+    gemm_stream_residual,
+    NormedRows,
+    PendingProduct,
     gemm_wide,
     gemm_wide_glu,
     gemm_wide_qkv,

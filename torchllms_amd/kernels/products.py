@@ -13,6 +13,7 @@ from .base import (  # noqa: F401
     F32,
     KernelError,
     SplitSums,
+    Unfinished,
     _gpu,
     _i32,
     _ptr,
@@ -24,7 +25,7 @@ from .base import (  # noqa: F401
     resolved,
     variant,
 )
-from .elementwise_ops import add_bias_, rope_kv_write, rope_table, silu_mul  # noqa: F401
+from .elementwise_ops import add_bias_, rmsnorm, rope_kv_write, rope_table, silu_mul  # noqa: F401
 
 def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """``x @ w.T`` in true 32-bit arithmetic; x [m, k], w [n, k], both float32."""
@@ -64,6 +65,100 @@ def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
         )
     )
     return out
+
+
+class NormedRows(Unfinished):
+    """``rmsnorm(rows, weight, eps)`` of at most 16 bfloat16 rows, not yet computed: ``gained`` are the
+    rows times ``weight`` and ``sums`` float32 [pieces, 16] are pieces of each row's sum of squares
+    (the rows side by side, at most 16), as ``PendingProduct.added_to`` leaves them.  What is left of the norm is one factor per row,
+    which ``linear_glu`` and ``qkv_rope_store`` apply to the sums of ``gained @ w.T`` where the
+    weight-streaming kernel runs: norm(x) W^T = ((x * weight) W^T) / sqrt(mean(x^2) + eps)."""
+
+    def __init__(self, rows: torch.Tensor, gained: torch.Tensor, sums: torch.Tensor, eps: float, weight: torch.Tensor):
+        self.rows = rows
+        self.gained = gained
+        self.sums = sums
+        self.eps = float(eps)
+        self.weight = weight
+
+    @property
+    def shape(self):
+        return tuple(self.rows.shape)
+
+    @property
+    def dtype(self):
+        return self.rows.dtype
+
+    def resolve(self) -> torch.Tensor:
+        return rmsnorm(self.rows, self.weight, self.eps)
+
+    def kernel_args(self):
+        sums = self.sums
+        if sums.dtype != torch.float32 or sums.dim() != 2 or sums.shape[1] != 16 or not sums.is_contiguous() or self.gained.shape[0] > 16:
+            raise KernelError("the sums of squares do not belong to these rows")
+        return sums.data_ptr(), sums.shape[0], self.eps
+
+
+class PendingProduct(Unfinished):
+    """``x @ w.T`` for at most 16 bfloat16 rows, to be run by the weight-streaming kernel with ``waves``
+    splits of K, and not yet run: whoever adds it to the residual stream calls ``added_to`` and gets
+    the sum from the product's own kernel, with what the norm of the sum needs."""
+
+    def __init__(self, x: torch.Tensor, w: torch.Tensor, waves: int):
+        self.x = x
+        self.w = w
+        self.waves = waves
+
+    @property
+    def shape(self):
+        return (self.x.shape[0], self.w.shape[0])
+
+    @property
+    def dtype(self):
+        return self.x.dtype
+
+    def resolve(self) -> torch.Tensor:
+        return gemm_stream(self.x, self.w, self.x.dtype, self.waves)
+
+    def added_to(self, h: torch.Tensor, weight: torch.Tensor, eps: float):
+        """``(h + x @ w.T, NormedRows of it)`` for a norm with gain ``weight``."""
+        rows, gained, sums = gemm_stream_residual(self.x, self.w, h, weight, self.waves)
+        return rows, NormedRows(rows, gained, sums, eps, weight)
+
+
+def gemm_stream_residual(x: torch.Tensor, w: torch.Tensor, h: torch.Tensor, gain: torch.Tensor, waves: int = 0):
+    """``rows = h + x @ w.T`` for at most 16 bfloat16 rows (the product rounded to bfloat16 before the
+    sum, as if it had been stored), ``rows * gain``, and the sums of squares of ``rows`` by blocks of
+    16 columns (float32 [ceil(N / 16), 16]: block by block, the rows side by side, of which the first
+    ``len(rows)`` are filled)."""
+    _gpu(x, w, h, gain)
+    if any(t.dtype != torch.bfloat16 for t in (x, w, h, gain)):
+        raise KernelError("gemm_stream_residual takes bfloat16 tensors")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1:
+        raise KernelError(f"gemm_stream_residual: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
+    m, k = x.shape
+    n = w.shape[0]
+    if tuple(h.shape) != (m, n) or h.stride(1) != 1:
+        raise KernelError(f"gemm_stream_residual: rows to add to of shape {tuple(h.shape)}, the product has {(m, n)}")
+    if tuple(gain.shape) != (n,) or not gain.is_contiguous():
+        raise KernelError(f"gemm_stream_residual: a gain of shape {tuple(gain.shape)} for rows of {n} elements")
+    out = torch.empty((2, m, n), dtype=torch.bfloat16, device=x.device)  # the rows, and the rows times the gain
+    sums = torch.empty(((n + 15) // 16, 16), dtype=torch.float32, device=x.device)
+    check(
+        core().tl_gemm_stream_residual(
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), h.data_ptr(), h.stride(0), gain.data_ptr(),
+            out[0].data_ptr(), out[1].data_ptr(), n, sums.data_ptr(), m, n, k, waves, _stream(),
+        )
+    )
+    return out[0], out[1], sums
+
+
+def _norm_args(norm: Optional[NormedRows], x: torch.Tensor):
+    if norm is None:
+        return None, 0, 0.0
+    if norm.gained is not x:
+        raise KernelError("the sums of squares do not belong to these rows")
+    return norm.kernel_args()
 
 
 WIDE_MAX_ROWS = 128
@@ -179,11 +274,13 @@ def gemm_wide_qkv(
     return out
 
 
-def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0, cols: int = 16) -> torch.Tensor:
+def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0, cols: int = 16, norm: Optional[NormedRows] = None) -> torch.Tensor:
     """``silu(x @ gate.T) * (x @ up.T)`` for at most 16 rows of bfloat16 ``x`` and ``w`` [2F, K] =
     gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``.  ``cols``: 16
-    or 8 columns of the result per block (8: a launch shaped like the plain product's)."""
+    or 8 columns of the result per block (8: a launch shaped like the plain product's).  ``norm``:
+    ``NormedRows`` whose ``gained`` rows ``x`` is; the result is then that of the normed rows."""
     _gpu(x, w)
+    sums, n_sums, eps = _norm_args(norm, x)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("gemm_stream_glu takes bfloat16 tensors")
     if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or x.stride(1) != 1 or w.stride(1) != 1 or w.shape[0] % 2:
@@ -193,7 +290,8 @@ def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0, cols: int 
     out = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     check(
         core().tl_gemm_stream_glu(
-            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k, waves, cols, _stream(),
+            x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k, waves, cols, sums, n_sums, eps,
+            _stream(),
         )
     )
     return out
@@ -212,11 +310,14 @@ def gemm_stream_qkv(
     slot_mapping: Optional[torch.Tensor],
     page_size: int,
     waves: int = 0,
+    norm: Optional[NormedRows] = None,
 ) -> torch.Tensor:
     """The fused projection ``x @ w.T`` of at most 16 rows into query | key | value heads with the
     rotation (interleaved pairs, from the ``rope_table`` of the rows' positions) and the cache
     write in the kernel's epilogue.  Returns [n, (Hq + 2 Hkv) * dh] whose query part is rotated;
-    the key and value parts are only filled when no pages are given."""
+    the key and value parts are only filled when no pages are given.  ``norm``: ``NormedRows`` whose
+    ``gained`` rows ``x`` is; the result is then that of the normed rows."""
+    sums, n_sums, eps = _norm_args(norm, x)
     width = qkv_shapes("gemm_stream_qkv", x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size)
     m, k = x.shape
     out = torch.empty((m, width), dtype=torch.bfloat16, device=x.device)
@@ -224,7 +325,7 @@ def gemm_stream_qkv(
         core().tl_gemm_stream_qkv(
             x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, k,
             n_q_heads, n_kv_heads, head_dim, rotary_dim, _ptr(cos_sin), _ptr(k_pages), _ptr(v_pages),
-            _ptr(slot_mapping), page_size, waves, _stream(),
+            _ptr(slot_mapping), page_size, waves, sums, n_sums, eps, _stream(),
         )
     )
     return out
@@ -508,19 +609,30 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
     return run_choice(linear_choice(x, w), x, w, out_dtype)
 
 
-def linear_to_sum(x: torch.Tensor, w: torch.Tensor):
-    """``x @ w.T`` for a result that is only ever added to the residual stream by ``rmsnorm(...,
-    delta=...)``: a tensor, or ``SplitSums`` when the product was split along K, which that
-    ``rmsnorm`` adds up while it reads them."""
+def linear_to_sum(x: torch.Tensor, w: torch.Tensor, may_wait: bool = False):
+    """``x @ w.T`` for a result that is only ever added to the residual stream by a norm's
+    ``forward_add`` (after its ``delta(...)``) or by ``rmsnorm(..., delta=...)``: a tensor, or
+    ``SplitSums`` when the product was split along K, which that ``rmsnorm`` adds up while it reads
+    them.  With ``may_wait`` the product of the weight-streaming kernel is not run at all but handed
+    on as a ``PendingProduct``, so that the kernel can add it to the residual stream itself."""
     if x.dtype == torch.float32:
         return gemm_f32(x, w)
     _gpu(x, w)
-    return run_choice(linear_choice(x, w, "sum"), x, w, x.dtype, leave_split=True)
+    choice = linear_choice(x, w, "sum")
+    if may_wait and choice is not None and choice[0] == "stream" and w.dtype == torch.bfloat16 and w.shape[0] % 4 == 0:
+        return PendingProduct(x, w, choice[1])
+    return run_choice(choice, x, w, x.dtype, leave_split=True)
 
 
 def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """``silu(x @ gate.T) * (x @ up.T)`` for ``w`` [2F, K] = gate rows | up rows: one fused kernel
-    where one of the decode kernels serves the shape, else the product followed by the gate."""
+    where one of the decode kernels serves the shape, else the product followed by the gate.  ``x``
+    may be ``NormedRows``: the weight-streaming kernel applies them, for any other they are normed first."""
+    if isinstance(x, NormedRows):
+        choice = linear_choice(x.gained, w, "glu")
+        if choice is not None and choice[0] == "stream":
+            return gemm_stream_glu(x.gained, w, choice[1], choice[2] if len(choice) > 2 else 16, norm=x)
+        x = x.resolve()
     if x.dtype != torch.bfloat16:
         return silu_mul(linear(x, w))
     _gpu(x, w)
@@ -556,14 +668,23 @@ def qkv_rope_store(
     and values appended to their pages; returns the row-major [n, (Hq + 2 Hkv) * dh] buffer whose
     query part the attention kernels read.  Fused into the product's own kernels where one of the
     decode kernels serves it (at most 128 bfloat16 rows, no bias, interleaved pairs, head size a
-    multiple of 4), else product, bias and rotary kernels in turn."""
+    multiple of 4), else product, bias and rotary kernels in turn.  ``x`` may be ``NormedRows``: the
+    weight-streaming kernel applies them, for any other they are normed first."""
+    norm = None
+    if isinstance(x, NormedRows):
+        norm, x = x, x.gained
+        choice = linear_choice(x, w, "qkv")
+        fusable = bias is None and head_dim % 4 == 0 and (rotary_dim == 0 or (pairing == 0 and cos_sin is not None))
+        if not (fusable and choice is not None and choice[0] == "stream"):
+            norm, x = None, norm.resolve()
     if x.dtype == torch.bfloat16:
         _gpu(x, w)
         choice = linear_choice(x, w, "qkv")
         fusable = bias is None and head_dim % 4 == 0 and (rotary_dim == 0 or (pairing == 0 and cos_sin is not None))
         if fusable and choice is not None and choice[0] == "stream":
             return gemm_stream_qkv(
-                x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size, choice[1]
+                x, w, n_q_heads, n_kv_heads, head_dim, rotary_dim, cos_sin, k_pages, v_pages, slot_mapping, page_size, choice[1],
+                norm=norm,
             )
         # (a product that is not split ends without a second kernel, so the rotary kernel follows it)
         if fusable and choice is not None and choice[0] == "wide" and choice[2] > 1:

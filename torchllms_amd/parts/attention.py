@@ -32,6 +32,7 @@ class Attention(Mixer):
 
     #: every launch is fixed by the step's shape: a decode step may be recorded in a HIP graph
     graph_safe = True
+    takes_normed_rows = True
 
     def __init__(
         self,
@@ -115,7 +116,7 @@ class Attention(Mixer):
     def linear_weights(self):
         return [(self.wqkv, "qkv"), (self.wo, "sum")]
 
-    def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:
+    def forward(self, x, ctx, cache):
         n_kv_in_row = 0 if self.shares_kv else self.num_kv_heads
         rot = self.position.rotary_args()
         g = cache.group
@@ -149,4 +150,4 @@ class Attention(Mixer):
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
             ctx, g, self.window, self.softmax_scale,
         )
-        return ops.linear_to_sum(attn, self.wo)
+        return ops.linear_to_sum(attn, self.wo, may_wait=True)

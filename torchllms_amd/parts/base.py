@@ -69,6 +69,11 @@ class StateNeed:
 class Part:
     """Base of all parts."""
 
+    #: True if the part's ``forward`` also takes ``kernels.ops.NormedRows`` in place of its input tensor
+    #: (a norm whose statistics are known but not applied): it passes them to ``ops.linear_glu`` or
+    #: ``ops.qkv_rope_store``, which apply them on the way, or makes a tensor of them with ``ops.resolved``
+    takes_normed_rows = False
+
     #: True only if what the part launches depends on the step's shape alone (no value read back
     #: to the host, no launch whose size depends on data): a decode step is replayed from a HIP
     #: graph only when every part of the model says so
@@ -105,6 +110,10 @@ class Part:
 class Norm(Part):
     """y = norm(x).  ``forward_add`` fuses the residual sum that precedes the norm.
 
+    ``forward_add_for`` is what a block calls: it names the part that will read the norm's output, so a
+    norm may leave work to that part's kernels where the part has said that it takes it
+    (``Part.takes_normed_rows``).
+
     A mixer or feed-forward whose last matrix product was split along K may hand its result on as
     ``kernels.ops.SplitSums`` (the slices not yet added) instead of a tensor.  Whoever passes a delta
     to a norm passes it through ``norm.delta(...)`` first: a norm whose kernel adds the slices while it
@@ -125,6 +134,11 @@ class Norm(Part):
         if delta is not None:
             h = h + delta
         return h, self.forward(h)
+
+    def forward_add_for(self, reader: Part, h: torch.Tensor, delta):
+        """``forward_add`` for a block: ``delta`` is whatever the part before returned, ``reader`` the
+        only part that reads the normed rows."""
+        return self.forward_add(h, self.delta(delta))
 
     def forward_rows(self, h: torch.Tensor, delta: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
         """``norm((h + delta)[rows])`` for an int32 index vector ``rows``."""

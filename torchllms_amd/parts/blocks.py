@@ -15,8 +15,8 @@ class PreNormBlock(Block):
     SLOTS = {"mixer_norm": "norm", "mixer": "mixer", "ffn_norm": "norm", "ffn": "feed_forward"}
 
     def forward(self, h, delta, ctx, cache):
-        h, y = self.mixer_norm.forward_add(h, self.mixer_norm.delta(delta))
+        h, y = self.mixer_norm.forward_add_for(self.mixer, h, delta)
         a = self.mixer.forward(y, ctx, cache["mixer"])
-        h, y = self.ffn_norm.forward_add(h, self.ffn_norm.delta(a))
+        h, y = self.ffn_norm.forward_add_for(self.ffn, h, a)
         f = self.ffn.forward(y, ctx)
         return h, f

@@ -16,6 +16,7 @@ class SwiGLU(FeedForward):
     (reference: torchllms/models/networks.py:592-605)."""
 
     graph_safe = True
+    takes_normed_rows = True
 
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size = hidden_size
@@ -35,5 +36,5 @@ class SwiGLU(FeedForward):
     def linear_weights(self):
         return [(self.w13, "glu"), (self.w2, "sum")]
 
-    def forward(self, x: torch.Tensor, ctx) -> torch.Tensor:
-        return ops.linear_to_sum(ops.linear_glu(x, self.w13), self.w2)
+    def forward(self, x, ctx):
+        return ops.linear_to_sum(ops.linear_glu(x, self.w13), self.w2, may_wait=True)

@@ -41,5 +41,11 @@ class RMSNorm(Norm):
             return h, ops.rmsnorm(h, self.weight, self.eps)
         return ops.rmsnorm(h, self.weight, self.eps, delta=delta, return_sum=True)
 
+    def forward_add_for(self, reader, h: torch.Tensor, delta):
+        if isinstance(delta, ops.PendingProduct) and getattr(reader, "takes_normed_rows", False) and self.weight.dtype == torch.bfloat16:
+            # the product's own kernel adds it to h and leaves the rows' statistics, which the reader's kernel applies
+            return delta.added_to(h, self.weight, self.eps)
+        return self.forward_add(h, delta)
+
     def forward_rows(self, h: torch.Tensor, delta: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
         return ops.rmsnorm(h, self.weight, self.eps, delta=delta, rows=rows)
