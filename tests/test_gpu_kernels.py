@@ -988,6 +988,38 @@ def test_gemm_stream_glu_applies_a_norm_from_the_rows_sums_of_squares(m, f, k, p
     torch.testing.assert_close(_ops().linear_glu(norm, w).float(), ref, **tol)
 
 
+def test_normed_rows_are_normed_first_where_another_kernel_serves_the_shape():
+    """``linear_glu`` and ``qkv_rope_store`` given ``NormedRows`` for a matrix that the table sends to the
+    library: the norm kernel runs on the rows, then whatever serves the shape."""
+    from torchllms_amd.kernels import products
+
+    torch.manual_seed(8)
+    m, k, f, eps = 5, 64, 48, 1e-3
+    x = torch.randn(m, k).bfloat16().to(DEV)
+    gain = (0.5 + torch.rand(k)).bfloat16().to(DEV)
+    w = (torch.randn(2 * f, k) * k ** -0.5).bfloat16().to(DEV)
+    norm = _ops().NormedRows(x, (x.float() * gain.float()).bfloat16(), _pieces_of_squares(x, 4), eps, gain)
+    keys = [(2 * f, k, products.row_bucket(m), use) for use in ("glu", "qkv")]
+    saved = {key: products.LINEAR_CHOICE.get(key) for key in keys}
+    try:
+        for key in keys:
+            products.LINEAR_CHOICE[key] = None
+        y = _ops().rmsnorm(x, gain, eps)
+        assert torch.equal(_ops().linear_glu(norm, w), _ops().silu_mul(torch.nn.functional.linear(y, w)))
+        pos = _i32(list(range(m)))
+        inv_freq = plain.rope_inverse_frequencies(16, 10000.0, None).to(DEV)
+        table = _ops().rope_table(pos, inv_freq)
+        got = _ops().qkv_rope_store(norm, w, None, 2, 2, 16, pos, inv_freq, 16, 0, table, None, None, None, 0)
+        want = _ops().qkv_rope_store(y, w, None, 2, 2, 16, pos, inv_freq, 16, 0, table, None, None, None, 0)
+        assert torch.equal(got, want)
+    finally:
+        for key, choice in saved.items():
+            if choice is None:
+                products.LINEAR_CHOICE.pop(key, None)
+            else:
+                products.LINEAR_CHOICE[key] = choice
+
+
 @pytest.mark.parametrize("m, hq, hkv, dh, rot, page, k, pieces", [(8, 32, 8, 128, 128, 16, 4096, 256), (1, 4, 4, 64, 64, 16, 256, 16),
                                                                    (13, 6, 3, 48, 24, 4, 136, 9), (16, 5, 1, 20, 0, 8, 64, 40), (3, 2, 2, 16, 16, 2, 8, 1)])
 def test_gemm_stream_qkv_applies_a_norm_from_the_rows_sums_of_squares(m, hq, hkv, dh, rot, page, k, pieces):
