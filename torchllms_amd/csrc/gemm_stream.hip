@@ -71,7 +71,6 @@ struct NormArgs {
   float* sums_out;
 };
 
-constexpr int kHeldSums = 16;  // pieces of a row's sum of squares that a lane asks for ahead
 constexpr int kSumRows = 16;   // rows side by side in a piece of the sums of squares
 
 // MR: groups of four rows of A that are fetched (M <= 4 * MR).  WAVES: waves per block = splits of K.
@@ -131,20 +130,27 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   QkvOperands qkv_operands = {};
   if constexpr (EPI == kQkv) qkv_operands = qkv_fetch(min(n16, M - 1), n0 + 4 * g4, qa);
 
-  // so are the pieces of the rows' sums of squares (lane = row n16; the row's 4 * WAVES lanes share
-  // the pieces between them) and the residual variant's four elements of the rows it adds to.  The
-  // loads stand under no branch, so that nothing of theirs is waited for before the walk: without
-  // sums they read the start of A, which nobody uses.
+  // so are the pieces of the rows' sums of squares and the residual variant's four elements of the
+  // rows it adds to.  The pieces of the 4 MR rows that the block may have are shared out over all its
+  // lanes: lane l of a wave takes row l % (4 MR), and the lanes of a row take its pieces in turn (eight
+  // each cover 256 pieces with eight rows and four waves, or sixteen rows and eight).  The loads stand
+  // under no branch, so that nothing of theirs is waited for before the walk: without sums they
+  // read the start of A, which nobody uses.
   constexpr bool NORMED = EPI == kGated || EPI == kGatedHalf || EPI == kQkv;
-  constexpr int kSumLanes = 4 * WAVES;
-  const int sum_first = 4 * wave + g4;
+  // pieces that a lane asks for ahead (any others it fetches at the end, and waits): with sixteen rows the
+  // registers allow fewer blocks a CU anyway, and sixteen pieces cover 256 with four waves
+  constexpr int kHeldSums = MR == 4 ? 16 : 8;
+  constexpr int kSumSide = 4 * MR;                       // rows side by side in the lanes of a wave
+  constexpr int kSumLanes = (kWave / kSumSide) * WAVES;  // lanes of the block that share a row's pieces
+  const int sum_first = lane / kSumSide + (kWave / kSumSide) * wave;
   const bool normed = NORMED && na.row_sums != nullptr;
-  const float* sum_row = (normed ? na.row_sums : reinterpret_cast<const float*>(A)) + (normed && n16 < M ? n16 : 0);
+  const float* sum_base = normed ? na.row_sums : reinterpret_cast<const float*>(A);
+  const uint32_t sum_row = normed && lane % kSumSide < M ? lane % kSumSide : 0;
   const int sum_last = normed ? na.n_row_sums - 1 : 0;
   float held[kHeldSums];
   if constexpr (NORMED) {
 #pragma unroll
-    for (int j = 0; j < kHeldSums; ++j) held[j] = sum_row[(size_t)min(sum_first + j * kSumLanes, sum_last) * kSumRows];
+    for (int j = 0; j < kHeldSums; ++j) held[j] = sum_base[(uint32_t)min(sum_first + j * kSumLanes, sum_last) * kSumRows + sum_row];
   }
   u32x2_t residual = {0u, 0u}, gain = {0u, 0u};
   if constexpr (EPI == kResidual) {
@@ -204,9 +210,29 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   // before its use cover both paths, that is, wait for the prefetch itself.  The last one or two
   // steps stand behind the loop, so that nothing is fetched that nobody uses (with two to four
   // steps a wave, as in the products with few columns, one spare fetch was a fifth of all).
+  // This lane's share of its row's sum of squares.  The pieces asked for at the start are added up as
+  // soon as the first tile of W has come (loads return in the order they were asked for, so the pieces
+  // are there too and nothing new is waited for), so that they hold no registers through the rest of
+  // the walk: registers decide between one block a CU and two.
+  float squares = 0.f;
+  auto add_held = [&]() {
+    if constexpr (NORMED) {
+#pragma unroll
+      for (int j = 0; j < kHeldSums; ++j) squares += normed && sum_first + j * kSumLanes <= sum_last ? held[j] : 0.f;
+      asm volatile("" : "+v"(squares));  // here, not wherever the result is used
+    }
+  };
   if (nst > 0) {
     fetch(step_of(0), w0, a0);
     int i = 0;
+    if (nst > 2) {  // the loop's first trip, with the pieces added in its middle
+      fetch(step_of(1), w1, a1);
+      consume(w0, a0);
+      add_held();
+      fetch(step_of(2), w0, a0);
+      consume(w1, a1);
+      i = 2;
+    }
     for (; i + 2 < nst; i += 2) {
       fetch(step_of(i + 1), w1, a1);
       consume(w0, a0);
@@ -237,14 +263,10 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     consume(w0, a0);
   }
 
-  // this lane's share of its row's sum of squares: the pieces asked for at the start, then any further ones
-  float squares = 0.f;
-  if constexpr (NORMED) {
-    if (normed) {
-#pragma unroll
-      for (int j = 0; j < kHeldSums; ++j) squares += sum_first + j * kSumLanes <= sum_last ? held[j] : 0.f;
-      for (int p = sum_first + kHeldSums * kSumLanes; p <= sum_last; p += kSumLanes) squares += sum_row[(size_t)p * kSumRows];
-    }
+  if (nst <= 2) add_held();
+  if constexpr (NORMED) {  // pieces beyond those asked for at the start (more than eight or sixteen for each of a row's lanes)
+    if (normed)
+      for (int p = sum_first + kHeldSums * kSumLanes; p <= sum_last; p += kSumLanes) squares += sum_base[(uint32_t)p * kSumRows + sum_row];
   }
 
   // acc[t][i] = C^T[n0 + 4 g4 + i][n16]; add the waves' shares in wave order (the wave's own W tile
@@ -276,9 +298,9 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
     }
   }
   if constexpr (NORMED) {
-    // the four lanes of a row: 16 and 32 lanes apart (every lane of the wave is here)
-    squares += __shfl_xor(squares, 16, kWave);
-    squares += __shfl_xor(squares, 32, kWave);
+    // the lanes of a row lie 4 MR apart (every lane of the wave is here); lane n16 < 4 MR then holds row n16's sum
+#pragma unroll
+    for (int apart = kSumSide; apart < kWave; apart *= 2) squares += __shfl_xor(squares, apart, kWave);
     if (normed) {
       const float scale = 1.0f / sqrtf(squares / na.width + na.eps);
 #pragma unroll
