@@ -368,7 +368,9 @@ class Engine:
         step is queued behind the sampling; nothing waits.  The caller vouches for the tokens (the
         sampling kernel returns token ids) and has to cope with a request that turns out to have
         ended with the token it is fed here: its row is then wasted, the other rows are as good
-        as any.  None, with nothing run, when the preparation does not fit."""
+        as any.  None, with nothing run, when the preparation does not fit.  The logits returned are
+        the recording's own: they hold until the engine's next step is queued, which is long enough
+        for whoever queues the sampling first."""
         last = self._last_decode
         if last is None or last[2] is not prepared.previous or prepared.epoch != self.cache.epoch:
             return None
@@ -376,7 +378,7 @@ class Engine:
             return None
         if token_ids.dtype != torch.int32 or token_ids.numel() != len(prepared.rids) or token_ids.device != prepared.graph.dev.device:
             return None
-        logits = prepared.graph.launch(token_ids)
+        logits = prepared.graph.launch(token_ids, lend=True)
         for rid in prepared.rids:
             self.cache.advance(rid, 1)
         self._last_decode = (prepared.rids, prepared.wants, prepared.layout, self.cache.epoch)

@@ -51,6 +51,9 @@ class Sampler:
                 top_k = torch.tensor([p.top_k or 0 for p in params], dtype=torch.int32, device=dev)
             self._key, self._fixed = key, (temperature, seeds, top_k)
         temperature, seeds, top_k = self._fixed
+        if self._counters is not None and self._counters.device == dev and self._counters.numel() >= n and all(p.temperature == 0 for p in params):
+            # greedy rows draw nothing: the counters are not read, so none are sent
+            return ops.sample(logits, temperature, seeds, self._counters[:n], top_k)
         if self._pinned is None or self._pinned.numel() < n or self._counters.device != dev:
             self._pinned = torch.empty((max(n, 64),), dtype=torch.int64, pin_memory=True)
             self._counters = torch.empty((max(n, 64),), dtype=torch.int64, device=dev)
