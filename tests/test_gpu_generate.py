@@ -118,11 +118,27 @@ def test_preparing_the_next_step_ahead_changes_no_token(model_b, precision):
     steps = llm.last_stats["steps"]
     assert any(r.stop_reason is not None for r in want) and any(r.stop_reason is None for r in want)
     llm.look_ahead = True
-    got = llm.generate(prompt_token_ids=prompts, temperature=0.9, max_new_tokens=60, seed=5, stop_token_ids=stops)
+    # a step launched ahead has its tokens written by the sampling kernel where it reads them: no copy, and the plan
+    # goes up without them
+    from torchllms_amd.engine.graphs import DecodeGraph
+
+    in_place = []
+    upload = DecodeGraph._upload
+
+    def counting(self, but_tokens=0):
+        in_place.append(but_tokens)
+        return upload(self, but_tokens)
+
+    DecodeGraph._upload = counting
+    try:
+        got = llm.generate(prompt_token_ids=prompts, temperature=0.9, max_new_tokens=60, seed=5, stop_token_ids=stops)
+    finally:
+        DecodeGraph._upload = upload
     assert [r.token_ids for r in got] == [r.token_ids for r in want]
     assert [r.stop_reason for r in got] == [r.stop_reason for r in want]
     assert llm.last_stats["steps"] == steps and llm.last_stats["prepared_steps"] > steps // 3
     assert llm.last_stats["launched_ahead"] > steps // 4  # queued behind the sampling, before the host had the tokens
+    assert sum(1 for n in in_place if n > 0) == llm.last_stats["launched_ahead"]
     llm.engine.cache.check_invariants()
     assert llm.engine.cache.live == []
 

@@ -55,6 +55,11 @@ class PreparedDecode:
     def __init__(self, rids, wants, previous, layout, graph, epoch):
         self.rids, self.wants, self.previous, self.layout, self.graph, self.epoch = rids, wants, previous, layout, graph, epoch
 
+    def token_section(self) -> torch.Tensor:
+        """int32 [requests] on the device: where the step reads its token ids.  A sampling kernel may write
+        them there; ``Engine.step_prepared_on_device`` given this tensor copies nothing."""
+        return self.graph.token_section(len(self.rids))
+
 
 class Engine:
     def __init__(

@@ -74,8 +74,17 @@ class DecodeGraph:
         off = self.offsets[0]
         self.host_np[off : off + len(tokens)] = tokens
 
-    def _upload(self) -> None:
-        self.dev.copy_(self.host, non_blocking=True)
+    def token_section(self, n: int) -> torch.Tensor:
+        """Where the recording reads the step's first ``n`` token ids: whoever produces them on the
+        device may write them there and hand this tensor to ``launch``."""
+        off = self.offsets[0]
+        return self.dev[off : off + n]
+
+    def _upload(self, but_tokens: int = 0) -> None:
+        """The packed plan to the device; without its first ``but_tokens`` token ids if they are there already."""
+        start = self.offsets[0] + but_tokens if but_tokens else 0
+        assert self.offsets[0] == 0  # the token ids lead the buffer
+        self.dev[start:].copy_(self.host[start:], non_blocking=True)
         self.copied.record()
 
     def _load(self, layout: StepLayout) -> None:
@@ -117,13 +126,20 @@ class DecodeGraph:
     def launch(self, tokens_on_device: torch.Tensor = None, lend: bool = False) -> torch.Tensor:
         """Upload the packed plan and replay.  ``tokens_on_device``: the step's token ids as an int32
         tensor on the device, which take the place of the plan's (they need not be known on the host:
-        the copy is queued behind whatever produces them).  ``lend``: return the recording's own logits,
+        the copy is queued behind whatever produces them; none is needed when they were written into
+        ``token_section`` itself).  ``lend``: return the recording's own logits,
         which the next replay overwrites, instead of a copy (a copy of 33 MB at 64 rows, and one more
         small launch between two steps at any size)."""
-        self._upload()
-        if tokens_on_device is not None:
-            off = self.offsets[0]
-            self.dev[off : off + tokens_on_device.numel()].copy_(tokens_on_device)
+        if tokens_on_device is None:
+            self._upload()
+        else:
+            n = tokens_on_device.numel()
+            section = self.token_section(n)
+            if tokens_on_device.data_ptr() == section.data_ptr():  # written in place: nothing to copy
+                self._upload(but_tokens=n)
+            else:
+                self._upload()
+                section.copy_(tokens_on_device)
         self.graph.replay()
         self.replays += 1
         return self.logits if lend else self.logits.clone()

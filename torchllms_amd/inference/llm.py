@@ -91,10 +91,16 @@ class GenerationLoop:
                 counters = [len(r.output) for r in sampling]
                 next_logits = None
                 if prepare is not None and launch is not None and _decodes_on(plan):
-                    pending = launch(logits, [r.params for r in sampling], counters)
-                    arriving = self._send_home(pending) if launch_ahead is not None else None
                     prepared = prepare()  # the GPU is busy with the step meanwhile
-                    if prepared is not None and arriving is not None and not sched.may_admit_before_a_request_ends():
+                    go_ahead = prepared is not None and launch_ahead is not None and not sched.may_admit_before_a_request_ends()
+                    # a step that is launched ahead gets its tokens where it reads them, straight from the sampling kernel
+                    section = getattr(prepared, "token_section", None) if go_ahead else None
+                    if section is not None:
+                        pending = launch(logits, [r.params for r in sampling], counters, out=section())
+                    else:
+                        pending = launch(logits, [r.params for r in sampling], counters)
+                    arriving = self._send_home(pending) if launch_ahead is not None else None
+                    if go_ahead:
                         next_logits = launch_ahead(prepared, [e.request.rid for e in plan.entries], pending)
                     if next_logits is not None:
                         prepared = None  # used

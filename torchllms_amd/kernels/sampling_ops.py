@@ -29,11 +29,13 @@ def sample(
     seeds: torch.Tensor,
     steps: torch.Tensor,
     top_k: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """One token per row of float32 ``logits`` [n, vocab]; see csrc/sampling.hip for the rule.  Without
     top-k and with few rows, several blocks share a row (``sample_chunks``); the tokens are the same.
-    ``temperature`` float32 [n]; ``seeds``/``steps`` int64 [n] (read as unsigned); ``top_k`` int32 [n]."""
-    _gpu(logits, temperature, seeds, steps, top_k)
+    ``temperature`` float32 [n]; ``seeds``/``steps`` int64 [n] (read as unsigned); ``top_k`` int32 [n].
+    ``out``: int32 [n] on the same device to receive the tokens (else a new tensor)."""
+    _gpu(logits, temperature, seeds, steps, top_k, out)
     _i32(top_k, "top_k")
     if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
         raise KernelError("sample: logits must be a row-major float32 matrix")
@@ -45,7 +47,10 @@ def sample(
             raise KernelError(f"sample: {what} must be int64 [n]")
     if top_k is not None and top_k.numel() != n:
         raise KernelError("sample: top_k must be int32 [n]")
-    out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    if out is None:
+        out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    elif out.dtype != torch.int32 or tuple(out.shape) != (n,) or not out.is_contiguous() or out.device != logits.device:
+        raise KernelError("sample: out must be int32 [n] beside the logits")
     chunks = sample_chunks(n, vocab) if top_k is None and logits.stride(0) % 4 == 0 and logits.data_ptr() % 16 == 0 else 1
     if chunks > 1:
         candidates = torch.empty((n, chunks, 2), dtype=torch.int32, device=logits.device)

@@ -32,10 +32,10 @@ class Sampler:
     def __call__(self, logits: torch.Tensor, params: Sequence[SamplingParams], steps: Sequence[int]) -> List[int]:
         return self.launch(logits, params, steps).tolist()
 
-    def launch(self, logits: torch.Tensor, params: Sequence[SamplingParams], steps: Sequence[int]) -> torch.Tensor:
+    def launch(self, logits: torch.Tensor, params: Sequence[SamplingParams], steps: Sequence[int], out: torch.Tensor = None) -> torch.Tensor:
         """Queue the sampling behind the step's kernels and return the token ids as a tensor on the
         device: the host goes on until it asks for them (``.tolist()``), which it has to do before
-        the next call."""
+        the next call.  ``out``: where on the device the token ids are to go (int32, one per row)."""
         n = logits.shape[0]
         if n == 0:
             return torch.empty((0,), dtype=torch.int32)
@@ -53,14 +53,14 @@ class Sampler:
         temperature, seeds, top_k = self._fixed
         if self._counters is not None and self._counters.device == dev and self._counters.numel() >= n and all(p.temperature == 0 for p in params):
             # greedy rows draw nothing: the counters are not read, so none are sent
-            return ops.sample(logits, temperature, seeds, self._counters[:n], top_k)
+            return ops.sample(logits, temperature, seeds, self._counters[:n], top_k, out=out)
         if self._pinned is None or self._pinned.numel() < n or self._counters.device != dev:
             self._pinned = torch.empty((max(n, 64),), dtype=torch.int64, pin_memory=True)
             self._counters = torch.empty((max(n, 64),), dtype=torch.int64, device=dev)
         self._pinned[:n] = torch.as_tensor([int(s) for s in steps], dtype=torch.int64)
         counters = self._counters[:n]
         counters.copy_(self._pinned[:n], non_blocking=True)
-        return ops.sample(logits, temperature, seeds, counters, top_k)
+        return ops.sample(logits, temperature, seeds, counters, top_k, out=out)
 
 
 def _as_i64(x: int) -> int:
