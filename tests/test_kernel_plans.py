@@ -68,7 +68,9 @@ def test_the_tuned_table_decides_per_shape_rows_and_use():
 def test_which_candidates_are_charged_a_kernel_of_their_own_for_the_second_half():
     stream, whole, split = ("stream", 4), ("wide", 2, 1, 3), ("wide", 1, 4, 3)
     for choice in (None, stream, whole, split):
-        assert products.fuses_tail(choice, "plain") and products.fuses_tail(choice, "sum")
+        assert products.fuses_tail(choice, "plain")
+    # the streaming product adds itself to the residual rows and leaves the norm's statistics; the library cannot
+    assert [products.fuses_tail(c, "sum") for c in (None, stream, whole, split)] == [False, True, True, True]
     assert [products.fuses_tail(c, "glu") for c in (None, stream, whole, split)] == [False, True, True, False]
     assert [products.fuses_tail(c, "qkv") for c in (None, stream, whole, split)] == [False, True, False, True]
 

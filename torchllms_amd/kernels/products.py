@@ -389,10 +389,15 @@ def row_bucket(m: int) -> int:
 
 
 def fuses_tail(choice, use: str) -> bool:
-    """Whether the kernel of ``choice`` does the second half of ``use`` itself."""
-    if use in ("plain", "sum") or choice is None:
-        return use in ("plain", "sum")
-    if choice[0] == "stream":
+    """Whether the kernel of ``choice`` does the second half of ``use`` itself.  For "sum" that half is the
+    sum with the residual rows and the statistics of the norm behind it: the streaming kernel does both
+    (``PendingProduct``), a split product leaves its slices to the norm kernel that runs anyway, the library
+    needs that kernel where the streaming product would not."""
+    if use == "plain":
+        return True
+    if choice is None:
+        return False
+    if choice[0] == "stream" or use == "sum":
         return True
     return choice[2] == 1 if use == "glu" else choice[2] > 1  # the gate ends a whole product, the rotation a split one
 
@@ -485,7 +490,8 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
     fastest on this GPU, and remember it.  ``weights``: the model's tensors of that shape; ``use``:
     one of ``LINEAR_USES``.  "glu" times the whole gated product as ``linear_glu`` would run it,
     "sum" a product that may stay split; for "qkv" the plain product is timed and a candidate that
-    cannot take rotation and cache write into itself is charged the kernel that has to follow it.
+    cannot take rotation and cache write into itself is charged the kernel that has to follow it, as is
+    the library for "sum" at up to 16 rows, where the streaming kernel saves the norm's kernel.
 
     Timing is made like a decode step: the launches are recorded into a HIP graph and replayed (a
     product that needs two kernels is then charged what a second graph node costs, not what a
@@ -539,7 +545,9 @@ def tune_linear(weights, out_dtype: torch.dtype = torch.bfloat16, use: str = "pl
         return best
 
     def cost(bucket, choice, fn) -> float:
-        tail = TAIL_KERNEL_US * 1e-3 * iters if use == "qkv" and not fuses_tail(choice, use) else 0.0
+        # (for "sum" only where the streaming kernel is a candidate: beyond its rows the norm kernel runs whoever multiplies)
+        charged = use == "qkv" or (use == "sum" and bucket <= STREAM_MAX_ROWS and n % 4 == 0)
+        tail = TAIL_KERNEL_US * 1e-3 * iters if charged and not fuses_tail(choice, use) else 0.0
         t = clock(fn) + tail
         if report is not None:
             report(bucket, choice, t / iters * 1e3)
