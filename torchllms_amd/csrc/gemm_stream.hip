@@ -72,6 +72,11 @@ struct NormArgs {
 };
 
 constexpr int kSumRows = 16;   // rows side by side in a piece of the sums of squares
+// Pieces of a row's sum of squares that a lane asks for before the walk along K (any others it fetches at the
+// end, and waits for each): with sixteen rows (MR = 4) the registers allow fewer blocks a CU anyway.
+constexpr int held_sums(int mr) { return mr == 4 ? 16 : 8; }
+// Pieces that a block of `waves` waves takes in without that wait: its lanes share out the pieces of 4 MR rows.
+constexpr int sums_taken_ahead(int mr, int waves) { return held_sums(mr) * (kWave / (4 * mr)) * waves; }
 
 // MR: groups of four rows of A that are fetched (M <= 4 * MR).  WAVES: waves per block = splits of K.
 // EPI kGated, kGatedHalf: W holds 2 N rows, gate rows then up rows; C[M, N] = silu(A gate^T) * (A up^T);
@@ -137,9 +142,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   // under no branch, so that nothing of theirs is waited for before the walk: without sums they
   // read the start of A, which nobody uses.
   constexpr bool NORMED = EPI == kGated || EPI == kGatedHalf || EPI == kQkv;
-  // pieces that a lane asks for ahead (any others it fetches at the end, and waits): with sixteen rows the
-  // registers allow fewer blocks a CU anyway, and sixteen pieces cover 256 with four waves
-  constexpr int kHeldSums = MR == 4 ? 16 : 8;
+  constexpr int kHeldSums = held_sums(MR);
   constexpr int kSumSide = 4 * MR;                       // rows side by side in the lanes of a wave
   constexpr int kSumLanes = (kWave / kSumSide) * WAVES;  // lanes of the block that share a row's pieces
   const int sum_first = lane / kSumSide + (kWave / kSumSide) * wave;
@@ -446,6 +449,12 @@ int run(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M,
     while (waves < 8 && strips * waves < enough && steps >= 2 * waves * 2) waves *= 2;
   }
   TL_REQUIRE(waves == 1 || waves == 2 || waves == 4 || waves == 8, "gemm_stream: waves must be 1, 2, 4 or 8");
+  if (na.row_sums != nullptr) {
+    // as many waves as take in all pieces of the sums of squares ahead (rows of 8,192 elements come in 512
+    // pieces): a wave that fetches its share at the end waits a trip to memory for every few of them
+    const int mr = M <= 4 ? 1 : M <= 8 ? 2 : 4;
+    while (waves < 8 && sums_taken_ahead(mr, waves) < na.n_row_sums && K / kStepK >= 2 * waves) waves *= 2;
+  }
   const bf16_t* a = (const bf16_t*)A;
   const bf16_t* w = (const bf16_t*)W;
   if (M <= 4) return launch_waves<1>(waves, a, lda, w, ldw, C, ldc, M, N, K, out_dtype, epi, qa, na, stream);

@@ -51,6 +51,7 @@ from .products import (  # noqa: F401
     gemm_stream_glu,
     gemm_stream_qkv,
     gemm_stream_residual,
+    NORMED_ROWS_MAX_WIDTH,
     NormedRows,
     PendingProduct,
     gemm_wide,

@@ -67,6 +67,11 @@ def gemm_stream(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     return out
 
 
+#: the widest rows whose norm the streaming products take over: their sums of squares come in width / 16 pieces, and
+#: 512 are what a block of eight waves asks for ahead of its walk (more would be fetched at its end, with a wait)
+NORMED_ROWS_MAX_WIDTH = 8192
+
+
 class NormedRows(Unfinished):
     """``rmsnorm(rows, weight, eps)`` of at most 16 bfloat16 rows, not yet computed: ``gained`` are the
     rows times ``weight`` and ``sums`` float32 [pieces, 16] are pieces of each row's sum of squares

@@ -42,7 +42,8 @@ class RMSNorm(Norm):
         return ops.rmsnorm(h, self.weight, self.eps, delta=delta, return_sum=True)
 
     def forward_add_for(self, reader, h: torch.Tensor, delta):
-        if isinstance(delta, ops.PendingProduct) and getattr(reader, "takes_normed_rows", False) and self.weight.dtype == torch.bfloat16:
+        if (isinstance(delta, ops.PendingProduct) and getattr(reader, "takes_normed_rows", False)
+                and self.weight.dtype == torch.bfloat16 and self.size <= ops.NORMED_ROWS_MAX_WIDTH):
             # the product's own kernel adds it to h and leaves the rows' statistics, which the reader's kernel applies
             return delta.added_to(h, self.weight, self.eps)
         return self.forward_add(h, delta)
