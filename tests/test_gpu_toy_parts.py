@@ -306,3 +306,62 @@ def test_toy_parts_in_bfloat16_stay_near_the_plain_model():
     worst = max((row - truth[rid][pos]).abs().max().item() for (rid, pos), row in got.items())
     scale = max(t.abs().max().item() for t in truth.values())
     assert worst < 0.06 * scale, (worst, scale)
+
+
+def test_a_toy_feed_forward_may_take_normed_rows_and_make_a_tensor_of_them():
+    """A part that says ``takes_normed_rows`` is handed the norm's rows with their statistics not yet
+    applied on bfloat16 steps of few rows; ``ops.resolved`` makes the normed tensor of them, the very
+    bits that the same part gets when it does not say so (the product before the norm adds itself to
+    the residual rows with the roundings of the norm kernel, which then runs on its result)."""
+    from torchllms_amd.config.spec import PartSpec
+    from torchllms_amd.kernels import ops
+    from torchllms_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, FeedForward, ParamSpec
+    from tests.test_gpu_parts import _ctx_and_cache, _step
+
+    seen = []
+
+    class Doubling(FeedForward):
+        graph_safe = True
+
+        def __init__(self, hidden_size):
+            self.hidden_size = hidden_size
+
+        def param_specs(self):
+            return {"w.weight": ParamSpec((self.hidden_size, self.hidden_size))}
+
+        def bind(self, tensors):
+            self.w = tensors["w.weight"]
+
+        def forward(self, x, ctx):
+            seen.append(type(x).__name__)
+            return ops.linear(ops.resolved(x), self.w) * 2
+
+    class DoublingThatTakesThem(Doubling):
+        takes_normed_rows = True
+
+    FEED_FORWARDS["toy_doubling"], FEED_FORWARDS["toy_doubling_takes"] = Doubling, DoublingThatTakesThem
+    try:
+        torch.manual_seed(3)
+        D, S = 64, 6
+        outs = []
+        for kind in ("toy_doubling", "toy_doubling_takes"):
+            block = BLOCKS["pre_norm"]({
+                "mixer": MIXERS.build(PartSpec("attention", dict(hidden_size=D, num_heads=4, num_kv_heads=2, head_dim=16, qkv_bias=False,
+                                                                 softmax_scale=0.25, window=0,
+                                                                 position=PartSpec("rope", dict(head_dim=16, rotary_dim=16, theta=1e4, scaling=None))))),
+                "ffn": FEED_FORWARDS.build(PartSpec(kind, dict(hidden_size=D))),
+                "mixer_norm": NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=1e-5))),
+                "ffn_norm": NORMS.build(PartSpec("rmsnorm", dict(size=D, eps=1e-5))),
+            })
+            gen = torch.Generator().manual_seed(5)
+            w = {n: ((torch.randn(s.shape, generator=gen) * 0.2) if s.init == "normal" else (0.5 + torch.rand(s.shape, generator=gen))).bfloat16()
+                 for n, s in block.param_specs().items()}
+            block.bind({k: v.to("cuda:0") for k, v in w.items()})
+            x = (torch.randn(S, D, generator=torch.Generator().manual_seed(6)) * 2).bfloat16().to("cuda:0")
+            cache = _ctx_and_cache(S, 2, 16, 4, torch.bfloat16)
+            h, delta = block.forward(x, None, _step(cache, "r", S), {"mixer": cache.kv_view(0)})
+            outs.append((h, ops.resolved(delta)))
+        assert seen == ["Tensor", "NormedRows"]
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    finally:
+        del FEED_FORWARDS["toy_doubling"], FEED_FORWARDS["toy_doubling_takes"]
