@@ -316,7 +316,7 @@ def test_a_toy_feed_forward_may_take_normed_rows_and_make_a_tensor_of_them():
     from torchllms_amd.config.spec import PartSpec
     from torchllms_amd.kernels import ops
     from torchllms_amd.parts import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, FeedForward, ParamSpec
-    from tests.test_gpu_parts import _ctx_and_cache, _step
+    from .test_gpu_parts import _ctx_and_cache, _step
 
     seen = []
 
