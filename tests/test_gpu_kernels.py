@@ -1331,10 +1331,12 @@ def _prefill(rows, hq, hkv, dh, page, window=0, seed=0, key_groups=1):
         (32, 8, 128, 16, [(77, 77), (500, 2), (130, 64), (33, 33)]),
         (8, 1, 32, 16, [(200, 200), (65, 3)]),
         (4, 4, 64, 8, [(150, 150)]),
-        (6, 2, 64, 4, [(90, 31), (40, 40)]),
+        (6, 2, 64, 8, [(90, 31), (40, 40)]),
         (16, 1, 128, 32, [(129, 129)]),
         (4, 1, 256, 16, [(100, 100), (70, 5)]),
-        (5, 5, 32, 2, [(61, 61)]),
+        (5, 5, 32, 16, [(61, 61)]),
+        (3, 1, 256, 2, [(61, 61), (30, 7)]),
+        (8, 2, 128, 4, [(150, 150), (99, 6)]),
         (5, 5, 32, 128, [(261, 261), (140, 3)]),
         (2, 2, 64, 16, [(1, 1), (2, 2), (17, 16)]),
     ],
@@ -1349,11 +1351,16 @@ def test_attention_prefill(hq, hkv, dh, page, rows, key_groups):
 
 def test_attention_prefill_takes_pages_of_a_power_of_two_only():
     """Pages of 12 tokens are refused by the MFMA kernel with a clear error (and sent to the plain
-    kernel by the dispatcher: tests/test_gpu_random_configs.py runs such page sizes end to end)."""
+    kernel by the dispatcher: tests/test_gpu_random_configs.py runs such page sizes end to end); so
+    are pages shorter than the rows that a wave fetches with one instruction (512 / head size)."""
     ops = _ops()
     assert ops.prefill_attention_supported(torch.bfloat16, 4, 2, 64, 16) and not ops.prefill_attention_supported(torch.bfloat16, 4, 2, 64, 12)
     with pytest.raises(ops.KernelError, match="page_size 12 is no power of two"):
         _prefill([(61, 61)], 5, 5, 32, 12)
+    assert ops.prefill_attention_supported(torch.bfloat16, 4, 2, 64, 8) and not ops.prefill_attention_supported(torch.bfloat16, 4, 2, 64, 4)
+    assert ops.prefill_attention_supported(torch.bfloat16, 4, 2, 256, 2) and not ops.prefill_attention_supported(torch.bfloat16, 4, 2, 32, 8)
+    with pytest.raises(ops.KernelError, match="pages of 4 tokens are shorter than the 8 rows"):
+        _prefill([(61, 61)], 6, 2, 64, 4)
 
 
 @pytest.mark.parametrize("key_groups", [1, 2])

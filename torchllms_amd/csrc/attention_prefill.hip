@@ -162,17 +162,17 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
   const int kvh = blockIdx.x;
   const int grp = GROUPS == 1 ? 0 : wave_uniform(threadIdx.x / (kWaves * kWave));
   bf16_t* const tiles = tile_memory<GROUPS>() + grp * 4 * kTileElems;  // this group's [buffer][keys | values]
-  const int wave = (threadIdx.x / kWave) % kWaves;  // within the group
+  const int wave = wave_uniform((threadIdx.x / kWave) % kWaves);  // within the group
   const int lane = threadIdx.x % kWave;
   const int n16 = lane % 16;
   const int g4 = lane / 16;
   const int R = a.group;
 
-  const int row = a.tile_row[tile];
-  const int q0 = a.tile_q0[tile];
-  const int tok0 = a.qo_indptr[row];
-  const int q_len = a.qo_indptr[row + 1] - tok0;
-  const int kv_len = a.kv_lens[row];
+  const int row = wave_uniform(a.tile_row[tile]);
+  const int q0 = wave_uniform(a.tile_q0[tile]);
+  const int tok0 = wave_uniform(a.qo_indptr[row]);
+  const int q_len = wave_uniform(a.qo_indptr[row + 1]) - tok0;
+  const int kv_len = wave_uniform(a.kv_lens[row]);
   const int pos0 = kv_len - q_len;  // position of the row's first new token
   const int32_t* bt = a.block_table + (size_t)row * a.bt_stride;
   const size_t head_elems = (size_t)a.page_size * DH;
@@ -228,16 +228,22 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
   const unsigned page_bytes = (unsigned)a.n_kv_heads * (unsigned)a.page_size * DH * 2;  // all kv heads of a page
   const char* const k_head = reinterpret_cast<const char*>(a.k_pages) + (size_t)kvh * head_elems * 2;  // this kv head's rows in page 0
   const char* const v_head = reinterpret_cast<const char*>(a.v_pages) + (size_t)kvh * head_elems * 2;
-  const int my_row = lane / kPieces + wave * kRowsPerLoad;  // this lane's row within a wave load's turn
+  // The rows of one wave load (64 lanes x 16 bytes: kRowsPerLoad rows) lie in one page (the host sees to
+  // it that a page holds at least as many rows, and tiles start at multiples of the tile's size), so a
+  // load's page is one number for the wave: it is looked up by a scalar load and the page's address is
+  // scalar arithmetic; a lane adds what does not change from tile to tile (its row within the load and
+  // its piece's slot).
+  typedef const int32_t __attribute__((address_space(4))) * table_ptr_t;  // read-only for the kernel's life
+  const table_ptr_t table = (table_ptr_t)(uintptr_t)bt;
   struct Rows {
     int page[kLoadsPerWave];
   };
   auto lookup = [&](int base, Rows& rows) {
 #pragma unroll
     for (int j = 0; j < kLoadsPerWave; ++j) {
-      int blk = (base + j * kWaves * kRowsPerLoad + my_row) >> a.page_shift;
+      int blk = (base + (j * kWaves + wave) * kRowsPerLoad) >> a.page_shift;
       blk = blk < blk_lo ? blk_lo : (blk > blk_hi ? blk_hi : blk);
-      rows.page[j] = bt[blk];
+      rows.page[j] = table[blk];
     }
   };
   auto dma = [&](int base, const Rows& rows, int buffer, bool values) {
@@ -246,9 +252,10 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
       const int first = (j * kWaves + wave) * kRowsPerLoad;
       const int r = first + lane / kPieces;
       const int piece = (lane % kPieces) ^ (values ? swizzle_v(r) : swizzle(r));
-      const unsigned in_page = (unsigned)((base + r) & (a.page_size - 1)) * (DH * 2) + 16 * piece;
+      const unsigned of_lane = (unsigned)(lane / kPieces) * (DH * 2) + 16 * piece;  // the same for every tile
+      const unsigned in_page = (unsigned)((base + first) & (a.page_size - 1)) * (DH * 2);
       const char* src = (values ? v_head : k_head) + ((size_t)(unsigned)rows.page[j] * page_bytes + in_page);
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const bf16_t*>(src),
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const bf16_t*>(src + of_lane),
                                        &tiles[(2 * buffer + (values ? 1 : 0)) * kTileElems + first * DH], 16, 0, 0);
     }
   };
@@ -541,6 +548,10 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   while ((1 << a.page_shift) < page_size) ++a.page_shift;
   if ((1 << a.page_shift) != page_size)
     return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: page_size %d is no power of two", page_size);
+  // (a wave fetches kRowsPerLoad rows with one instruction and looks up one page for them)
+  if (page_size < kRowsPerLoad)
+    return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: pages of %d tokens are shorter than the %d rows a wave fetches at once at head size %d",
+                        page_size, kRowsPerLoad, DH);
   a.scale_log2e = scale * 1.4426950408889634f;
   dim3 grid(n_kv_heads, n_tiles);  // consecutive blocks share a query tile: their loads of q overlap
   const bool windowed = window > 0;

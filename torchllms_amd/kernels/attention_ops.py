@@ -249,9 +249,12 @@ PREFILL_HEAD_DIMS = (32, 64, 128, 256)
 
 def prefill_attention_supported(dtype: torch.dtype, n_q_heads: int, n_kv_heads: int, head_dim: int, page_size: int = 16) -> bool:
     """Whether the MFMA prefill kernel takes these sizes (else the plain kernel runs): bfloat16, head
-    size 32, 64, 128 or 256, at most 16 query heads per kv head, pages of a power of two of tokens."""
+    size 32, 64, 128 or 256, at most 16 query heads per kv head, pages of a power of two of tokens that
+    hold at least the rows a wave fetches with one instruction (1 KB: 512 / head size rows, which then
+    share one entry of the block table)."""
     return (dtype == torch.bfloat16 and head_dim in PREFILL_HEAD_DIMS and n_q_heads % n_kv_heads == 0
-            and n_q_heads // n_kv_heads <= 16 and page_size > 0 and page_size & (page_size - 1) == 0)
+            and n_q_heads // n_kv_heads <= 16 and page_size > 0 and page_size & (page_size - 1) == 0
+            and page_size * head_dim >= 512)
 
 
 def prefill_queries_per_tile(n_q_heads: int, n_kv_heads: int, head_dim: int) -> int:
